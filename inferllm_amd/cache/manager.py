@@ -1,0 +1,234 @@
+"""The cache of a model: slots, paged key/value storage per group of layers, and
+fixed-size state per sequence.
+
+Layout.  A *cache line* is the storage one run of a layer uses (the schedule
+names it).  Lines with the same needs form a *group* with storage of its own:
+
+* kind "full": every key and value of a sequence is kept;
+* kind "window": only the last `window` keys are ever read, so a sequence keeps a
+  ring of pages and its storage stops growing.
+
+A group holds K and V as [line][page][kv head][row in page][head_dim]; a page has
+`page_size` (64) rows, so one kv head's part of a page is contiguous.  Each group
+has its own page pool and its own page table [slot][logical page] -> page.  The
+last slot and the last page of every group are spare: rows that only pad a batch
+point there.  Sequence lengths live in `slot_len`, one int per slot, on the host
+and on the device.
+
+Beside the groups, `StateSpec`s describe tensors of fixed size per sequence
+([slot, *shape]), zeroed when a slot is handed out.
+
+The reference keeps, per attention op, two tensors [n_ctx, embd] and a cursor
+(src/core/kvstorage.h:9-54), grown lazily in steps of 100 rows
+(src/core/kvstotage.cpp:53-76), for its single sequence.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .slots import CacheError, CacheFull, FreeList
+
+PAGE_SIZE = 64
+
+
+def round_up(n: int, m: int) -> int:
+    return (n + m - 1) // m * m
+
+
+@dataclass(frozen=True)
+class KVSpec:
+    """What one cache line needs: kept keys ("full" or "window"), kv heads, head size."""
+    kind: str
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+    def __post_init__(self):
+        if self.kind not in ("full", "window"):
+            raise CacheError(f"unknown cache kind {self.kind!r}")
+        if self.kind == "window" and not (self.window and self.window > 0):
+            raise CacheError("a window cache needs a positive window")
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state per sequence for one cache line: shape and dtype."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class KVGroup:
+    """Storage, page pool and page table of the lines that share one `KVSpec`."""
+
+    def __init__(self, spec: KVSpec, lines: Sequence[int], n_slots: int, max_tokens: int,
+                 max_seq_len: int, dtype: torch.dtype, device, page_size: int = PAGE_SIZE):
+        self.spec = spec
+        self.lines = list(lines)
+        self.page_size = page_size
+        pages_full = max(1, max_tokens // page_size)
+        seq_pages = max(1, round_up(max_seq_len, page_size) // page_size)
+        if spec.kind == "window":
+            # pages that the last `window` keys of any position can touch
+            self.ring = (spec.window + page_size - 2) // page_size + 1
+            if self.ring >= seq_pages:
+                self.ring = 0           # the window never wraps: same as "full"
+        else:
+            self.ring = 0
+        self.pages_per_seq = self.ring if self.ring else seq_pages
+        self.n_pages = min(pages_full, n_slots * self.pages_per_seq)
+        self.pool = FreeList(self.n_pages, "page")
+        self.spare_page = self.n_pages
+        shape = (len(self.lines), self.n_pages + 1, spec.num_kv_heads, page_size, spec.head_dim)
+        self.k = torch.zeros(shape, dtype=dtype, device=device)
+        self.v = torch.zeros(shape, dtype=dtype, device=device)
+        self.table_host = torch.full((n_slots + 1, self.pages_per_seq), self.spare_page,
+                                     dtype=torch.int32)
+        self.table = self.table_host.to(device)
+        self.held: Dict[int, List[int]] = {}     # slot -> pages in logical order
+        self._dirty = set()
+
+    def line_index(self, line: int) -> int:
+        return self.lines.index(line)
+
+    def pages_needed(self, length: int) -> int:
+        n = (length + self.page_size - 1) // self.page_size
+        return min(n, self.ring) if self.ring else n
+
+    def reserve(self, slot: int, length: int) -> None:
+        pages = self.held.setdefault(slot, [])
+        need = self.pages_needed(length)
+        if need > self.pages_per_seq:
+            raise CacheFull(f"a sequence of {length} tokens needs {need} pages; "
+                            f"{self.pages_per_seq} is the most one sequence may hold")
+        if need - len(pages) > self.pool.n_free():
+            raise CacheFull(f"cache full: {need - len(pages)} more pages of {self.page_size} tokens "
+                            f"needed, {self.pool.n_free()} of {self.n_pages} free")
+        while len(pages) < need:
+            p = self.pool.alloc()
+            self.table_host[slot, len(pages)] = p
+            pages.append(p)
+            self._dirty.add(slot)
+
+    def release(self, slot: int, poison: bool = False) -> None:
+        pages = self.held.pop(slot, [])
+        if poison and pages and self.k.dtype.is_floating_point:
+            idx = torch.tensor(pages, dtype=torch.long, device=self.k.device)
+            self.k[:, idx] = float("nan")
+            self.v[:, idx] = float("nan")
+        for p in pages:
+            self.pool.free(p)
+        self.table_host[slot].fill_(self.spare_page)
+        self._dirty.add(slot)
+
+    def upload(self) -> None:
+        for slot in sorted(self._dirty):
+            self.table[slot].copy_(self.table_host[slot])
+        self._dirty.clear()
+
+
+class CacheManager:
+    """Slots, KV groups and per-sequence state for one model on one device.
+
+    `max_tokens` is the most tokens that live sequences hold together, each
+    sequence rounded up to whole pages; `max_slots` the most live sequences;
+    `max_seq_len` the longest one sequence may become.
+    """
+
+    def __init__(self, kv_lines: Dict[int, KVSpec], state_lines: Dict[int, StateSpec],
+                 max_tokens: int, max_slots: int, max_seq_len: int, dtype: torch.dtype, device,
+                 page_size: int = PAGE_SIZE, poison_freed: bool = False):
+        if max_slots <= 0 or max_tokens <= 0 or max_seq_len <= 0:
+            raise CacheError("max_slots, max_tokens and max_seq_len must be positive")
+        self.page_size = page_size
+        self.max_tokens = round_up(max_tokens, page_size)
+        self.max_slots = max_slots
+        self.max_seq_len = max_seq_len
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.poison_freed = poison_freed
+        self.slots = FreeList(max_slots, "slot")
+        self.spare_slot = max_slots
+        by_spec: Dict[KVSpec, List[int]] = {}
+        for line in sorted(kv_lines):
+            by_spec.setdefault(kv_lines[line], []).append(line)
+        self.groups: List[KVGroup] = [
+            KVGroup(spec, lines, max_slots, self.max_tokens, max_seq_len, dtype, device, page_size)
+            for spec, lines in by_spec.items()]
+        self._group_of: Dict[int, KVGroup] = {l: g for g in self.groups for l in g.lines}
+        self.states: Dict[int, torch.Tensor] = {
+            line: torch.zeros((max_slots + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
+            for line, s in state_lines.items()}
+        self.len_host = torch.zeros(max_slots + 1, dtype=torch.int32)
+        self.slot_len = self.len_host.to(device)
+        self._len_dirty = False
+
+    # ------------------------------------------------------------ slots
+    def alloc_slot(self) -> int:
+        slot = self.slots.alloc()
+        self.len_host[slot] = 0
+        self._len_dirty = True
+        for t in self.states.values():
+            t[slot].zero_()
+        return slot
+
+    def free_slot(self, slot: int) -> None:
+        self.slots.free(slot)           # raises if not held
+        for g in self.groups:
+            g.release(slot, self.poison_freed)
+        self.len_host[slot] = 0
+        self._len_dirty = True
+
+    def length(self, slot: int) -> int:
+        return int(self.len_host[slot])
+
+    # ------------------------------------------------------------ steps
+    def extend(self, slot: int, start_pos: int, n_tokens: int) -> None:
+        """Make room for `n_tokens` more tokens of `slot`, which must now hold `start_pos`."""
+        if slot not in self.slots._held:
+            raise CacheError(f"slot {slot} is not held")
+        have = int(self.len_host[slot])
+        if start_pos != have:
+            raise CacheError(f"slot {slot} holds {have} tokens; a step starting at {start_pos} "
+                             "does not follow")
+        new_len = have + n_tokens
+        if new_len > self.max_seq_len:
+            raise CacheFull(f"sequence would reach {new_len} tokens; the limit is {self.max_seq_len}")
+        for g in self.groups:
+            g.reserve(slot, new_len)
+        self.len_host[slot] = new_len
+        self._len_dirty = True
+
+    def upload(self) -> None:
+        """Bring page tables and lengths on the device up to date with the host."""
+        for g in self.groups:
+            g.upload()
+        if self._len_dirty:
+            self.slot_len.copy_(self.len_host)
+            self._len_dirty = False
+
+    # ------------------------------------------------------------ views for parts
+    def kv_line(self, line: int):
+        """(K, V, group) of a cache line; K and V are [page, kv head, row, head_dim]."""
+        g = self._group_of[line]
+        i = g.line_index(line)
+        return g.k[i], g.v[i], g
+
+    def state_line(self, line: int) -> Optional[torch.Tensor]:
+        return self.states.get(line)
+
+    def tokens_held(self) -> int:
+        """Tokens held now, each sequence rounded up to whole pages."""
+        return sum(round_up(int(self.len_host[s]), self.page_size) for s in self.slots.held())
+
+    def check(self) -> None:
+        self.slots.check()
+        for g in self.groups:
+            g.pool.check()
+            held = [p for pages in g.held.values() for p in pages]
+            if sorted(held) != g.pool.held():
+                raise CacheError("pages held by slots differ from pages taken from the pool")
+            if set(g.held) - set(self.slots.held()):
+                raise CacheError("a freed slot still holds pages")

@@ -1,0 +1,67 @@
+// C entry points of the kernel library.  Every function launches on `stream`
+// and returns ILLM_OK, ILLM_ERR_ARG (sizes or dtypes it does not take; nothing
+// was launched) or ILLM_ERR_LAUNCH.  Pointers are device pointers.  dtype codes:
+// 0 = float32, 1 = bfloat16.
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+int illm_version();
+
+// out[t, :] = table[tokens[t], :] as float32.
+int illm_embed(const int32_t* tokens, const void* table, int table_dt, float* out,
+               int T, int E, int V, void* stream);
+
+// Residual add and RMS norm.  in_row = row_idx ? row_idx[r] : r;
+// v = x[in_row] (+ delta[in_row]); when delta is given and row_idx is not, v is
+// written back to x.  out[r] = v * rsqrt(mean(v^2) + eps) * w.
+int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const void* w, int w_dt,
+                     void* out, int out_dt, const int32_t* row_idx, int rows, int E, float eps,
+                     void* stream);
+
+// out[t, f] = silu(gate_up[t, f]) * gate_up[t, F + f].
+int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* stream);
+
+// Rotate q and k of packed rows [q (nh*hd) | k (nkv*hd) | v (nkv*hd)] in place by the
+// angles of `cos_sin` ([max_pos][rot/2][2] float32; null: no rotation) at row_pos[t],
+// pairing 0 = (i, i + rot/2), 1 = (2i, 2i+1); then store k and v of each row in the
+// paged cache of row_slot[t] (skipped when kcache is null).
+int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_pos, int rot, int pairing,
+                    const int32_t* row_pos, const int32_t* row_slot, const int32_t* slot_len,
+                    void* kcache, void* vcache, const int32_t* page_table, int table_stride,
+                    int page_size, int ring, int T, int nh, int nkv, int hd, void* stream);
+
+// Y[M, N] = X[M, K] . W[N, K]^T, float32 accumulation in a fixed order; any sizes.
+int illm_gemm_generic(const void* X, int x_dt, const void* W, int w_dt, void* Y, int y_dt,
+                      int M, int N, int K, void* stream);
+
+// Causal attention over packed rows of whole prompts (keys and values of the step
+// itself).  cu_seqlens[n_seqs + 1]; window <= 0: all earlier keys.
+int illm_attn_prefill_generic(const void* qkv, void* out, int dt, const int32_t* cu_seqlens,
+                              int n_seqs, int max_len, int nh, int nkv, int hd, float scale,
+                              int window, void* stream);
+
+// One query row per sequence over the paged cache.  partial: float32
+// [B][nh][nsplit][hd + 2] scratch.  slot_len[slot] = keys of the sequence, the new one included.
+int illm_attn_decode_generic(const void* qkv, void* out, int dt, const void* kcache,
+                             const void* vcache, const int32_t* page_table, int table_stride,
+                             int page_size, int ring, const int32_t* seq_slot,
+                             const int32_t* slot_len, float* partial, int nsplit, int B, int nh,
+                             int nkv, int hd, float scale, int window, void* stream);
+
+// out[b] = index of the largest logit of row b (lowest index on ties).
+int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream);
+
+// Temperature / top-k / top-p / repeat-penalty sampling, one draw per row.
+// scratch: float32 [B][V].  last_tokens: [B][n_last] (-1 = empty) or null.
+// counters[b]: index of the draw in the request's stream; seeds[b]: the request's seed.
+int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V, float temp,
+                int top_k, float top_p, float repeat_penalty, const int32_t* last_tokens,
+                int n_last, const uint64_t* seeds, const int32_t* counters, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

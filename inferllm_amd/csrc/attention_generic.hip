@@ -1,0 +1,251 @@
+// Causal attention in float32 arithmetic for any head size up to 256, any number
+// of heads and groups, float32 or bfloat16 storage: one kernel for whole prompts
+// (keys and values of the step itself) and one for a single new token per sequence
+// over the paged cache.  These are the kernels of the 32-bit path and the
+// fallback for sizes the MFMA kernels do not take.
+//
+// What they compute is the reference's chain scores -> scale and mask -> softmax
+// -> context (src/core/op.cpp:485-498; src/kern/naive/naive.cpp:606-632, :531-553,
+// :209-240, :664-691), with query head h reading kv head h / (heads / kv_heads)
+// (naive.cpp:576-604).  The reference materialises the scores [heads, S, P+S]
+// (op.cpp:323-326); here they live tile by tile with a running max and sum.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+#define AQ 32  // query rows of a block
+#define AK 32  // keys of a tile
+#define NEG_INF (-INFINITY)
+
+// grid (query tiles, heads, sequences); 256 threads: 8 per query row.
+__global__ void __launch_bounds__(256)
+attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out, int dt,
+                            const int32_t* __restrict__ cu, int nh, int nkv, int hd, float scale,
+                            int window) {
+    extern __shared__ float smem[];
+    const int hp = hd + 1;
+    float* qs = smem;            // [AQ][hp]
+    float* ks = qs + AQ * hp;    // [AK][hp]
+    float* vs = ks + AK * hp;    // [AK][hp]
+    float* ps = vs + AK * hp;    // [AQ][AK + 1]
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int start = cu[b], len = cu[b + 1] - start;
+    const int q0 = blockIdx.x * AQ;
+    if (q0 >= len) return;
+    const int kvh = h / (nh / nkv);
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * hd;
+    const int tid = threadIdx.x, i = tid >> 3, g = tid & 7;
+
+    for (int e = tid; e < AQ * hd; e += 256) {
+        const int r = e / hd, d = e - r * hd;
+        qs[r * hp + d] = (q0 + r < len)
+                             ? ld_f(qkv, dt, (size_t)(start + q0 + r) * rowlen + (size_t)h * hd + d)
+                             : 0.f;
+    }
+    float m_i = NEG_INF, l_i = 0.f;
+    float acc[32];
+#pragma unroll
+    for (int k = 0; k < 32; ++k) acc[k] = 0.f;
+    const int qpos = q0 + i;
+    const int k_hi = min(len, q0 + AQ);
+    int k_lo = window > 0 ? max(0, q0 - window + 1) : 0;
+    k_lo = (k_lo / AK) * AK;
+
+    for (int k0 = k_lo; k0 < k_hi; k0 += AK) {
+        __syncthreads();
+        for (int e = tid; e < AK * hd; e += 256) {
+            const int r = e / hd, d = e - r * hd;
+            float kv = 0.f, vv = 0.f;
+            if (k0 + r < len) {
+                const size_t base = (size_t)(start + k0 + r) * rowlen;
+                kv = ld_f(qkv, dt, base + (size_t)(nh + kvh) * hd + d);
+                vv = ld_f(qkv, dt, base + (size_t)(nh + nkv + kvh) * hd + d);
+            }
+            ks[r * hp + d] = kv;
+            vs[r * hp + d] = vv;
+        }
+        __syncthreads();
+        float s[4];
+        float tm = NEG_INF;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int j = g + 8 * c, kj = k0 + j;
+            float a = 0.f;
+            for (int d = 0; d < hd; ++d) a = fmaf(qs[i * hp + d], ks[j * hp + d], a);
+            const bool ok = qpos < len && kj <= qpos && (window <= 0 || kj > qpos - window);
+            s[c] = ok ? a * scale : NEG_INF;
+            tm = fmaxf(tm, s[c]);
+        }
+        tm = fmaxf(tm, __shfl_xor(tm, 1, ILLM_WAVE));
+        tm = fmaxf(tm, __shfl_xor(tm, 2, ILLM_WAVE));
+        tm = fmaxf(tm, __shfl_xor(tm, 4, ILLM_WAVE));
+        const float m_new = fmaxf(m_i, tm);
+        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m_i - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const float p = (s[c] == NEG_INF) ? 0.f : expf(s[c] - m_new);
+            ps[i * (AK + 1) + g + 8 * c] = p;
+            psum += p;
+        }
+        psum += __shfl_xor(psum, 1, ILLM_WAVE);
+        psum += __shfl_xor(psum, 2, ILLM_WAVE);
+        psum += __shfl_xor(psum, 4, ILLM_WAVE);
+        l_i = l_i * alpha + psum;
+        m_i = m_new;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            const int d = g + 8 * k;
+            if (d < hd) {
+                float a = acc[k] * alpha;
+                for (int j = 0; j < AK; ++j) a = fmaf(ps[i * (AK + 1) + j], vs[j * hp + d], a);
+                acc[k] = a;
+            }
+        }
+    }
+    if (qpos < len) {
+        const float inv = 1.0f / l_i;
+        const size_t ob = (size_t)(start + qpos) * nh * hd + (size_t)h * hd;
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            const int d = g + 8 * k;
+            if (d < hd) st_f(out, dt, ob + d, acc[k] * inv);
+        }
+    }
+}
+
+extern "C" int illm_attn_prefill_generic(const void* qkv, void* out, int dt,
+                                         const int32_t* cu_seqlens, int n_seqs, int max_len,
+                                         int nh, int nkv, int hd, float scale, int window,
+                                         void* stream) {
+    if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
+        !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535)
+        return ILLM_ERR_ARG;
+    if (n_seqs == 0 || max_len == 0) return ILLM_OK;
+    const size_t smem = ((size_t)(AQ + 2 * AK) * (hd + 1) + AQ * (AK + 1)) * sizeof(float);
+    if (smem > 48 * 1024) {
+        if (hipFuncSetAttribute((const void*)attn_prefill_generic_kernel,
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)smem) != hipSuccess) {
+            (void)hipGetLastError();
+            return ILLM_ERR_ARG;
+        }
+    }
+    hipLaunchKernelGGL(attn_prefill_generic_kernel, dim3((max_len + AQ - 1) / AQ, nh, n_seqs),
+                       dim3(256), smem, (hipStream_t)stream, qkv, out, dt, cu_seqlens, nh, nkv, hd,
+                       scale, window);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- decode
+// grid (heads, sequences, splits); 256 threads; tiles of 256 keys aligned at absolute
+// positions, so a key's place in the sums does not depend on the number of splits
+// beyond the split boundaries.  Each block leaves (acc[hd], max, sum) in `partial`.
+__global__ void __launch_bounds__(256)
+attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __restrict__ kcache,
+                           const void* __restrict__ vcache,
+                           const int32_t* __restrict__ page_table, int table_stride,
+                           int page_size, int ring, const int32_t* __restrict__ seq_slot,
+                           const int32_t* __restrict__ slot_len, float* __restrict__ partial,
+                           int nsplit, int nh, int nkv, int hd, float scale, int window) {
+    __shared__ float qs[256];
+    __shared__ float ps[256];
+    __shared__ float red[16];
+    const int h = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
+    const int tid = threadIdx.x;
+    const int slot = seq_slot[b];
+    const int len = slot_len[slot];
+    const int kvh = h / (nh / nkv);
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * hd;
+    const int k_first = window > 0 ? max(0, len - window) : 0;
+    const int first_tile = k_first / 256;
+    const int n_tiles = (len + 255) / 256 - first_tile;
+    const int per_split = (n_tiles + nsplit - 1) / nsplit;
+    const int t_lo = first_tile + sp * per_split;
+    const int t_hi = min(first_tile + n_tiles, t_lo + per_split);
+
+    if (tid < hd) qs[tid] = ld_f(qkv, dt, (size_t)b * rowlen + (size_t)h * hd + tid);
+    float m = NEG_INF, l = 0.f, acc = 0.f;
+    for (int t = t_lo; t < t_hi; ++t) {
+        __syncthreads();
+        const int kj = t * 256 + tid;
+        float s = NEG_INF;
+        if (kj >= k_first && kj < len) {
+            const size_t off = cache_row_offset(page_table, table_stride, slot, kj, page_size,
+                                                ring, nkv, kvh, hd);
+            float a = 0.f;
+            for (int d = 0; d < hd; ++d) a = fmaf(qs[d], ld_f(kcache, dt, off + d), a);
+            s = a * scale;
+        }
+        const float m_new = fmaxf(m, block_max(s, red));
+        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
+        const float p = (s == NEG_INF) ? 0.f : expf(s - m_new);
+        ps[tid] = p;
+        const float psum = block_sum(p, red);
+        l = l * alpha + psum;
+        m = m_new;
+        __syncthreads();
+        if (tid < hd) {
+            float a = acc * alpha;
+            const int jn = min(256, len - t * 256);
+            for (int j = 0; j < jn; ++j) {
+                const float pj = ps[j];
+                if (pj == 0.f) continue;
+                const size_t off = cache_row_offset(page_table, table_stride, slot, t * 256 + j,
+                                                    page_size, ring, nkv, kvh, hd);
+                a = fmaf(pj, ld_f(vcache, dt, off + tid), a);
+            }
+            acc = a;
+        }
+    }
+    float* pp = partial + (((size_t)b * nh + h) * nsplit + sp) * (size_t)(hd + 2);
+    if (tid < hd) pp[tid] = acc;
+    if (tid == 0) {
+        pp[hd] = m;
+        pp[hd + 1] = l;
+    }
+}
+
+// grid (heads, sequences): combine the splits' partial results.
+__global__ void attn_decode_merge_kernel(const float* __restrict__ partial, void* __restrict__ out,
+                                         int dt, int nsplit, int nh, int hd) {
+    const int h = blockIdx.x, b = blockIdx.y;
+    const float* pp = partial + ((size_t)b * nh + h) * nsplit * (size_t)(hd + 2);
+    float m = NEG_INF;
+    for (int s = 0; s < nsplit; ++s) m = fmaxf(m, pp[(size_t)s * (hd + 2) + hd]);
+    float L = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = pp[(size_t)s * (hd + 2) + hd];
+        if (ms != NEG_INF) L += expf(ms - m) * pp[(size_t)s * (hd + 2) + hd + 1];
+    }
+    const float inv = 1.0f / L;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float ms = pp[(size_t)s * (hd + 2) + hd];
+            if (ms != NEG_INF) a += expf(ms - m) * pp[(size_t)s * (hd + 2) + d];
+        }
+        st_f(out, dt, ((size_t)b * nh + h) * hd + d, a * inv);
+    }
+}
+
+extern "C" int illm_attn_decode_generic(const void* qkv, void* out, int dt, const void* kcache,
+                                        const void* vcache, const int32_t* page_table,
+                                        int table_stride, int page_size, int ring,
+                                        const int32_t* seq_slot, const int32_t* slot_len,
+                                        float* partial, int nsplit, int B, int nh, int nkv, int hd,
+                                        float scale, int window, void* stream) {
+    if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 || !illm_dtype_ok(dt) ||
+        nsplit <= 0 || nsplit > 65535 || B > 65535 || page_size <= 0 || table_stride <= 0)
+        return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    hipLaunchKernelGGL(attn_decode_generic_kernel, dim3(nh, B, nsplit), dim3(256), 0,
+                       (hipStream_t)stream, qkv, dt, kcache, vcache, page_table, table_stride,
+                       page_size, ring, seq_slot, slot_len, partial, nsplit, nh, nkv, hd, scale,
+                       window);
+    hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(nh, B), dim3(64), 0, (hipStream_t)stream,
+                       (const float*)partial, out, dt, nsplit, nh, hd);
+    return illm_launch_status();
+}

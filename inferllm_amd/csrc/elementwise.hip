@@ -1,0 +1,176 @@
+// Row-wise kernels: embedding rows, residual add + RMS norm, SiLU-multiply,
+// rotation of q/k with the store of k/v into the paged cache.
+//
+// Formulas as the reference computes them: embedding row copy
+// (src/kern/naive/naive.cpp:43-54), RMS norm = x * 1/sqrt(mean(x^2) + eps), then
+// the weight (naive.cpp:186-207, src/core/op.cpp:37-47), silu(x) = x / (1 + exp(-x))
+// (naive.cpp:80-89), rotation of pairs (i, i + hd/2) by pos * base^(-2i/rot)
+// (naive.cpp:389-414) or of pairs (2i, 2i+1) (naive.cpp:415-440).  The reference
+// runs each as a kernel of its own (src/kern/gpu/kernel_gpu.cu:127-148, :260-294,
+// :183-258, :343-401); here the residual add is fused with the norm and the cache
+// store with the rotation.
+#include "api.h"
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const void* __restrict__ table,
+                             int table_dt, float* __restrict__ out, int E, int V) {
+    const int t = blockIdx.x;
+    int id = tokens[t];
+    id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+    const size_t src = (size_t)id * E, dst = (size_t)t * E;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) out[dst + i] = ld_f(table, table_dt, src + i);
+}
+
+extern "C" int illm_embed(const int32_t* tokens, const void* table, int table_dt, float* out,
+                          int T, int E, int V, void* stream) {
+    if (T < 0 || E <= 0 || V <= 0 || !illm_dtype_ok(table_dt)) return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(embed_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream, tokens, table,
+                       table_dt, out, E, V);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- add + rmsnorm
+// One block per row.  The sum of squares is taken in float32 in an order that
+// depends on E and the block size only, never on the row's place in the batch.
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ delta,
+                                   int delta_dt, const void* __restrict__ w, int w_dt,
+                                   void* __restrict__ out, int out_dt,
+                                   const int32_t* __restrict__ row_idx, int E, float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const int in_row = row_idx ? row_idx[r] : r;
+    const size_t ib = (size_t)in_row * E, ob = (size_t)r * E;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) {
+        float v = x[ib + i];
+        if (delta) {
+            v += ld_f(delta, delta_dt, ib + i);
+            if (!row_idx) x[ib + i] = v;
+        }
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)E + eps);
+    for (int i = threadIdx.x; i < E; i += blockDim.x) {
+        float v = x[ib + i];
+        if (delta && row_idx) v += ld_f(delta, delta_dt, ib + i);
+        st_f(out, out_dt, ob + i, (v * scale) * ld_f(w, w_dt, i));
+    }
+}
+
+extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const void* w,
+                                int w_dt, void* out, int out_dt, const int32_t* row_idx,
+                                int rows, int E, float eps, void* stream) {
+    if (rows < 0 || E <= 0 || !illm_dtype_ok(w_dt) || !illm_dtype_ok(out_dt) ||
+        (delta && !illm_dtype_ok(delta_dt)))
+        return ILLM_ERR_ARG;
+    if (rows == 0) return ILLM_OK;
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x,
+                       delta, delta_dt, w, w_dt, out, out_dt, row_idx, E, eps);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- silu * up
+__global__ void silu_mul_kernel(const void* __restrict__ gu, void* __restrict__ out, int dt,
+                                int F) {
+    const size_t t = blockIdx.y;
+    const int f = blockIdx.x * blockDim.x + threadIdx.x;
+    if (f >= F) return;
+    const float g = ld_f(gu, dt, t * 2 * F + f);
+    const float u = ld_f(gu, dt, t * 2 * F + F + f);
+    st_f(out, dt, t * F + f, (g / (1.0f + expf(-g))) * u);
+}
+
+extern "C" int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* stream) {
+    if (T < 0 || F <= 0 || !illm_dtype_ok(dt)) return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    // gridDim.y is limited to 65535: rows beyond that go in further launches
+    for (int t0 = 0; t0 < T; t0 += 65535) {
+        const int rows = T - t0 < 65535 ? T - t0 : 65535;
+        const size_t esz = dt == ILLM_BF16 ? 2 : 4;
+        hipLaunchKernelGGL(silu_mul_kernel, dim3((F + 255) / 256, rows), dim3(256), 0,
+                           (hipStream_t)stream,
+                           (const void*)((const char*)gate_up + (size_t)t0 * 2 * F * esz),
+                           (void*)((char*)out + (size_t)t0 * F * esz), dt, F);
+    }
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- rotation + cache store
+// grid (T, nh + nkv): block (t, h) handles head h of row t; heads >= nh are k heads,
+// whose block also stores the matching v head.  The angles come from a float32
+// table that the host fills from double precision.
+__global__ void rope_store_kernel(void* __restrict__ qkv, int dt,
+                                  const float* __restrict__ cos_sin, int rot, int pairing,
+                                  const int32_t* __restrict__ row_pos,
+                                  const int32_t* __restrict__ row_slot,
+                                  const int32_t* __restrict__ slot_len, void* __restrict__ kcache,
+                                  void* __restrict__ vcache,
+                                  const int32_t* __restrict__ page_table, int table_stride,
+                                  int page_size, int ring, int nh, int nkv, int hd) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const int pos = row_pos[t];
+    const size_t row = (size_t)t * (size_t)(nh + 2 * nkv) * hd;
+    const size_t base = row + (size_t)h * hd;  // q heads, then k heads follow directly
+    const int half = rot / 2;
+    if (cos_sin) {
+        const float* cs = cos_sin + (size_t)pos * rot;  // [rot/2][2]
+        for (int i = threadIdx.x; i < half; i += blockDim.x) {
+            const int a = pairing == 0 ? i : 2 * i;
+            const int b = pairing == 0 ? i + hd / 2 : 2 * i + 1;  // partner at hd/2 (naive.cpp:393)
+            const float c = cs[2 * i], s = cs[2 * i + 1];
+            const float x0 = ld_f(qkv, dt, base + a), x1 = ld_f(qkv, dt, base + b);
+            st_f(qkv, dt, base + a, x0 * c - x1 * s);
+            st_f(qkv, dt, base + b, x0 * s + x1 * c);
+        }
+    }
+    if (h < nh || kcache == nullptr) return;
+    const int kvh = h - nh;
+    const int slot = row_slot[t];
+    if (ring > 0) {
+        // a later row of this step lands on the same ring page: this one is already outside
+        const int last_page = (slot_len[slot] - 1) / page_size;
+        if (pos / page_size + ring <= last_page) return;
+    }
+    __syncthreads();  // the rotated k of this block is read back below
+    const size_t dst = cache_row_offset(page_table, table_stride, slot, pos, page_size, ring, nkv,
+                                        kvh, hd);
+    const size_t vsrc = row + (size_t)(nh + nkv + kvh) * hd;
+    const size_t esz = dt == ILLM_BF16 ? 2 : 4;
+    if (esz == 2) {
+        const bf16_t* ks = (const bf16_t*)qkv + base;
+        const bf16_t* vs = (const bf16_t*)qkv + vsrc;
+        bf16_t* kd = (bf16_t*)kcache + dst;
+        bf16_t* vd = (bf16_t*)vcache + dst;
+        for (int i = threadIdx.x; i < hd; i += blockDim.x) { kd[i] = ks[i]; vd[i] = vs[i]; }
+    } else {
+        const float* ks = (const float*)qkv + base;
+        const float* vs = (const float*)qkv + vsrc;
+        float* kd = (float*)kcache + dst;
+        float* vd = (float*)vcache + dst;
+        for (int i = threadIdx.x; i < hd; i += blockDim.x) { kd[i] = ks[i]; vd[i] = vs[i]; }
+    }
+}
+
+extern "C" int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_pos, int rot,
+                               int pairing, const int32_t* row_pos, const int32_t* row_slot,
+                               const int32_t* slot_len, void* kcache, void* vcache,
+                               const int32_t* page_table, int table_stride, int page_size,
+                               int ring, int T, int nh, int nkv, int hd, void* stream) {
+    if (T < 0 || nh <= 0 || nkv < 0 || hd <= 0 || !illm_dtype_ok(dt)) return ILLM_ERR_ARG;
+    if (cos_sin && (rot <= 0 || rot > hd || (rot & 1) || max_pos <= 0)) return ILLM_ERR_ARG;
+    if (pairing != 0 && pairing != 1) return ILLM_ERR_ARG;
+    if (kcache && (!vcache || !page_table || !row_slot || page_size <= 0 || table_stride <= 0))
+        return ILLM_ERR_ARG;
+    if (ring > 0 && !slot_len) return ILLM_ERR_ARG;
+    if (nh + nkv > 65535) return ILLM_ERR_ARG;
+    if (T == 0) return ILLM_OK;
+    hipLaunchKernelGGL(rope_store_kernel, dim3(T, nh + nkv), dim3(64), 0, (hipStream_t)stream, qkv,
+                       dt, cos_sin, rot, pairing, row_pos, row_slot, slot_len, kcache, vcache,
+                       page_table, table_stride, page_size, ring, nh, nkv, hd);
+    return illm_launch_status();
+}
+
+extern "C" int illm_version() { return 1; }

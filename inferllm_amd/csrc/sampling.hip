@@ -1,0 +1,267 @@
+// Next-token choice on the device: argmax, and the reference's sampler
+// (src/utils.cpp:31-115): logits times 1/temp, repeat penalty on the ids of the
+// last-n window (negative logits multiplied, others divided, :46-56), the top_k
+// largest kept (:21-29), softmax with the max subtracted (:65-84), the shortest
+// prefix in descending order whose probability reaches top_p kept and renormalised
+// (:86-101), one draw from what is left (:111-114).
+//
+// The reference sorts on the CPU; here nothing is sorted.  The k-th largest value
+// and the top_p cut are found by bisection over the order-preserving integer image
+// of the floats (ties go to the lower id, as a stable descending sort would put
+// them), and the draw is the inverse CDF over the kept ids in ascending id order
+// at a uniform number that is a hash of (seed, counter): the same request gives the
+// same tokens whatever else is in the batch.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+#define SB 1024  // threads of a sampling block
+
+__device__ __forceinline__ uint32_t order_key(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// splitmix64 of seed + (counter + 1) * golden ratio; 24 bits -> [0, 1)
+__device__ __forceinline__ float uniform_from(uint64_t seed, int32_t counter) {
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (uint64_t)((int64_t)counter + 1);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+template <typename T>
+__device__ __forceinline__ T block_sum_t(T v, T* red) {
+    const int lane = threadIdx.x & (ILLM_WAVE - 1), w = threadIdx.x / ILLM_WAVE;
+#pragma unroll
+    for (int o = ILLM_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, ILLM_WAVE);
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    T t = 0;
+    for (int i = 0; i < SB / ILLM_WAVE; ++i) t += red[i];
+    return t;
+}
+
+// exclusive prefix over the block's threads in thread order; `total` = sum of all
+template <typename T>
+__device__ __forceinline__ T block_exclusive_scan(T v, T* red, T* total) {
+    const int lane = threadIdx.x & (ILLM_WAVE - 1), w = threadIdx.x / ILLM_WAVE;
+    T inc = v;
+#pragma unroll
+    for (int o = 1; o < ILLM_WAVE; o <<= 1) {
+        const T n = __shfl_up(inc, o, ILLM_WAVE);
+        if (lane >= o) inc += n;
+    }
+    __syncthreads();
+    if (lane == ILLM_WAVE - 1) red[w] = inc;
+    __syncthreads();
+    T before = 0, all = 0;
+    for (int i = 0; i < SB / ILLM_WAVE; ++i) {
+        if (i < w) before += red[i];
+        all += red[i];
+    }
+    *total = all;
+    return before + inc - v;
+}
+
+// ---------------------------------------------------------------- argmax
+__global__ void __launch_bounds__(SB)
+argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int V) {
+    __shared__ float bv[SB / ILLM_WAVE];
+    __shared__ int bi[SB / ILLM_WAVE];
+    const float* row = logits + (size_t)blockIdx.x * V;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += SB) {
+        const float v = row[i];
+        if (v > best || (v == best && i < idx) || idx == 0x7fffffff) {
+            if (!(v != v)) { best = v; idx = i; }   // NaN never wins
+        }
+    }
+#pragma unroll
+    for (int o = ILLM_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, ILLM_WAVE);
+        const int oi = __shfl_xor(idx, o, ILLM_WAVE);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int lane = threadIdx.x & (ILLM_WAVE - 1), w = threadIdx.x / ILLM_WAVE;
+    if (lane == 0) { bv[w] = best; bi[w] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < SB / ILLM_WAVE; ++i)
+            if (bv[i] > best || (bv[i] == best && bi[i] < idx)) { best = bv[i]; idx = bi[i]; }
+        out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    }
+}
+
+extern "C" int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream) {
+    if (B < 0 || V <= 0) return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits, out, V);
+    return illm_launch_status();
+}
+
+// ---------------------------------------------------------------- sampler
+struct Keep {  // an id is kept iff key > t, or key == t and id <= cut
+    uint32_t t;
+    int cut;
+};
+
+__device__ __forceinline__ bool kept(const Keep& k, uint32_t key, int id) {
+    return key > k.t || (key == k.t && id <= k.cut);
+}
+
+// id of the r-th (1-based) kept id whose key equals k.t, in ascending id order
+__device__ int nth_equal_id(const float* s, int lo, int hi, const Keep& k, int r, int* red_i,
+                            int* shared_out) {
+    int mine = 0;
+    for (int i = lo; i < hi; ++i) mine += (order_key(s[i]) == k.t && i <= k.cut) ? 1 : 0;
+    int total;
+    const int before = block_exclusive_scan<int>(mine, red_i, &total);
+    __syncthreads();
+    if (threadIdx.x == 0) *shared_out = k.cut;
+    __syncthreads();
+    if (r > before && r <= before + mine) {
+        int c = before;
+        for (int i = lo; i < hi; ++i)
+            if (order_key(s[i]) == k.t && i <= k.cut && ++c == r) { *shared_out = i; break; }
+    }
+    __syncthreads();
+    return *shared_out;
+}
+
+__global__ void __launch_bounds__(SB)
+sample_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
+              int32_t* __restrict__ out, int V, float temp, int top_k, float top_p,
+              float repeat_penalty, const int32_t* __restrict__ last_tokens, int n_last,
+              const uint64_t* __restrict__ seeds, const int32_t* __restrict__ counters) {
+    __shared__ float red_f[SB / ILLM_WAVE];
+    __shared__ int red_i[SB / ILLM_WAVE];
+    __shared__ int last[256];
+    __shared__ int sh_i;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const float* row = logits + (size_t)b * V;
+    float* s = scratch + (size_t)b * V;
+    const int chunk = (V + SB - 1) / SB;
+    const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
+    const int nl = last_tokens ? min(n_last, 256) : 0;
+    if (tid < nl) last[tid] = last_tokens[(size_t)b * n_last + tid];
+    __syncthreads();
+
+    // 1. scaled and penalised scores; their max
+    const float inv_temp = 1.0f / temp;
+    float mx = -INFINITY;
+    for (int i = lo; i < hi; ++i) {
+        float l = row[i];
+        bool rep = false;
+        for (int j = 0; j < nl; ++j) rep |= (last[j] == i);
+        float v = l * inv_temp;
+        if (rep) v = l < 0.f ? v * repeat_penalty : v / repeat_penalty;
+        s[i] = v;
+        mx = fmaxf(mx, v);
+    }
+    mx = block_max(mx, red_f);
+
+    // 2. top_k: largest t with count(key >= t) >= k
+    Keep keep = {0u, V};
+    if (top_k > 0 && top_k < V) {
+        uint32_t t = 0;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = t | (1u << bit);
+            int c = 0;
+            for (int i = lo; i < hi; ++i) c += order_key(s[i]) >= cand ? 1 : 0;
+            if (block_sum_t<int>(c, red_i) >= top_k) t = cand;
+        }
+        int c = 0;
+        for (int i = lo; i < hi; ++i) c += order_key(s[i]) > t ? 1 : 0;
+        const int above = block_sum_t<int>(c, red_i);
+        keep.t = t;
+        keep.cut = nth_equal_id(s, lo, hi, keep, top_k - above, red_i, &sh_i);
+    }
+
+    // 3. top_p over the kept ids, in descending order of score
+    if (top_p < 1.0f) {
+        float z = 0.f;
+        for (int i = lo; i < hi; ++i)
+            if (kept(keep, order_key(s[i]), i)) z += expf(s[i] - mx);
+        z = block_sum_t<float>(z, red_f);
+        const float need = top_p * z;
+        uint32_t t = 0;  // every threshold up to keep.t holds the whole kept mass
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = t | (1u << bit);
+            float mass = 0.f;
+            for (int i = lo; i < hi; ++i) {
+                const uint32_t key = order_key(s[i]);
+                if (key >= cand && kept(keep, key, i)) mass += expf(s[i] - mx);
+            }
+            if (block_sum_t<float>(mass, red_f) >= need) t = cand;
+        }
+        // t is now the largest threshold whose kept mass still reaches top_p
+        float mass = 0.f, eq_p = 0.f;
+        int eq = 0;
+        for (int i = lo; i < hi; ++i) {
+            const uint32_t key = order_key(s[i]);
+            if (!kept(keep, key, i)) continue;
+            if (key > t) mass += expf(s[i] - mx);
+            else if (key == t) { eq += 1; eq_p = expf(s[i] - mx); }
+        }
+        const float above = block_sum_t<float>(mass, red_f);
+        const int n_eq = block_sum_t<int>(eq, red_i);
+        const float one = block_max(eq_p, red_f);
+        int m = one > 0.f ? (int)ceilf((need - above) / one) : n_eq;
+        m = max(1, min(m, n_eq));
+        Keep k2 = {t, keep.t == t ? keep.cut : V};
+        k2.cut = nth_equal_id(s, lo, hi, k2, m, red_i, &sh_i);
+        keep = k2;
+    }
+
+    // 4. inverse CDF over the kept ids in ascending id order
+    float mine = 0.f;
+    for (int i = lo; i < hi; ++i)
+        if (kept(keep, order_key(s[i]), i)) mine += expf(s[i] - mx);
+    float total;
+    const float before = block_exclusive_scan<float>(mine, red_f, &total);
+    const float u = uniform_from(seeds[b], counters[b]);
+    const float target = u * total;
+    __syncthreads();
+    if (tid == 0) sh_i = -1;
+    __syncthreads();
+    if (mine > 0.f && target >= before && target < before + mine) {
+        float c = before;
+        int pick = -1;
+        for (int i = lo; i < hi; ++i) {
+            if (!kept(keep, order_key(s[i]), i)) continue;
+            pick = i;
+            c += expf(s[i] - mx);
+            if (target < c) break;
+        }
+        atomicMax(&sh_i, pick);
+    }
+    __syncthreads();
+    if (sh_i < 0) {
+        // rounding put the target past the last kept id: take that id
+        int lastk = -1;
+        for (int i = lo; i < hi; ++i)
+            if (kept(keep, order_key(s[i]), i)) lastk = i;
+        atomicMax(&sh_i, lastk);
+        __syncthreads();
+    }
+    if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
+}
+
+extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V,
+                           float temp, int top_k, float top_p, float repeat_penalty,
+                           const int32_t* last_tokens, int n_last, const uint64_t* seeds,
+                           const int32_t* counters, void* stream) {
+    if (B < 0 || V <= 0 || !(temp > 0.f) || !(top_p > 0.f) || !(repeat_penalty > 0.f) ||
+        n_last < 0 || n_last > 256 || !seeds || !counters || !scratch)
+        return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    hipLaunchKernelGGL(sample_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits, scratch,
+                       out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last, seeds,
+                       counters);
+    return illm_launch_status();
+}

@@ -1,0 +1,133 @@
+"""The engine: a model folder (or a configuration and a seed) in, logits and
+generated tokens out, on one GPU.
+
+Python entry point of the library, in the role of the reference's `Model` facade
+(include/model.h:27-59: load, init, prefill, decode, decode_iter, reset_token,
+decode_summary) with batches of sequences in place of its single one.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from ..cache.manager import PAGE_SIZE, CacheManager, round_up
+from ..config.registry import config_from_dict, load_config
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from ..weights.loader import load_named_tensors
+from ..weights.random_init import random_tensors
+from .generate import GenerationLoop, GenerationStats
+from .model import DecoderModel
+from .step import StepEntry, StepRunner
+
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16,
+           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    """"float32" or "bfloat16" (the reference's strings are src/core/model_imp.h:17-33)."""
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype!r}: use 'float32' or 'bfloat16'") from None
+
+
+class Engine:
+    """One model on one GPU with its cache, step function and generation loop.
+
+    dtype "bfloat16": weights as stored, bfloat16 activations and cache, float32
+    residual stream, statistics and logits.  dtype "float32": everything in true
+    float32 (own multiply-add kernels; no matrix-core or reduced-precision mode).
+
+    Cache size: `max_tokens` is the most tokens live sequences hold together (each
+    rounded up to 64), `max_batch` the most live sequences, `max_seq_len` the longest
+    sequence (default: the model's max positions).
+    """
+
+    def __init__(self, config, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
+                 max_batch: int = 8, max_seq_len: Optional[int] = None,
+                 max_tokens: Optional[int] = None, use_graphs: bool = True,
+                 poison_freed: bool = False):
+        self.config = config
+        self.dtype = parse_dtype(dtype)
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise ValueError("the engine runs on a GPU only (device 'cuda:N')")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible; the engine has no CPU path")
+        torch.cuda.set_device(self.device)
+        self.spec = config.to_spec()
+        self.model = DecoderModel(self.spec)
+        self.model.load(tensors)
+        limit = self.spec.max_positions
+        self.max_seq_len = min(int(max_seq_len), limit) if max_seq_len else limit
+        self.max_batch = int(max_batch)
+        if max_tokens is None:
+            max_tokens = self.max_batch * round_up(self.max_seq_len, PAGE_SIZE)
+        self.cache = CacheManager(self.model.kv_lines(), self.model.state_lines(),
+                                  max_tokens=int(max_tokens), max_slots=self.max_batch,
+                                  max_seq_len=self.max_seq_len, dtype=self.dtype,
+                                  device=self.device, poison_freed=poison_freed)
+        self.runner = StepRunner(self.model, self.cache, self.dtype, self.device, use_graphs)
+        self.last_stats: Optional[GenerationStats] = None
+
+    # ------------------------------------------------------------ construction
+    @classmethod
+    def from_pretrained(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        """From a folder with config.json and model.safetensors (or its shards)."""
+        config = load_config(model_dir)
+        model = DecoderModel(config.to_spec())
+        tensors = load_named_tensors(model_dir, model.wants(), parse_dtype(dtype), device,
+                                     config.to_spec().ignored_tensor_suffixes)
+        return cls(config, tensors, dtype, device, **kw)
+
+    @classmethod
+    def from_random(cls, config: Union[dict, object], seed: int = 0, dtype="bfloat16",
+                    device="cuda:0", **kw) -> "Engine":
+        """Seeded random weights drawn on the device (no folder is written)."""
+        if isinstance(config, dict):
+            config = config_from_dict(config)
+        dt = parse_dtype(dtype)
+        wants = DecoderModel(config.to_spec()).wants()
+        tensors = dict(random_tensors(wants, seed, dt, device))
+        return cls(config, tensors, dtype, device, **kw)
+
+    # ------------------------------------------------------------ low level
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """See `StepRunner.step`.  The returned tensor is valid until the next step."""
+        return self.runner.step(entries)
+
+    # ------------------------------------------------------------ generation
+    def generate(self, prompts: Sequence[Sequence[int]], temperature: float = 0.0,
+                 top_k: int = 0, top_p: float = 1.0, repeat_penalty: float = 1.0,
+                 repeat_last_n: int = 64, seed: int = 0, max_new_tokens: int = 128,
+                 stop_token_ids: Optional[Sequence[int]] = None,
+                 include_stop: bool = False) -> List[List[int]]:
+        """Generated token ids for every prompt (lists of token ids).
+
+        `stop_token_ids` defaults to the model's eos ids; a stop token ends its
+        sequence and is left out of the result unless `include_stop`."""
+        params = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p,
+                                repeat_penalty=repeat_penalty, repeat_last_n=repeat_last_n,
+                                seed=seed)
+        sampler = Sampler(params, self.device)
+        stops = list(self.spec.eos_token_ids) if stop_token_ids is None else list(stop_token_ids)
+        vocab = self.spec.vocab_size
+        for i, p in enumerate(prompts):
+            for t in p:
+                if not (0 <= int(t) < vocab):
+                    raise ValueError(f"request {i}: token id {t} outside the vocabulary of {vocab}")
+        loop = GenerationLoop(self.step, sampler, self.alloc_slot, self.free_slot,
+                              max_batch=self.max_batch, max_tokens=self.cache.max_tokens,
+                              max_seq_len=self.max_seq_len, page_size=self.cache.page_size,
+                              sync=lambda: torch.cuda.synchronize(self.device))
+        out = loop.run(prompts, params, max_new_tokens, stops, include_stop)
+        self.last_stats = loop.stats
+        return out

@@ -1,0 +1,176 @@
+"""The generation loop above the step function.
+
+Requests are served in batches, one after another: a batch takes as many of the
+waiting prompts (in order) as slots and cache room allow, runs all its prompts
+(unequal lengths) in one step, then one token per live sequence per step.  A
+sequence ends at a stop token, at its `max_new_tokens`, or when it reaches the
+longest length the cache allows; it then leaves the batch (its slot is given
+back) while the others go on.  No request joins a batch that has started.
+
+The loop only decides; computing is behind three callables, so its decisions can
+be tested without a GPU.  The reference's loop is `application/chat.cpp:221-275`
+over `ModelImp::decode_iter` (src/core/model_imp.cpp:55-79): one sequence, ended by
+token 2 or a full context, `n_predict` declared but unused (chat.cpp:23).
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, List, Optional, Sequence
+
+from ..cache.manager import round_up
+from ..sampling.params import SamplingParams, request_seed
+from .step import StepEntry
+
+
+@dataclass
+class GenerationStats:
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_seconds: float = 0.0
+    decode_steps: int = 0
+    batches: int = 0
+
+    def summary(self) -> str:
+        """Like the reference's decode_summary (src/core/model_imp.cpp:133-141), but the
+        decode rate counts generated tokens only."""
+        pf = self.prompt_tokens / self.prefill_seconds if self.prefill_seconds > 0 else 0.0
+        decoded = max(0, self.generated_tokens - self.batches)   # first tokens come from prefill
+        dc = decoded / self.decode_seconds if self.decode_seconds > 0 else 0.0
+        return (f"prefill: {self.prompt_tokens} tokens, {self.prefill_seconds * 1e3:.1f} ms, "
+                f"{pf:.1f} token/s\n"
+                f"decode:  {self.generated_tokens} tokens in {self.decode_steps} steps, "
+                f"{self.decode_seconds * 1e3:.1f} ms, {dc:.1f} token/s")
+
+
+@dataclass
+class _Live:
+    index: int                 # request index in the call
+    slot: int
+    prompt_len: int
+    seed: int
+    out: List[int] = field(default_factory=list)
+    history: List[int] = field(default_factory=list)
+
+
+class GenerationLoop:
+    """`step(entries) -> logits`, `sample(logits, seeds, counters, histories) -> ids`,
+    `alloc_slot() -> slot`, `free_slot(slot)`; limits of the cache as numbers."""
+
+    def __init__(self, step: Callable, sample: Callable, alloc_slot: Callable[[], int],
+                 free_slot: Callable[[int], None], max_batch: int, max_tokens: int,
+                 max_seq_len: int, page_size: int = 64, sync: Optional[Callable[[], None]] = None):
+        self.step, self.sample = step, sample
+        self.alloc_slot, self.free_slot = alloc_slot, free_slot
+        self.max_batch, self.max_tokens, self.max_seq_len = max_batch, max_tokens, max_seq_len
+        self.page_size = page_size
+        self.sync = sync or (lambda: None)
+        self.stats = GenerationStats()
+
+    # ------------------------------------------------------------ decisions
+    def room_needed(self, prompt_len: int, max_new_tokens: int) -> int:
+        """Cache room to set aside for a request: the tokens it can come to hold, in whole pages.
+        The last generated token is never fed back, so it needs no room."""
+        most = min(self.max_seq_len, prompt_len + max(0, max_new_tokens - 1))
+        return round_up(max(most, 1), self.page_size)
+
+    def next_batch(self, waiting: Sequence[int], prompt_lens: Sequence[int],
+                   max_new_tokens: int) -> List[int]:
+        """The prefix of `waiting` (request indices) that fits slots and cache room."""
+        batch: List[int] = []
+        room = 0
+        for i in waiting:
+            need = self.room_needed(prompt_lens[i], max_new_tokens)
+            if len(batch) >= self.max_batch or room + need > self.max_tokens:
+                break
+            batch.append(i)
+            room += need
+        if not batch:
+            i = waiting[0]
+            raise ValueError(f"request {i} ({prompt_lens[i]} prompt tokens, {max_new_tokens} new) "
+                             f"needs more cache room than there is ({self.max_tokens} tokens)")
+        return batch
+
+    @staticmethod
+    def ended(token: int, n_generated: int, total_len: int, stop_ids, max_new_tokens: int,
+              max_seq_len: int) -> Optional[str]:
+        """Why a sequence ends after drawing `token`, or None if it goes on.
+        total_len: tokens of the sequence, the drawn one included."""
+        if token in stop_ids:
+            return "stop"
+        if n_generated >= max_new_tokens:
+            return "length"
+        if total_len > max_seq_len:
+            return "context"        # the drawn token could not be fed back
+        return None
+
+    # ------------------------------------------------------------ the loop
+    def run(self, prompts: Sequence[Sequence[int]], params: SamplingParams, max_new_tokens: int,
+            stop_token_ids: Sequence[int] = (), include_stop: bool = False) -> List[List[int]]:
+        for i, p in enumerate(prompts):
+            if len(p) == 0:
+                raise ValueError(f"request {i}: empty prompt")
+            if len(p) > self.max_seq_len:
+                raise ValueError(f"request {i}: prompt of {len(p)} tokens is longer than the "
+                                 f"cache allows ({self.max_seq_len})")
+        stop_ids = set(int(t) for t in stop_token_ids)
+        results: List[List[int]] = [[] for _ in prompts]
+        if max_new_tokens <= 0:
+            return results
+        waiting = list(range(len(prompts)))
+        lens = [len(p) for p in prompts]
+        while waiting:
+            batch = self.next_batch(waiting, lens, max_new_tokens)
+            waiting = waiting[len(batch):]
+            self._run_batch(batch, prompts, params, max_new_tokens, stop_ids, include_stop, results)
+        return results
+
+    def _run_batch(self, batch, prompts, params, max_new_tokens, stop_ids, include_stop, results):
+        live: List[_Live] = []
+        try:
+            for i in batch:
+                live.append(_Live(index=i, slot=self.alloc_slot(), prompt_len=len(prompts[i]),
+                                  seed=request_seed(params.seed, i),
+                                  history=[int(t) for t in prompts[i]]))
+            self.stats.batches += 1
+            self.sync()
+            t0 = time.perf_counter()
+            logits = self.step([StepEntry(s.slot, prompts[s.index], [s.prompt_len - 1])
+                                for s in live])
+            tokens = self.sample(logits, [s.seed for s in live], [0] * len(live),
+                                 [s.history for s in live])
+            self.sync()
+            self.stats.prefill_seconds += time.perf_counter() - t0
+            self.stats.prompt_tokens += sum(s.prompt_len for s in live)
+            t0 = time.perf_counter()
+            while True:
+                going: List[_Live] = []
+                for s, tok in zip(live, tokens):
+                    tok = int(tok)
+                    self.stats.generated_tokens += 1
+                    why = self.ended(tok, len(s.out) + 1, s.prompt_len + len(s.out) + 1, stop_ids,
+                                     max_new_tokens, self.max_seq_len)
+                    if why != "stop" or include_stop:
+                        s.out.append(tok)
+                    s.history.append(tok)
+                    if why is None:
+                        going.append(s)
+                    else:
+                        results[s.index] = s.out
+                        self.free_slot(s.slot)
+                        s.slot = -1
+                live = going
+                if not live:
+                    break
+                logits = self.step([StepEntry(s.slot, [s.history[-1]], [0]) for s in live])
+                tokens = self.sample(logits, [s.seed for s in live], [len(s.out) for s in live],
+                                     [s.history for s in live])
+                self.stats.decode_steps += 1
+            self.sync()
+            self.stats.decode_seconds += time.perf_counter() - t0
+        finally:
+            for s in live:
+                if s.slot >= 0:
+                    self.free_slot(s.slot)
+                    s.slot = -1

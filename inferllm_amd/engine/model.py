@@ -1,0 +1,105 @@
+"""A decoder built from a `ModelSpec`: embedding, blocks, the order they run in,
+last norm, head.  Nothing here knows an architecture by name.
+
+The reference's counterpart is `Graph`: a list of modules run in order
+(src/core/graph.cpp:166-197) built by `construct_llm` (src/graph/llama_like.cpp:54-109).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..cache.manager import KVSpec, StateSpec
+from ..config.spec import ModelSpec
+from ..parts import build_part, part_class
+from ..parts.base import Block, StepContext
+from ..weights.loader import TensorWant
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = build_part("embedding", spec.embedding)
+        self.layers: List[Block] = []
+        for ls in spec.layers:
+            position = build_part("position", ls.position) if ls.position is not None else None
+            self.layers.append(part_class("block", ls.block)(
+                mixer=build_part("mixer", ls.mixer),
+                feed_forward=build_part("feed_forward", ls.feed_forward),
+                mixer_norm=build_part("norm", ls.mixer_norm),
+                feed_forward_norm=build_part("norm", ls.feed_forward_norm),
+                position=position))
+        self.final_norm = build_part("norm", spec.final_norm)
+        self.head = build_part("head", spec.head)
+        self.schedule = list(spec.schedule)
+        for e in self.schedule:
+            if not (0 <= e.layer < len(self.layers)):
+                raise ValueError(f"schedule names layer {e.layer}; the model has {len(self.layers)}")
+        writers = {}
+        for e in self.schedule:
+            if e.writes_cache:
+                writers.setdefault(e.cache_line, e.layer)
+            elif e.cache_line not in writers:
+                raise ValueError(f"schedule: cache line {e.cache_line} is read before any run writes it")
+        self.loaded = False
+
+    # ------------------------------------------------------------ weights
+    def wants(self) -> Dict[str, TensorWant]:
+        out: Dict[str, TensorWant] = {}
+        for part in [self.embedding, *self.layers, self.final_norm, self.head]:
+            for name, want in part.wants().items():
+                if name in out and tuple(out[name].shape) != tuple(want.shape):
+                    raise ValueError(f"tensor {name!r} is wanted with two shapes: "
+                                     f"{out[name].shape} and {want.shape}")
+                if name in out and not out[name].optional:
+                    continue
+                out[name] = want
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for part in [self.embedding, *self.layers, self.final_norm, self.head]:
+            part.load(tensors)
+        self.loaded = True
+
+    # ------------------------------------------------------------ cache needs
+    def kv_lines(self) -> Dict[int, KVSpec]:
+        out: Dict[int, KVSpec] = {}
+        for e in self.schedule:
+            spec = self.layers[e.layer].mixer.kv_spec()
+            if spec is None:
+                continue
+            if e.cache_line in out and out[e.cache_line] != spec:
+                raise ValueError(f"cache line {e.cache_line} is shared by mixers with different needs")
+            out[e.cache_line] = spec
+        return out
+
+    def state_lines(self) -> Dict[int, StateSpec]:
+        out: Dict[int, StateSpec] = {}
+        for e in self.schedule:
+            spec = self.layers[e.layer].mixer.state_spec()
+            if spec is not None:
+                out[e.cache_line] = spec
+        return out
+
+    # ------------------------------------------------------------ compute
+    def forward(self, ctx: StepContext, out_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """Run the step's rows through every scheduled layer; logits (float32
+        [len(out_rows), vocab]) for the rows asked for, or None if none is."""
+        x = self.embedding.forward(ctx)
+        for layer in self.layers:
+            if layer.position is not None:
+                layer.position.on_embedding(x, ctx)
+                break
+        pending = None
+        for e in self.schedule:
+            pending = self.layers[e.layer].forward(x, pending, ctx, e.cache_line, e.writes_cache)
+        if out_rows is None or out_rows.numel() == 0:
+            return None
+        h = self.final_norm.forward(x, pending, ctx, row_idx=out_rows)
+        return self.head.forward(h, ctx)
+
+
+def expected_tensors(spec: ModelSpec) -> Dict[str, TensorWant]:
+    """Checkpoint tensor name -> shape and kind, for a spec (no weights are allocated)."""
+    return DecoderModel(spec).wants()

@@ -1,0 +1,190 @@
+"""The step function: one batch of sequences, either all at their first token
+(whole prompts of unequal lengths) or all going on by one token.
+
+It runs only the tokens it is given, packed as one batch, against the cache that
+earlier steps left, and returns float32 logits at the places asked for.  Steps
+of single tokens are replayed from a HIP graph captured per batch-size bucket;
+rows that only fill a bucket up use the cache's spare slot and page and change
+no result.
+
+The reference's counterpart is `Graph::execute(tokens, logits, nr_past, prefill)`
+for one sequence, with logits of the last token only and none on prefill
+(src/core/graph.cpp:166-197).
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..parts.base import StepContext
+from .model import DecoderModel
+
+
+class StepError(ValueError):
+    """A batch the step function does not take (mixed phases, bad token ids, ...)."""
+
+
+@dataclass
+class StepEntry:
+    """One sequence's share of a step: its slot, its next tokens and the indices
+    among these tokens whose logits are wanted."""
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=tuple)
+
+
+def _bucket(n: int) -> int:
+    b = 1
+    while b < n:
+        b *= 2
+    return b
+
+
+class _DecodeGraph:
+    """Static buffers and the captured graph for decode steps of one bucket size."""
+
+    def __init__(self, runner: "StepRunner", size: int):
+        self.size = size
+        dev = runner.device
+        self.meta = torch.zeros(3 * size, dtype=torch.int32, device=dev)   # tokens | pos | slot
+        self.cu = torch.arange(size + 1, dtype=torch.int32, device=dev)
+        self.rows = torch.arange(size, dtype=torch.int32, device=dev)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+
+    def context(self, runner: "StepRunner") -> StepContext:
+        n = self.size
+        return StepContext(
+            device=runner.device, act_dtype=runner.act_dtype, prefill=False, n_rows=n, n_seqs=n,
+            tokens=self.meta[:n], row_pos=self.meta[n:2 * n], row_slot=self.meta[2 * n:],
+            cu_seqlens=self.cu, seq_slot=self.meta[2 * n:], max_len=runner.cache.max_seq_len,
+            cache=runner.cache)
+
+
+class StepRunner:
+    """Owns the model, the cache and the decode graphs; `step` is the one entry."""
+
+    def __init__(self, model: DecoderModel, cache: CacheManager, act_dtype: torch.dtype,
+                 device: torch.device, use_graphs: bool = True):
+        self.model, self.cache = model, cache
+        self.act_dtype, self.device = act_dtype, device
+        self.vocab_size = model.spec.vocab_size
+        self.use_graphs = use_graphs and os.environ.get("INFERLLM_NO_GRAPH", "0") != "1"
+        self._graphs: Dict[int, _DecodeGraph] = {}
+
+    # ------------------------------------------------------------ checks
+    def _phase(self, entries: Sequence[StepEntry]) -> bool:
+        """True for a step of whole prompts, False for a step of single tokens."""
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        slots = [e.slot for e in entries]
+        if len(set(slots)) != len(slots):
+            raise StepError("a slot appears twice in one step")
+        for e in entries:
+            if len(e.tokens) == 0:
+                raise StepError(f"slot {e.slot}: no tokens in this step")
+            for t in e.tokens:
+                if not (0 <= int(t) < self.vocab_size):
+                    raise StepError(f"slot {e.slot}: token id {t} outside the vocabulary "
+                                    f"of {self.vocab_size}")
+            for w in e.want:
+                if not (0 <= int(w) < len(e.tokens)):
+                    raise StepError(f"slot {e.slot}: wanted place {w} is not among the "
+                                    f"{len(e.tokens)} tokens of this step")
+        starts = [self.cache.length(e.slot) == 0 for e in entries]
+        if all(starts):
+            return True
+        if not any(starts) and all(len(e.tokens) == 1 for e in entries):
+            return False
+        raise StepError("the sequences of a step must either all start at their first token "
+                        "or all go on by one token")
+
+    # ------------------------------------------------------------ the step
+    @torch.no_grad()
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one step; float32 logits [wanted, vocab] in the order of the entries
+        and of their `want`, or None when nothing is wanted."""
+        prefill = self._phase(entries)
+        starts = [self.cache.length(e.slot) for e in entries]
+        for e, s in zip(entries, starts):
+            self.cache.extend(e.slot, s, len(e.tokens))
+        self.cache.upload()
+        if prefill:
+            return self._prefill(entries)
+        return self._decode(entries, starts)
+
+    def _prefill(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        tokens: List[int] = []
+        pos: List[int] = []
+        slot: List[int] = []
+        cu = [0]
+        want: List[int] = []
+        for e in entries:
+            n = len(e.tokens)
+            want.extend(cu[-1] + int(w) for w in e.want)
+            tokens.extend(int(t) for t in e.tokens)
+            pos.extend(range(n))
+            slot.extend([e.slot] * n)
+            cu.append(cu[-1] + n)
+        T, B = len(tokens), len(entries)
+        host = torch.tensor(tokens + pos + slot + cu + [e.slot for e in entries] + want,
+                            dtype=torch.int32)
+        meta = host.to(self.device)
+        o = 0
+        parts = []
+        for n in (T, T, T, B + 1, B, len(want)):
+            parts.append(meta[o:o + n])
+            o += n
+        ctx = StepContext(
+            device=self.device, act_dtype=self.act_dtype, prefill=True, n_rows=T, n_seqs=B,
+            tokens=parts[0], row_pos=parts[1], row_slot=parts[2], cu_seqlens=parts[3],
+            seq_slot=parts[4], max_len=max(len(e.tokens) for e in entries), cache=self.cache)
+        return self.model.forward(ctx, parts[5] if want else None)
+
+    def _decode(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> Optional[torch.Tensor]:
+        B = len(entries)
+        size = _bucket(B) if self.use_graphs else B
+        pad = size - B
+        spare = self.cache.spare_slot
+        host = torch.tensor([int(e.tokens[0]) for e in entries] + [0] * pad
+                            + list(starts) + [0] * pad
+                            + [e.slot for e in entries] + [spare] * pad, dtype=torch.int32)
+        wanted = [i for i, e in enumerate(entries) if len(e.want)]
+        if not self.use_graphs:
+            meta = host.to(self.device)
+            ctx = StepContext(
+                device=self.device, act_dtype=self.act_dtype, prefill=False, n_rows=B, n_seqs=B,
+                tokens=meta[:B], row_pos=meta[B:2 * B], row_slot=meta[2 * B:],
+                cu_seqlens=torch.arange(B + 1, dtype=torch.int32, device=self.device),
+                seq_slot=meta[2 * B:], max_len=max(starts) + 1, cache=self.cache)
+            rows = torch.tensor(wanted, dtype=torch.int32, device=self.device) if wanted else None
+            return self.model.forward(ctx, rows)
+        g = self._graphs.get(size)
+        if g is None:
+            g = self._graphs[size] = _DecodeGraph(self, size)
+        g.meta.copy_(host)
+        if g.graph is None:
+            self._capture(g)
+        g.graph.replay()
+        if not wanted:
+            return None
+        if wanted == list(range(B)):
+            return g.logits[:B]
+        return g.logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
+
+    def _capture(self, g: _DecodeGraph) -> None:
+        ctx = g.context(self)
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            self.model.forward(ctx, g.rows)        # warm-up: the libraries set themselves up
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            g.logits = self.model.forward(g.context(self), g.rows)
+        g.graph = graph

@@ -1,0 +1,275 @@
+"""The kernel library as Python functions over torch tensors.
+
+Every function checks on the host that shapes, dtypes and devices are what its
+kernel and launch grid assume, then launches on torch's current HIP stream.
+Tensors must live on the GPU: there is no CPU path, and a missing or unbuildable
+library raises (`kernels.build.KernelLibraryError`).  Parts call these through the
+module (`ops.add_rmsnorm(...)`).
+
+Matrix products: float32 operands always go to the library's own float32 kernel
+(plain fused multiply-adds, fixed summation order).  bfloat16 operands go to the
+MFMA kernels of this library when the shape fits them (few rows: decoding), and
+to the vendor GEMM through `torch.matmul` otherwise, which is where the reference
+uses a vendor GEMM too (cublasSgemm, src/kern/gpu/kernel_gpu.cu:420-435).
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+_ERRORS = {1: "sizes or dtypes the kernel does not take", 2: "the HIP runtime refused the launch"}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _lib():
+    return build.library()
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"dtype {t.dtype} is not served (float32 and bfloat16 are)") from None
+
+
+def _p(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must be on the GPU (there is no CPU path)")
+            _need(t.is_contiguous(), "kernel operands must be contiguous")
+
+
+def _i32(t: Optional[torch.Tensor], n: Optional[int] = None) -> None:
+    if t is not None:
+        _need(t.dtype == torch.int32, "index tensors must be int32")
+        if n is not None:
+            _need(t.numel() >= n, f"index tensor has {t.numel()} entries, {n} needed")
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise KernelError(f"{what}: {_ERRORS.get(rc, rc)}")
+
+
+# ------------------------------------------------------------------ rows
+def embed(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """float32 [T, E] rows of `table` [V, E] at int32 `tokens` [T]."""
+    _gpu(tokens, table)
+    _i32(tokens)
+    _need(table.dim() == 2 and tokens.dim() == 1, "embed: tokens [T], table [V, E]")
+    T, (V, E) = tokens.numel(), table.shape
+    out = torch.empty((T, E), dtype=torch.float32, device=table.device)
+    _check(_lib().illm_embed(_p(tokens), _p(table), _code(table), _p(out), T, E, V, _stream()),
+           "embed")
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMS norm of the float32 residual rows `x` [T, E] after adding `delta` to them.
+
+    Without `row_idx` the sum is written back to `x`.  With `row_idx` only those
+    rows are normed (and `x` is left as it is).
+    """
+    _gpu(x, delta, weight, row_idx)
+    _i32(row_idx)
+    _need(x.dtype == torch.float32 and x.dim() == 2, "add_rmsnorm: x must be float32 [T, E]")
+    T, E = x.shape
+    _need(weight.shape == (E,), f"add_rmsnorm: weight {tuple(weight.shape)} for width {E}")
+    if delta is not None:
+        _need(delta.shape == x.shape, "add_rmsnorm: delta must have x's shape")
+    rows = T if row_idx is None else row_idx.numel()
+    out = torch.empty((rows, E), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_add_rmsnorm(
+        _p(x), _p(delta), _code(delta) if delta is not None else 0, _p(weight), _code(weight),
+        _p(out), _code(out), _p(row_idx), rows, E, ctypes.c_float(eps), _stream()), "add_rmsnorm")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up from rows [gate (F) | up (F)]."""
+    _gpu(gate_up)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "silu_mul: rows of [gate | up]")
+    T, F2 = gate_up.shape
+    out = torch.empty((T, F2 // 2), dtype=gate_up.dtype, device=gate_up.device)
+    _check(_lib().illm_silu_mul(_p(gate_up), _p(out), _code(gate_up), T, F2 // 2, _stream()),
+           "silu_mul")
+    return out
+
+
+def rope_store(qkv: torch.Tensor, cos_sin: Optional[torch.Tensor], rot: int, pairing: int,
+               row_pos: torch.Tensor, row_slot: Optional[torch.Tensor],
+               slot_len: Optional[torch.Tensor], kcache: Optional[torch.Tensor],
+               vcache: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+               page_size: int, ring: int, nh: int, nkv: int, hd: int) -> None:
+    """Rotate q and k of packed rows in place; store k and v in the paged cache.
+
+    qkv [T, (nh + 2 nkv) hd]; cos_sin float32 [max_pos, rot/2, 2] or None (no rotation);
+    kcache / vcache [pages, nkv, page_size, hd] or None (nothing stored);
+    page_table int32 [slots, pages per sequence].
+    """
+    _gpu(qkv, cos_sin, row_pos, row_slot, slot_len, kcache, vcache, page_table)
+    _i32(row_pos, qkv.shape[0]); _i32(row_slot, qkv.shape[0]); _i32(slot_len); _i32(page_table)
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd,
+          f"rope_store: rows of {qkv.shape[1]} for {nh}+2*{nkv} heads of {hd}")
+    max_pos = 0
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and
+              cos_sin.shape[1] * 2 == rot and cos_sin.shape[2] == 2,
+              "rope_store: angle table must be float32 [max_pos, rot/2, 2]")
+        max_pos = cos_sin.shape[0]
+    stride = 1
+    if kcache is not None:
+        _need(vcache is not None and page_table is not None and row_slot is not None,
+              "rope_store: a cache needs vcache, page_table and row_slot")
+        _need(kcache.dtype == qkv.dtype and vcache.dtype == qkv.dtype,
+              "rope_store: cache dtype differs from the activations'")
+        _need(kcache.shape[1:] == (nkv, page_size, hd) and vcache.shape == kcache.shape,
+              f"rope_store: cache shape {tuple(kcache.shape)} vs (pages, {nkv}, {page_size}, {hd})")
+        _need(page_table.dim() == 2, "rope_store: page_table [slots, pages]")
+        stride = page_table.shape[1]
+    _check(_lib().illm_rope_store(
+        _p(qkv), _code(qkv), _p(cos_sin), max_pos, rot, pairing, _p(row_pos), _p(row_slot),
+        _p(slot_len), _p(kcache), _p(vcache), _p(page_table), stride, page_size, ring, T, nh, nkv,
+        hd, _stream()), "rope_store")
+
+
+# ------------------------------------------------------------------ products
+def gemm_generic(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M, K] . w [N, K]^T by the library's float32 multiply-add kernel."""
+    _gpu(x, w)
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1],
+          f"linear: x {tuple(x.shape)} against w {tuple(w.shape)}")
+    M, K = x.shape
+    N = w.shape[0]
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_gemm_generic(_p(x), _code(x), _p(w), _code(w), _p(y), _code(y), M, N, K,
+                                    _stream()), "gemm_generic")
+    return y
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x . w^T, w stored [out, in] (src/kern/naive/naive.cpp:363-379)."""
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.float32 or w.dtype == torch.float32:
+        return gemm_generic(x, w, out_dtype)
+    M, K = x.shape
+    if M <= SKINNY_MAX_ROWS and skinny_fits(M, w.shape[0], K):
+        return gemm_skinny_bf16(x, w, out_dtype)
+    _gpu(x, w)
+    y = torch.matmul(x, w.t())
+    return y if out_dtype == y.dtype else y.to(out_dtype)
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def skinny_fits(M: int, N: int, K: int) -> bool:
+    return False
+
+
+def gemm_skinny_bf16(x, w, out_dtype):
+    raise KernelError("no skinny kernel in this build")
+
+
+# ------------------------------------------------------------------ attention
+def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_len: int, nh: int,
+                 nkv: int, hd: int, scale: float, window: int) -> torch.Tensor:
+    """Causal attention of whole prompts over packed rows; returns [T, nh * hd]."""
+    _gpu(qkv, cu_seqlens)
+    _i32(cu_seqlens, n_seqs + 1)
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_prefill: packed qkv rows")
+    _need(nh % nkv == 0, "attn_prefill: heads must be a multiple of kv heads")
+    out = torch.empty((T, nh * hd), dtype=qkv.dtype, device=qkv.device)
+    _check(_lib().illm_attn_prefill_generic(
+        _p(qkv), _p(out), _code(qkv), _p(cu_seqlens), n_seqs, max_len, nh, nkv, hd,
+        ctypes.c_float(scale), window, _stream()), f"attn_prefill (head_dim {hd})")
+    return out
+
+
+def decode_splits(B: int, nh: int, max_len: int) -> int:
+    """How many ways to cut the keys of a decode step so that the launch fills the chip."""
+    blocks = max(1, B * nh)
+    want = max(1, 1024 // blocks)
+    tiles = max(1, (max_len + 255) // 256)
+    return max(1, min(want, tiles, 64))
+
+
+def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                page_table: torch.Tensor, page_size: int, ring: int, seq_slot: torch.Tensor,
+                slot_len: torch.Tensor, nh: int, nkv: int, hd: int, scale: float, window: int,
+                nsplit: int) -> torch.Tensor:
+    """One new token per sequence against the paged cache; returns [B, nh * hd]."""
+    _gpu(qkv, kcache, vcache, page_table, seq_slot, slot_len)
+    _i32(page_table); _i32(seq_slot, qkv.shape[0]); _i32(slot_len)
+    B = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_decode: packed qkv rows")
+    _need(kcache.dtype == qkv.dtype and vcache.shape == kcache.shape and
+          kcache.shape[1:] == (nkv, page_size, hd), "attn_decode: cache shape or dtype")
+    _need(nh % nkv == 0, "attn_decode: heads must be a multiple of kv heads")
+    out = torch.empty((B, nh * hd), dtype=qkv.dtype, device=qkv.device)
+    partial = torch.empty((B, nh, nsplit, hd + 2), dtype=torch.float32, device=qkv.device)
+    _check(_lib().illm_attn_decode_generic(
+        _p(qkv), _p(out), _code(qkv), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
+        page_size, ring, _p(seq_slot), _p(slot_len), _p(partial), nsplit, B, nh, nkv, hd,
+        ctypes.c_float(scale), window, _stream()), f"attn_decode (head_dim {hd})")
+    return out
+
+
+# ------------------------------------------------------------------ sampling
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    _gpu(logits)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "argmax: float32 [B, V]")
+    B, V = logits.shape
+    out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    _check(_lib().illm_argmax(_p(logits), _p(out), B, V, _stream()), "argmax")
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float,
+           repeat_penalty: float, last_tokens: Optional[torch.Tensor], seeds: torch.Tensor,
+           counters: torch.Tensor) -> torch.Tensor:
+    """One draw per row; see csrc/sampling.hip.  seeds: int64 [B] (bit pattern used), counters int32 [B]."""
+    _gpu(logits, last_tokens, seeds, counters)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample: float32 [B, V]")
+    B, V = logits.shape
+    _need(seeds.dtype == torch.int64 and seeds.numel() >= B, "sample: seeds int64 [B]")
+    _i32(counters, B); _i32(last_tokens)
+    n_last = 0
+    if last_tokens is not None:
+        _need(last_tokens.dim() == 2 and last_tokens.shape[0] == B, "sample: last_tokens [B, n]")
+        n_last = last_tokens.shape[1]
+    _need(temperature > 0 and top_p > 0 and repeat_penalty > 0 and n_last <= 256,
+          "sample: temperature, top_p and repeat_penalty must be positive, window <= 256")
+    out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+    scratch = torch.empty((B, V), dtype=torch.float32, device=logits.device)
+    _check(_lib().illm_sample(
+        _p(logits), _p(scratch), _p(out), B, V, ctypes.c_float(temperature), int(top_k),
+        ctypes.c_float(top_p), ctypes.c_float(repeat_penalty), _p(last_tokens), n_last, _p(seeds),
+        _p(counters), _stream()), "sample")
+    return out

@@ -1,0 +1,99 @@
+"""Causal self-attention with grouped kv heads over the paged cache."""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from ..cache.manager import KVSpec
+from ..kernels import ops
+from ..weights.loader import TensorWant
+from .base import Mixer, StepContext, register_part
+
+
+def _fuse(ws):
+    """One [sum of outs, in] matrix from several; float32 if the stored dtypes differ."""
+    if len({w.dtype for w in ws}) > 1:
+        ws = [w.to(torch.float32) for w in ws]
+    return torch.cat(ws, dim=0).contiguous()
+
+
+@register_part("mixer", "attention")
+class Attention(Mixer):
+    """q, k, v projections (one fused product), position encoding of q and k, the
+    store of k and v, softmax(q k^T * scale + causal mask) v, output projection.
+
+    src/core/op.cpp:412-498 with src/core/graph.h:107-111 (the `wo` product); scale
+    1/sqrt(head_dim) after the dot product (op.cpp:488).  Query head h reads kv head
+    h / (num_heads / num_kv_heads) (src/kern/naive/naive.cpp:576-604).  `window`
+    keeps only the last `window` keys visible; `softmax_scale` replaces the default.
+    Whole prompts attend over the step's own rows; single tokens over the cache.
+    """
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 window: Optional[int] = None, softmax_scale: Optional[float] = None, tensors=None):
+        super().__init__(tensors)
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if head_dim > 256:
+            raise ValueError(f"head_dim {head_dim} is beyond the attention kernels' limit of 256")
+        self.E, self.nh, self.nkv, self.hd = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.window = int(window) if window else None
+        self.scale = float(softmax_scale) if softmax_scale else 1.0 / math.sqrt(self.hd)
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        return {"q": TensorWant((self.nh * self.hd, self.E)),
+                "k": TensorWant((self.nkv * self.hd, self.E)),
+                "v": TensorWant((self.nkv * self.hd, self.E)),
+                "o": TensorWant((self.E, self.nh * self.hd))}
+
+    def kv_spec(self) -> KVSpec:
+        return KVSpec("window" if self.window else "full", self.nkv, self.hd, self.window)
+
+    def load(self, tensors) -> None:
+        self.w_qkv = _fuse([self._take(tensors, n) for n in ("q", "k", "v")])
+        self.w_o = self._take(tensors, "o").contiguous()
+
+    def forward(self, h, ctx: StepContext, line, writes_cache, position):
+        nh, nkv, hd = self.nh, self.nkv, self.hd
+        kc, vc, group = ctx.cache.kv_line(line)
+        window = self.window or 0
+        if writes_cache:
+            qkv = ops.linear(h, self.w_qkv)
+            if position is not None:
+                position.on_qkv(qkv, ctx, nh, nkv, hd, kc, vc, group)
+            else:
+                ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot, ctx.cache.slot_len, kc,
+                               vc, group.table, group.page_size, group.ring, nh, nkv, hd)
+            if ctx.prefill:
+                ctx.exchange[("kv_rows", line)] = qkv
+        else:
+            # keys and values are those that an earlier run of this step stored on the line
+            q = ops.linear(h, self.w_qkv[: nh * hd])
+            if ctx.prefill:
+                src = ctx.exchange[("kv_rows", line)]
+                qkv = torch.cat([q, src[:, nh * hd:]], dim=1)
+            else:
+                qkv = torch.cat([q, q.new_zeros((q.shape[0], 2 * nkv * hd))], dim=1)
+            if position is not None:
+                # rotates q (and the copied k again is avoided by handing no k heads: see below)
+                self._encode_q_only(qkv, ctx, position)
+        if ctx.prefill:
+            o = ops.attn_prefill(qkv, ctx.cu_seqlens, ctx.n_seqs, ctx.max_len, nh, nkv, hd,
+                                 self.scale, window)
+        else:
+            nsplit = ops.decode_splits(ctx.n_seqs, nh, ctx.max_len if not window else min(ctx.max_len, window))
+            o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
+                                ctx.seq_slot, ctx.cache.slot_len, nh, nkv, hd, self.scale, window,
+                                nsplit)
+        return ops.linear(o, self.w_o)
+
+    def _encode_q_only(self, qkv, ctx, position) -> None:
+        nh, nkv, hd = self.nh, self.nkv, self.hd
+        q = qkv[:, : nh * hd].contiguous()
+        # a q-only view: rows of nh heads and no kv heads
+        position.on_qkv(q, ctx, nh, 0, hd, None, None, None)
+        qkv[:, : nh * hd] = q

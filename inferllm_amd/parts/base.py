@@ -1,0 +1,175 @@
+"""Interfaces of the parts a decoder is put together from, and their registries.
+
+A part is built from keyword parameters (its sizes and constants) and a map from
+its own parameter names to checkpoint tensor names.  It says which tensors it
+wants (`wants`), takes them (`load`) and computes (`forward`).  No part knows
+which model it is in: everything it needs comes through its constructor and the
+`StepContext` of the step.
+
+Five kinds: mixer (attention and whatever else mixes tokens), feed-forward, norm,
+position encoding, block (the arrangement of the other four around the residual
+stream); plus the embedding and the head at the model's ends.  Each kind has a
+registry from a name to a class, so another part is added by registering a class,
+without touching the files here.  The reference assembles its graph the same way
+from ops with constants as constructor arguments (src/graph/llama_like.cpp:54-109).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional
+
+import torch
+
+from ..cache.manager import CacheManager, KVSpec, StateSpec
+from ..weights.loader import TensorWant
+
+
+@dataclass
+class StepContext:
+    """What a step hands to every part.
+
+    Rows are the step's tokens, packed sequence after sequence.  All index tensors
+    are int32 on the device.  `prefill` steps carry whole prompts that start at
+    position 0; other steps carry one token per sequence.
+    """
+    device: torch.device
+    act_dtype: torch.dtype            # dtype of activations between kernels (residual is float32)
+    prefill: bool
+    n_rows: int
+    n_seqs: int
+    tokens: torch.Tensor              # [rows]
+    row_pos: torch.Tensor             # [rows] absolute position of each row
+    row_slot: torch.Tensor            # [rows] cache slot of each row
+    cu_seqlens: torch.Tensor          # [seqs + 1] row offsets of the sequences
+    seq_slot: torch.Tensor            # [seqs]
+    max_len: int                      # longest sequence after this step (host number)
+    cache: CacheManager
+    exchange: Dict[Any, Any] = field(default_factory=dict)   # between runs of layers in one step
+
+
+class Part:
+    """Base of all parts: parameter names -> checkpoint names in `self.tensors`."""
+
+    def __init__(self, tensors: Optional[Dict[str, str]] = None):
+        self.tensors: Dict[str, str] = dict(tensors or {})
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        """Own parameter name -> what is wanted of it."""
+        return {}
+
+    def wants(self) -> Dict[str, TensorWant]:
+        """Checkpoint tensor name -> what is wanted of it."""
+        return {self.tensors[p]: w for p, w in self.shapes().items()}
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Take the wanted tensors out of `tensors` (checkpoint name -> tensor on the device)."""
+
+    def _take(self, tensors: Dict[str, torch.Tensor], param: str) -> torch.Tensor:
+        return tensors[self.tensors[param]]
+
+
+class Mixer(Part):
+    def kv_spec(self) -> Optional[KVSpec]:
+        """Keys/values the mixer keeps per token, or None."""
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        """Fixed-size state the mixer keeps per sequence, or None."""
+        return None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, line: int, writes_cache: bool,
+                position: Optional["PositionEncoding"]) -> torch.Tensor:
+        """h [rows, hidden] (activation dtype) -> what is added to the residual stream."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: StepContext,
+                row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Add `delta` to the float32 residual rows `x` (in place unless `row_idx`
+        picks rows) and return the normed rows in the activation dtype."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def on_embedding(self, x: torch.Tensor, ctx: StepContext) -> None:
+        """Hook for encodings that act on the embedded rows (in place)."""
+
+    def on_qkv(self, qkv: torch.Tensor, ctx: StepContext, nh: int, nkv: int, hd: int,
+               kcache, vcache, group) -> None:
+        """Encode q and k of packed rows in place and store k, v in the cache (if given)."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
+                 feed_forward_norm: Norm, position: Optional[PositionEncoding]):
+        super().__init__()
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+        self.position = position
+
+    def parts(self) -> List[Part]:
+        ps = [self.mixer, self.feed_forward, self.mixer_norm, self.feed_forward_norm]
+        return ps + ([self.position] if self.position is not None else [])
+
+    def wants(self) -> Dict[str, TensorWant]:
+        out: Dict[str, TensorWant] = {}
+        for p in self.parts():
+            out.update(p.wants())
+        return out
+
+    def load(self, tensors) -> None:
+        for p in self.parts():
+            p.load(tensors)
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
+                line: int, writes_cache: bool) -> Optional[torch.Tensor]:
+        """x: float32 residual rows, updated in place; `pending` is what the previous
+        block still has to add.  Returns what this block leaves to be added."""
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        """float32 residual rows [rows, hidden] for ctx.tokens."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        """Normed rows -> float32 logits [rows, vocab]."""
+        raise NotImplementedError
+
+
+# ---------------------------------------------------------------- registries
+_KINDS = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+_REGISTRY: Dict[str, Dict[str, type]] = {k: {} for k in _KINDS}
+
+
+def register_part(kind: str, name: str) -> Callable[[type], type]:
+    """Class decorator: `@register_part("mixer", "attention")`."""
+    if kind not in _REGISTRY:
+        raise KeyError(f"unknown kind of part {kind!r}; kinds: {_KINDS}")
+
+    def deco(cls: type) -> type:
+        _REGISTRY[kind][name] = cls
+        return cls
+    return deco
+
+
+def part_class(kind: str, name: str) -> type:
+    try:
+        return _REGISTRY[kind][name]
+    except KeyError:
+        raise KeyError(f"no {kind} named {name!r}; registered: {sorted(_REGISTRY[kind])}") from None
+
+
+def build_part(kind: str, spec) -> Part:
+    """A part from a `PartSpec` (registry name, parameters, tensor names)."""
+    return part_class(kind, spec.kind)(tensors=spec.tensors, **spec.params)

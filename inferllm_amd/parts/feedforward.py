@@ -1,0 +1,39 @@
+"""Feed-forward parts."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import TensorWant
+from .attention import _fuse
+from .base import FeedForward, StepContext, register_part
+
+
+@register_part("feed_forward", "swiglu")
+class SwiGLU(FeedForward):
+    """down( silu(h gate^T) * (h up^T) ), gate and up as one fused product.
+
+    src/core/graph.cpp:57-79 (w1 = gate, w3 = up, w2 = down); silu(x) = x / (1 + exp(-x))
+    (src/kern/naive/naive.cpp:80-89).  The reference runs silu and the multiply as two
+    elementwise kernels (src/kern/gpu/kernel_gpu.cu:183-258).
+    """
+
+    def __init__(self, hidden_size: int, intermediate_size: int, tensors=None):
+        super().__init__(tensors)
+        self.E, self.F = int(hidden_size), int(intermediate_size)
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def shapes(self) -> Dict[str, TensorWant]:
+        return {"gate": TensorWant((self.F, self.E)), "up": TensorWant((self.F, self.E)),
+                "down": TensorWant((self.E, self.F))}
+
+    def load(self, tensors) -> None:
+        self.w_gate_up = _fuse([self._take(tensors, "gate"), self._take(tensors, "up")])
+        self.w_down = self._take(tensors, "down").contiguous()
+
+    def forward(self, h, ctx: StepContext):
+        gu = ops.linear(h, self.w_gate_up)
+        return ops.linear(ops.silu_mul(gu), self.w_down)

@@ -1,0 +1,192 @@
+"""Plain torch versions of every kernel's contract (float64 inside).
+
+Two uses: the expected side of each kernel's own test on the GPU, and, patched
+over `inferllm_amd.kernels.ops` on the CPU, a stand-in that lets the step
+function, the cache and the generation loop run without a GPU so that their
+bookkeeping is tested where there is none.  They share no code with the kernels.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+F64 = torch.float64
+
+
+def embed(tokens, table):
+    return table[tokens.long()].to(torch.float32)
+
+
+def add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx=None):
+    if delta is not None:
+        s = (x.to(F64) + delta.to(F64)).to(torch.float32)
+        if row_idx is None:
+            x.copy_(s)
+    else:
+        s = x
+    if row_idx is not None:
+        s = s[row_idx.long()]
+    v = s.to(F64)
+    scale = 1.0 / torch.sqrt((v * v).mean(dim=-1, keepdim=True) + eps)
+    return ((v * scale) * weight.to(F64)).to(out_dtype)
+
+
+def silu_mul(gate_up):
+    F = gate_up.shape[1] // 2
+    g, u = gate_up[:, :F].to(F64), gate_up[:, F:].to(F64)
+    return (g / (1.0 + torch.exp(-g)) * u).to(gate_up.dtype)
+
+
+def cache_offsets(page_table, slot, pos, page_size, ring):
+    lp = pos // page_size
+    if ring > 0:
+        lp = lp % ring
+    return int(page_table[slot, lp]), pos % page_size
+
+
+def rope_store(qkv, cos_sin, rot, pairing, row_pos, row_slot, slot_len, kcache, vcache,
+               page_table, page_size, ring, nh, nkv, hd):
+    T = qkv.shape[0]
+    view = qkv.view(T, nh + 2 * nkv, hd)
+    if cos_sin is not None:
+        heads = view[:, : nh + nkv, :].to(F64)
+        cs = cos_sin[row_pos.long()].to(F64)          # [T, rot/2, 2]
+        c, s = cs[:, None, :, 0], cs[:, None, :, 1]
+        half = rot // 2
+        if pairing == 0:
+            a = heads[:, :, :half].clone()
+            b = heads[:, :, hd // 2: hd // 2 + half].clone()
+            heads[:, :, :half] = a * c - b * s
+            heads[:, :, hd // 2: hd // 2 + half] = a * s + b * c
+        else:
+            a = heads[:, :, 0:rot:2].clone()
+            b = heads[:, :, 1:rot:2].clone()
+            heads[:, :, 0:rot:2] = a * c - b * s
+            heads[:, :, 1:rot:2] = a * s + b * c
+        view[:, : nh + nkv, :] = heads.to(qkv.dtype)
+    if kcache is None:
+        return
+    for t in range(T):
+        slot, pos = int(row_slot[t]), int(row_pos[t])
+        if ring > 0:
+            last_page = (int(slot_len[slot]) - 1) // page_size
+            if pos // page_size + ring <= last_page:
+                continue
+        page, r = cache_offsets(page_table, slot, pos, page_size, ring)
+        kcache[page, :, r, :] = view[t, nh: nh + nkv, :]
+        vcache[page, :, r, :] = view[t, nh + nkv:, :]
+
+
+def linear(x, w, out_dtype=None):
+    return (x.to(F64) @ w.to(F64).t()).to(out_dtype or x.dtype)
+
+
+def gemm_generic(x, w, out_dtype):
+    return linear(x, w, out_dtype)
+
+
+def _attend(q, k, v, scale, visible):
+    """q [nh, hd], k/v [L, nkv, hd], visible: bool [L]."""
+    nh, nkv = q.shape[0], k.shape[1]
+    per = nh // nkv
+    out = torch.zeros(nh, q.shape[1], dtype=F64)
+    for h in range(nh):
+        s = (k[:, h // per, :].to(F64) @ q[h].to(F64)) * scale
+        s = s.masked_fill(~visible, -math.inf)
+        p = torch.softmax(s, dim=0)
+        out[h] = p @ v[:, h // per, :].to(F64)
+    return out
+
+
+def attn_prefill(qkv, cu_seqlens, n_seqs, max_len, nh, nkv, hd, scale, window):
+    T = qkv.shape[0]
+    view = qkv.view(T, nh + 2 * nkv, hd)
+    out = torch.zeros(T, nh * hd, dtype=qkv.dtype, device=qkv.device)
+    for b in range(n_seqs):
+        s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
+        k, v = view[s0:s1, nh: nh + nkv], view[s0:s1, nh + nkv:]
+        idx = torch.arange(s1 - s0)
+        for a in range(s1 - s0):
+            vis = idx <= a
+            if window and window > 0:
+                vis = vis & (idx > a - window)
+            out[s0 + a] = _attend(view[s0 + a, :nh], k, v, scale, vis).reshape(-1).to(qkv.dtype)
+    return out
+
+
+def decode_splits(B, nh, max_len):
+    return 2
+
+
+def attn_decode(qkv, kcache, vcache, page_table, page_size, ring, seq_slot, slot_len, nh, nkv, hd,
+                scale, window, nsplit):
+    B = qkv.shape[0]
+    view = qkv.view(B, nh + 2 * nkv, hd)
+    out = torch.zeros(B, nh * hd, dtype=qkv.dtype, device=qkv.device)
+    for b in range(B):
+        slot = int(seq_slot[b])
+        n = int(slot_len[slot])
+        first = max(0, n - window) if window and window > 0 else 0
+        ks, vs = [], []
+        for pos in range(first, n):
+            page, r = cache_offsets(page_table, slot, pos, page_size, ring)
+            ks.append(kcache[page, :, r, :])
+            vs.append(vcache[page, :, r, :])
+        if not ks:
+            continue
+        k, v = torch.stack(ks), torch.stack(vs)
+        vis = torch.ones(k.shape[0], dtype=torch.bool)
+        out[b] = _attend(view[b, :nh], k, v, scale, vis).reshape(-1).to(qkv.dtype)
+    return out
+
+
+def argmax(logits):
+    return torch.argmax(logits, dim=-1).to(torch.int32)   # first index on ties
+
+
+def kept_distribution(logits_row, temperature, top_k, top_p, repeat_penalty, last_tokens):
+    """ids kept by the sampler and their probabilities (float64), in descending order."""
+    V = logits_row.numel()
+    s = logits_row.to(F64) / temperature
+    if last_tokens is not None:
+        for t in set(int(x) for x in last_tokens if int(x) >= 0):
+            s[t] = s[t] * repeat_penalty if float(logits_row[t]) < 0 else s[t] / repeat_penalty
+    order = sorted(range(V), key=lambda i: (-float(s[i]), i))
+    if 0 < top_k < V:
+        order = order[:top_k]
+    sc = torch.tensor([float(s[i]) for i in order], dtype=F64)
+    p = torch.exp(sc - sc.max())
+    p = p / p.sum()
+    if top_p < 1.0:
+        cum = torch.cumsum(p, 0)
+        n = int((cum >= top_p).nonzero()[0]) + 1 if bool((cum >= top_p).any()) else len(order)
+        order, p = order[:n], p[:n] / p[:n].sum()
+    return order, p
+
+
+def sample(logits, temperature, top_k, top_p, repeat_penalty, last_tokens, seeds, counters):
+    from inferllm_amd.sampling.params import uniform
+    out = []
+    for b in range(logits.shape[0]):
+        ids, p = kept_distribution(logits[b], temperature, top_k, top_p, repeat_penalty,
+                                   last_tokens[b] if last_tokens is not None else None)
+        pairs = sorted(zip(ids, p.tolist()))              # inverse CDF in ascending id order
+        u = uniform(int(seeds[b]) & ((1 << 64) - 1), int(counters[b]))
+        cum, pick = 0.0, pairs[-1][0]
+        for i, pi in pairs:
+            cum += pi
+            if u < cum:
+                pick = i
+                break
+        out.append(pick)
+    return torch.tensor(out, dtype=torch.int32)
+
+
+def patch(monkeypatch):
+    """Put these functions in place of the GPU ops (CPU tests only)."""
+    from inferllm_amd.kernels import ops
+    for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic",
+                 "attn_prefill", "decode_splits", "attn_decode", "argmax", "sample"):
+        monkeypatch.setattr(ops, name, globals()[name])

@@ -1,0 +1,54 @@
+"""Tiny configurations and helpers shared by the tests.
+
+A and B are the two tiny LLaMA shapes of the build's baseline; C adds what those
+two share (another head count, tied embeddings, a head size in steps of 16 with
+8-fold groups).  They differ in every size and constant.
+"""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+
+TINY_A = {"architectures": ["LlamaForCausalLM"], "hidden_size": 64, "intermediate_size": 172,
+          "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 4,
+          "vocab_size": 256, "rms_norm_eps": 1e-6, "rope_theta": 10000.0,
+          "max_position_embeddings": 128, "tie_word_embeddings": False,
+          "bos_token_id": 1, "eos_token_id": 2}
+TINY_B = {"architectures": ["LlamaForCausalLM"], "hidden_size": 96, "intermediate_size": 256,
+          "num_hidden_layers": 3, "num_attention_heads": 4, "num_key_value_heads": 2,
+          "head_dim": 24, "vocab_size": 320, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+          "max_position_embeddings": 256, "tie_word_embeddings": False,
+          "bos_token_id": 1, "eos_token_id": [2, 3]}
+TINY_C = {"architectures": ["LlamaForCausalLM"], "hidden_size": 80, "intermediate_size": 200,
+          "num_hidden_layers": 1, "num_attention_heads": 8, "num_key_value_heads": 1,
+          "head_dim": 32, "vocab_size": 411, "rms_norm_eps": 3e-5, "rope_theta": 25000.0,
+          "max_position_embeddings": 512, "tie_word_embeddings": True,
+          "bos_token_id": 0, "eos_token_id": 5}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+
+def make_model_dir(tmp_path, config: dict, seed: int, dtype=torch.float32) -> str:
+    """Write a random model folder for `config` under tmp_path; returns the folder."""
+    import inferllm_amd as I
+    d = os.path.join(str(tmp_path), f"model_{abs(hash(json.dumps(config, sort_keys=True))) % 10**8}_{seed}_{str(dtype)[6:]}")
+    if not os.path.isdir(d):
+        I.write_random_model(d, I.config_from_dict(config), seed=seed, dtype=dtype)
+    return d
+
+
+def read_weights(model_dir: str):
+    """All tensors of a model folder as float tensors on the CPU (for the plain model)."""
+    from inferllm_amd.weights import open_model_files
+    out = {}
+    for f in open_model_files(model_dir):
+        for n in f.names():
+            out[n] = f.read(n)
+        f.close()
+    return out
+
+
+def random_ids(n: int, vocab: int, seed: int):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
