@@ -1,0 +1,285 @@
+"""Each HIP kernel alone against its plain torch contract (tests/kernel_refs.py),
+at sizes other than the engine's tiny models: widths and vocabularies that are no
+power of two, head sizes in steps of 16 (and 24), odd head and group counts.
+Shapes include those of the reference's own op tests (test/GPU/test_opr.cpp:9-119)."""
+import math
+
+import pytest
+import torch
+
+import kernel_refs as R
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def ops():
+    from inferllm_amd.kernels import ops as o
+    return o
+
+
+def tol(dtype):
+    return (2e-5, 2e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+
+
+def close(got, want, dtype, scale=1.0):
+    a, r = tol(dtype)
+    assert got.shape == want.shape
+    torch.testing.assert_close(got.double().cpu(), want.double().cpu(), atol=a * scale, rtol=r)
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,E,ids", [(10, 128, [1, 9, 3, 3]), (411, 80, [0, 410, 7]), (1000, 4100, [999])])
+def test_embed(dtype, V, E, ids):
+    table = rnd(V, E, dtype=dtype)
+    t = torch.tensor(ids, dtype=torch.int32)
+    got = ops().embed(t.to(DEV), table.to(DEV))
+    assert torch.equal(got.cpu(), R.embed(t, table))       # rows are copied bit for bit
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("T,E,eps", [(4, 4096, 1e-5), (3, 80, 1e-6), (1, 1001, 3e-2), (70, 96, 1e-5)])
+def test_add_rmsnorm(out_dtype, w_dtype, T, E, eps):
+    x = rnd(T, E, seed=1) * 0.05            # small rows: eps matters
+    w = (1 + rnd(E, seed=2) * 0.1).to(w_dtype)
+    for delta_dtype in (None, torch.float32, torch.bfloat16):
+        delta = None if delta_dtype is None else rnd(T, E, seed=3, std=0.05).to(delta_dtype)
+        xr, xg = x.clone(), x.clone().to(DEV)
+        want = R.add_rmsnorm(xr, delta, w, eps, out_dtype)
+        got = ops().add_rmsnorm(xg, None if delta is None else delta.to(DEV), w.to(DEV), eps, out_dtype)
+        close(got, want, out_dtype)
+        close(xg, xr, torch.float32)          # the sum is written back
+        if T > 2:
+            idx = torch.tensor([T - 1, 0], dtype=torch.int32)
+            xr2, xg2 = x.clone(), x.clone().to(DEV)
+            want = R.add_rmsnorm(xr2, delta, w, eps, out_dtype, idx)
+            got = ops().add_rmsnorm(xg2, None if delta is None else delta.to(DEV), w.to(DEV), eps,
+                                    out_dtype, idx.to(DEV))
+            close(got, want, out_dtype)
+            assert torch.equal(xg2.cpu(), x)   # gathered rows leave x alone
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,F", [(4, 10), (5, 130), (3, 11008), (1, 173)])
+def test_silu_mul(dtype, T, F):
+    gu = rnd(T, 2 * F, dtype=dtype, std=3.0)
+    gu[0, 0] = 0.0; gu[0, 1] = -60.0; gu[0, 2] = 40.0
+    close(ops().silu_mul(gu.to(DEV)), R.silu_mul(gu), dtype, scale=10)
+
+
+def make_cache(n_pages, nkv, page, hd, dtype):
+    return (torch.full((n_pages, nkv, page, hd), float("nan"), dtype=dtype),
+            torch.full((n_pages, nkv, page, hd), float("nan"), dtype=dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,rot,pairing", [(4, 2, 24, 24, 0), (3, 3, 16, 16, 1), (8, 1, 128, 128, 0),
+                                                    (5, 5, 48, 32, 0), (2, 1, 256, 256, 1)])
+def test_rope_store(dtype, nh, nkv, hd, rot, pairing):
+    from inferllm_amd.parts.position import rotary_table
+    page, max_pos = 8, 64
+    table = rotary_table(12345.0, rot, max_pos, "cpu")
+    lens = [13, 1, 20]
+    slots = [2, 0, 3]
+    pos = [p for n in lens for p in range(n)]
+    slot = [s for n, s in zip(lens, slots) for _ in range(n)]
+    T = len(pos)
+    qkv = rnd(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=5)
+    pt = torch.full((5, 4), 11, dtype=torch.int32)
+    pt[2, :2] = torch.tensor([7, 3]); pt[0, :1] = 9; pt[3, :3] = torch.tensor([0, 5, 1])
+    slot_len = torch.tensor([1, 0, 13, 20, 0], dtype=torch.int32)
+    kc, vc = make_cache(12, nkv, page, hd, dtype)
+    rp, rs = torch.tensor(pos, dtype=torch.int32), torch.tensor(slot, dtype=torch.int32)
+    q_ref, kc_ref, vc_ref = qkv.clone(), kc.clone(), vc.clone()
+    R.rope_store(q_ref, table, rot, pairing, rp, rs, slot_len, kc_ref, vc_ref, pt, page, 0, nh, nkv, hd)
+    q_g, kc_g, vc_g = qkv.to(DEV), kc.to(DEV), vc.to(DEV)
+    ops().rope_store(q_g, table.to(DEV), rot, pairing, rp.to(DEV), rs.to(DEV), slot_len.to(DEV),
+                     kc_g, vc_g, pt.to(DEV), page, 0, nh, nkv, hd)
+    close(q_g, q_ref, dtype, scale=4)
+    for got, want in ((kc_g, kc_ref), (vc_g, vc_ref)):
+        got, want = got.cpu(), want
+        assert torch.equal(torch.isnan(got), torch.isnan(want))      # exactly the same rows are written
+        close(torch.nan_to_num(got), torch.nan_to_num(want), dtype, scale=4)
+    # position 0 leaves the row as it is
+    first = [0, 13, 14]
+    assert torch.equal(q_g.cpu()[first], qkv[first])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_store_window_ring(dtype):
+    """A ring of pages: rows that a later row of the same step overwrites are skipped."""
+    nh, nkv, hd, page, ring = 2, 2, 16, 4, 3
+    n = 23
+    qkv = rnd(n, (nh + 2 * nkv) * hd, dtype=dtype, seed=9)
+    pt = torch.tensor([[4, 2, 6]], dtype=torch.int32)
+    slot_len = torch.tensor([n], dtype=torch.int32)
+    rp = torch.arange(n, dtype=torch.int32); rs = torch.zeros(n, dtype=torch.int32)
+    kc, vc = make_cache(8, nkv, page, hd, dtype)
+    kr, vr = kc.clone(), vc.clone()
+    R.rope_store(qkv.clone(), None, 0, 0, rp, rs, slot_len, kr, vr, pt, page, ring, nh, nkv, hd)
+    kg, vg = kc.to(DEV), vc.to(DEV)
+    ops().rope_store(qkv.to(DEV), None, 0, 0, rp.to(DEV), rs.to(DEV), slot_len.to(DEV), kg, vg,
+                     pt.to(DEV), page, ring, nh, nkv, hd)
+    assert torch.equal(torch.nan_to_num(kg.cpu()), torch.nan_to_num(kr))
+    assert torch.equal(torch.nan_to_num(vg.cpu()), torch.nan_to_num(vr))
+    # the last ring*page - (page - 1 - (n-1) % page) positions are there, e.g. position n-1
+    view = qkv.view(n, nh + 2 * nkv, hd)
+    assert torch.equal(kg.cpu()[int(pt[0, ((n - 1) // page) % ring]), :, (n - 1) % page], view[n - 1, nh:nh + nkv])
+
+
+@pytest.mark.parametrize("xd,wd,yd", [(torch.float32,) * 3, (torch.bfloat16,) * 3,
+                                      (torch.bfloat16, torch.bfloat16, torch.float32),
+                                      (torch.bfloat16, torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("M,N,K", [(1, 2, 128), (4, 128, 128), (70, 411, 80), (65, 64, 1001), (3, 1000, 172)])
+def test_gemm_generic(xd, wd, yd, M, N, K):
+    x, w = rnd(M, K, dtype=xd, seed=1), rnd(N, K, dtype=wd, seed=2)
+    got = ops().gemm_generic(x.to(DEV), w.to(DEV), yd)
+    close(got, R.linear(x, w, yd), yd, scale=math.sqrt(K))
+
+
+def test_gemm_generic_row_bits_do_not_depend_on_batch():
+    x, w = rnd(70, 300, seed=1), rnd(130, 300, seed=2)
+    whole = ops().gemm_generic(x.to(DEV), w.to(DEV), torch.float32).cpu()
+    for r in (0, 17, 69):
+        alone = ops().gemm_generic(x[r:r + 1].to(DEV), w.to(DEV), torch.float32).cpu()
+        assert torch.equal(alone[0], whole[r])
+
+
+def test_gemm_identity_and_linearity():
+    x = rnd(5, 96, seed=3)
+    eye = torch.eye(96)
+    assert torch.equal(ops().gemm_generic(x.to(DEV), eye.to(DEV), torch.float32).cpu(), x)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,lens,window", [
+    (4, 4, 16, [7], 0), (4, 2, 24, [5, 11, 2], 0), (16, 16, 8, [2], 0), (32, 2, 128, [5, 70], 0),
+    (3, 1, 48, [33, 64, 1, 100], 0), (2, 2, 256, [40], 0), (4, 2, 32, [90, 17], 13), (5, 5, 16, [130], 64)])
+def test_attn_prefill(dtype, nh, nkv, hd, lens, window):
+    T = sum(lens)
+    qkv = rnd(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=7)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    scale = 1.0 / math.sqrt(hd)
+    got = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), len(lens), max(lens), nh, nkv, hd, scale, window)
+    want = R.attn_prefill(qkv, cu, len(lens), max(lens), nh, nkv, hd, scale, window)
+    close(got, want, dtype, scale=2)
+
+
+def paged_case(dtype, nkv, hd, lens, page, ring=0, seed=3):
+    """Random cache contents laid out through a shuffled page table."""
+    B = len(lens)
+    per_seq = max((n + page - 1) // page for n in lens) if not ring else ring
+    n_pages = B * per_seq + 3
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_pages - 1, generator=g)[: B * per_seq].reshape(B, per_seq)
+    pt = torch.full((B + 2, per_seq), n_pages - 1, dtype=torch.int32)
+    slots = list(range(B, 0, -1))                    # slot numbers differ from batch order
+    for b, s in enumerate(slots):
+        pt[s] = perm[b].to(torch.int32)
+    kc, vc = rnd(n_pages, nkv, page, hd, dtype=dtype, seed=seed + 1), rnd(n_pages, nkv, page, hd, dtype=dtype, seed=seed + 2)
+    slot_len = torch.zeros(B + 2, dtype=torch.int32)
+    for b, s in enumerate(slots):
+        slot_len[s] = lens[b]
+    return pt, kc, vc, torch.tensor(slots, dtype=torch.int32), slot_len
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,lens,window,nsplit", [
+    (4, 4, 16, [7], 0, 1), (4, 2, 24, [5, 11, 2], 0, 2), (32, 2, 128, [300, 70], 0, 3),
+    (3, 1, 48, [33, 64, 1, 600], 0, 4), (2, 2, 256, [257], 0, 2), (4, 2, 32, [90, 17, 700], 13, 2),
+    (5, 5, 16, [130, 520], 64, 5)])
+def test_attn_decode(dtype, nh, nkv, hd, lens, window, nsplit):
+    page = 16
+    ring = 0
+    if window:
+        ring = (window + page - 2) // page + 1
+    pt, kc, vc, slots, slot_len = paged_case(dtype, nkv, hd, lens, page, ring)
+    B = len(lens)
+    qkv = rnd(B, (nh + 2 * nkv) * hd, dtype=dtype, seed=11)
+    scale = 1.0 / math.sqrt(hd)
+    got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring, slots.to(DEV),
+                            slot_len.to(DEV), nh, nkv, hd, scale, window, nsplit)
+    want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, slot_len, nh, nkv, hd, scale, window, nsplit)
+    close(got, want, dtype, scale=2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_decode_finds_one_far_key(dtype):
+    """One key among hundreds is made to stand out: the output must be its value."""
+    nh, nkv, hd, page, n = 4, 2, 32, 16, 777
+    pt, kc, vc, slots, slot_len = paged_case(dtype, nkv, hd, [n], page)
+    qkv = rnd(1, (nh + 2 * nkv) * hd, dtype=dtype, seed=1)
+    target = 5
+    pg, r = R.cache_offsets(pt, int(slots[0]), target, page, 0)
+    q = qkv.view(1, nh + 2 * nkv, hd)
+    for kvh in range(nkv):
+        kc[pg, kvh, r] = q[0, kvh * (nh // nkv)].float().mul(40).to(dtype)   # huge score for head kvh*per
+    got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, 0, slots.to(DEV),
+                            slot_len.to(DEV), nh, nkv, hd, 1.0, 0, 4).cpu().view(nh, hd)
+    for kvh in range(nkv):
+        close(got[kvh * (nh // nkv)], vc[pg, kvh, r], dtype)
+
+
+@pytest.mark.parametrize("B,V", [(1, 256), (3, 320), (2, 32000), (64, 411), (1, 128256)])
+def test_argmax(B, V):
+    logits = rnd(B, V, seed=4)
+    logits[0, V - 1] = 50.0
+    if B > 1:
+        logits[1, 3] = 60.0; logits[1, 200] = 60.0           # a tie: the lower id wins
+    got = ops().argmax(logits.to(DEV)).cpu()
+    assert got.tolist() == R.argmax(logits).tolist()
+    assert got[0] == V - 1 and (B == 1 or got[1] == 3)
+
+
+def interval_ok(logits_row, token, u, temperature, top_k, top_p, penalty, last):
+    """The drawn token's interval of the id-ordered CDF over the kept ids contains u (with slack)."""
+    ids, p = R.kept_distribution(logits_row, temperature, top_k, top_p, penalty, last)
+    pairs = sorted(zip(ids, p.tolist()))
+    cum = 0.0
+    for i, pi in pairs:
+        if i == token:
+            return cum - 1e-4 <= u <= cum + pi + 1e-4
+        cum += pi
+    return False
+
+
+@pytest.mark.parametrize("V,temperature,top_k,top_p,penalty", [
+    (256, 0.8, 0, 1.0, 1.0), (320, 0.8, 40, 0.95, 1.1), (411, 0.1, 40, 0.95, 1.3), (1000, 1.5, 5, 1.0, 1.0),
+    (32000, 1.0, 0, 0.9, 1.0), (300, 0.7, 1, 1.0, 1.0), (128256, 0.9, 50, 0.8, 1.2)])
+def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top_p, penalty):
+    from inferllm_amd.sampling.params import uniform
+    B = 6
+    logits = rnd(B, V, seed=8, std=2.0)
+    logits[2] = 0.0                                            # all equal: ties everywhere
+    last = torch.full((B, 8), -1, dtype=torch.int32)
+    last[:, :3] = torch.tensor([1, 5, V - 1], dtype=torch.int32)
+    seeds = torch.tensor([3, 99, 12345, -7, 2**62, 0], dtype=torch.int64)
+    counters = torch.tensor([0, 1, 2, 3, 4, 5], dtype=torch.int32)
+    got = ops().sample(logits.to(DEV), temperature, top_k, top_p, penalty,
+                       last.to(DEV) if penalty != 1.0 else None, seeds.to(DEV), counters.to(DEV)).cpu().tolist()
+    for b in range(B):
+        u = uniform(int(seeds[b]) & ((1 << 64) - 1), int(counters[b]))
+        assert interval_ok(logits[b], got[b], u, temperature, top_k, top_p, penalty,
+                           last[b] if penalty != 1.0 else None), (b, got[b], u)
+    if top_k == 1:
+        assert got == torch.argmax(logits, -1).tolist() or penalty != 1.0
+
+
+def test_sample_frequencies_match_probabilities():
+    V, n = 7, 4000
+    row = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, 1.5, -3.0])
+    logits = row.repeat(n, 1)
+    seeds = torch.arange(n, dtype=torch.int64) * 7919 + 1
+    counters = torch.zeros(n, dtype=torch.int32)
+    got = ops().sample(logits.to(DEV), 0.9, 0, 1.0, 1.0, None, seeds.to(DEV), counters.to(DEV)).cpu()
+    freq = torch.bincount(got.long(), minlength=V).double() / n
+    p = torch.softmax(row.double() / 0.9, 0)
+    chi2 = float((n * (freq - p) ** 2 / p).sum())
+    assert chi2 < 30.0, (chi2, freq, p)           # 6 degrees of freedom: far beyond any honest draw

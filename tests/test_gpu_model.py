@@ -1,0 +1,188 @@
+"""The engine on the GPU against the plain implementation (tests/plain_llama.py),
+in float32 and in bfloat16: whole requests, the last 32 tokens one by one, batches
+of unequal lengths with slots used again, long decoding, the first tokens of a
+sequence, greedy generation through the entry point."""
+import math
+
+import pytest
+import torch
+
+import plain_llama
+from tiny import CONFIGS, make_model_dir, random_ids, read_weights
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+# Largest |engine - plain| over a request, divided by the largest |plain logit| of it.
+# float32: rounding of sums of a few hundred float32 terms.  bfloat16: activations carry
+# 8 bits (2^-8 = 0.4 %) and pass through up to 3 blocks and the head.
+BUDGET = {"float32": 2e-5, "bfloat16": 3e-2}
+STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+_cache = {}
+
+
+def setup(tmp_path_factory, name, dtype, **kw):
+    """(engine, plain logits function) for a tiny configuration; folders are per session."""
+    import inferllm_amd as I
+    config = CONFIGS[name]
+    key = (name, dtype)
+    if key not in _cache:
+        d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=7, dtype=STORE[dtype])
+        _cache[key] = (d, read_weights(d))
+    d, w = _cache[key]
+    kw.setdefault("max_batch", 4)
+    eng = I.Engine.from_pretrained(d, dtype=dtype, device=DEV, poison_freed=True, **kw)
+    return eng, (lambda ids: plain_llama.forward_logits(config, w, ids)), config
+
+
+def err(got, want):
+    return float((got.double().cpu() - want).abs().max() / want.abs().max())
+
+
+def requests_for(config, lens, seed=0):
+    return [random_ids(n, config["vocab_size"], seed + 31 * i + n) for i, n in enumerate(lens)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_requests(tmp_path_factory, name, dtype):
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, name, dtype)
+    for ids in requests_for(config, [7, 1, 2, 100, 65]):
+        s = eng.alloc_slot()
+        got = eng.step([StepEntry(s, ids, list(range(len(ids))))])
+        assert err(got, plain(ids)) < BUDGET[dtype]
+        eng.free_slot(s)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_32_tokens_one_by_one(tmp_path_factory, name, dtype):
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, name, dtype)
+    for ids in requests_for(config, [33, 100, 128], seed=5):
+        want = plain(ids)
+        s = eng.alloc_slot()
+        head = len(ids) - 32
+        got = [eng.step([StepEntry(s, ids[:head], list(range(head)))]).clone()]
+        for t in ids[head:]:
+            got.append(eng.step([StepEntry(s, [t], [0])]).clone())
+        got = torch.cat(got)
+        per_pos = (got.double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+        assert float(per_pos.max()) < BUDGET[dtype], f"first bad position {int((per_pos >= BUDGET[dtype]).nonzero()[0])}"
+        eng.free_slot(s)
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_unequal_batches_with_slot_reuse(tmp_path_factory, name, dtype, graphs):
+    """Batches of three requests of unequal lengths, one batch after another in two
+    slots' worth of spare room; shorter requests end earlier; every position's
+    logits equal the plain model's."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, name, dtype, max_batch=3, max_tokens=64 * 5,
+                               use_graphs=graphs)
+    reqs = requests_for(config, [70, 9, 40, 3, 66, 12, 5, 90, 33], seed=9)
+    want = [plain(r) for r in reqs]
+    prompt = [max(1, len(r) - 6 - i) for i, r in enumerate(reqs)]
+    for b0 in range(0, len(reqs), 3):
+        batch = list(range(b0, b0 + 3))
+        slot = {i: eng.alloc_slot() for i in batch}
+        got = {i: [] for i in batch}
+        out = eng.step([StepEntry(slot[i], reqs[i][:prompt[i]], list(range(prompt[i]))) for i in batch])
+        o = 0
+        for i in batch:
+            got[i].append(out[o:o + prompt[i]].clone()); o += prompt[i]
+        at = dict((i, prompt[i]) for i in batch)
+        live = [i for i in batch if at[i] < len(reqs[i])]
+        for i in batch:
+            if i not in live:
+                eng.free_slot(slot[i])
+        while live:
+            out = eng.step([StepEntry(slot[i], [reqs[i][at[i]]], [0]) for i in live])
+            for j, i in enumerate(live):
+                got[i].append(out[j:j + 1].clone()); at[i] += 1
+            for i in [i for i in live if at[i] == len(reqs[i])]:
+                eng.free_slot(slot[i])
+            live = [i for i in live if at[i] < len(reqs[i])]
+        for i in batch:
+            assert err(torch.cat(got[i]), want[i]) < BUDGET[dtype], f"request {i}"
+        eng.cache.check()
+        assert eng.cache.slots.n_held() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(tmp_path_factory, dtype):
+    """Decode 250 tokens one by one after a 3-token prompt (crossing several pages)."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "B", dtype)
+    ids = requests_for(config, [253], seed=2)[0]
+    want = plain(ids)
+    s = eng.alloc_slot()
+    got = [eng.step([StepEntry(s, ids[:3], [0, 1, 2])]).clone()]
+    for t in ids[3:]:
+        got.append(eng.step([StepEntry(s, [t], [0])]).clone())
+    per_pos = (torch.cat(got).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+    assert float(per_pos.max()) < BUDGET[dtype], f"first bad position {int((per_pos >= BUDGET[dtype]).nonzero()[0])}"
+    eng.free_slot(s)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(tmp_path_factory, dtype):
+    """A one-token prompt, then tokens one by one from position 1 on."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "A", dtype)
+    ids = requests_for(config, [6], seed=4)[0]
+    want = plain(ids)
+    s = eng.alloc_slot()
+    got = [eng.step([StepEntry(s, [t], [0])]).clone() for t in ids]
+    assert err(torch.cat(got), want) < BUDGET[dtype]
+    eng.free_slot(s)
+
+
+def test_padding_and_batch_company_change_nothing_float32(tmp_path_factory):
+    """The same request alone and among others: float32 logits agree to rounding."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "B", "float32", max_batch=4)
+    reqs = requests_for(config, [40, 7, 19], seed=6)
+    s = eng.alloc_slot()
+    alone = eng.step([StepEntry(s, reqs[0], [len(reqs[0]) - 1])]).clone()
+    eng.free_slot(s)
+    slots = [eng.alloc_slot() for _ in reqs]
+    out = eng.step([StepEntry(sl, r, [len(r) - 1]) for sl, r in zip(reversed(slots), reqs)])
+    assert float((out[0] - alone[0]).abs().max()) < 1e-6
+    for sl in slots:
+        eng.free_slot(sl)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_equals_plain(tmp_path_factory, name):
+    import inferllm_amd as I
+    config = CONFIGS[name]
+    eng, plain, _ = setup(tmp_path_factory, name, "float32", max_batch=2)
+    _, w = _cache[(name, "float32")]
+    prompts = requests_for(config, [7, 11, 2, 5, 30], seed=8)
+    n_new = 9 if name == "A" else 6
+    got = eng.generate(prompts, max_new_tokens=n_new, stop_token_ids=[])
+    want = [plain_llama.generate_greedy(config, w, p, n_new) for p in prompts]
+    assert got == want
+    # a stop token ends its sequence early and is left out
+    stop = want[1][2]
+    got = eng.generate(prompts[:3], max_new_tokens=n_new, stop_token_ids=[stop])
+    assert got == [plain_llama.generate_greedy(config, w, p, n_new, [stop]) for p in prompts[:3]]
+    eng.cache.check()
+    assert eng.cache.slots.n_held() == 0
+
+
+def test_temperature_sampling_is_reproducible_and_batch_independent(tmp_path_factory):
+    eng, plain, config = setup(tmp_path_factory, "B", "float32", max_batch=3)
+    prompts = requests_for(config, [5, 11, 2], seed=1)
+    a = eng.generate(prompts, temperature=0.8, seed=42, max_new_tokens=6, stop_token_ids=[])
+    b = eng.generate(prompts, temperature=0.8, seed=42, max_new_tokens=6, stop_token_ids=[])
+    c = eng.generate(prompts, temperature=0.8, seed=43, max_new_tokens=6, stop_token_ids=[])
+    assert a == b and a != c
+    eng1, _, _ = setup(tmp_path_factory, "B", "float32", max_batch=1)     # one at a time
+    assert eng1.generate(prompts, temperature=0.8, seed=42, max_new_tokens=6, stop_token_ids=[]) == a
