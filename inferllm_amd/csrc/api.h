@@ -52,6 +52,19 @@ int illm_attn_decode_generic(const void* qkv, void* out, int dt, const void* kca
                              const int32_t* slot_len, float* partial, int nsplit, int B, int nh,
                              int nkv, int hd, float scale, int window, void* stream);
 
+// The same for bfloat16 with head_dim % 8 == 0 and page_size % 64 == 0 (anything else:
+// ILLM_ERR_ARG); nsplit == 1 needs no `partial`.
+int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache, const void* vcache,
+                          const int32_t* page_table, int table_stride, int page_size, int ring,
+                          const int32_t* seq_slot, const int32_t* slot_len, float* partial,
+                          int nsplit, int B, int nh, int nkv, int hd, float scale, int window,
+                          void* stream);
+
+// Y[M, N] = X[M, K] . W[N, K]^T for bfloat16 X and W, 1 <= M <= 64, K % 8 == 0, on the
+// matrix cores with float32 accumulation; Y float32 or bfloat16.
+int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
+                          void* stream);
+
 // out[b] = index of the largest logit of row b (lowest index on ties).
 int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream);
 

@@ -1,0 +1,270 @@
+// Decode attention for bfloat16: one new token per sequence over the paged cache.
+//
+// The step is bound by reading K and V once.  A 64-lane wave is a work unit: it
+// walks tiles of keys of one (sequence, kv head), all query heads of the group at
+// once, so K and V are read once per group.  LPR lanes share a key row with one
+// 16-byte load each (8 head dims per lane); 64/LPR keys are covered by one load
+// instruction, and a tile's loads are all issued before any is used.  Scores are
+// reduced over the LPR lanes of a row, the running max / sum are wave-wide, and
+// each lane accumulates P.V for its 8 dims over the keys of its row group; the
+// groups are added once at the end.  Splits of the key range run as separate
+// one-wave blocks and leave (acc, max, sum) for the merge kernel.
+//
+// Same chain as src/core/op.cpp:485-498 with S = 1, grouped as
+// src/kern/naive/naive.cpp:576-604.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+#define NEG_INF (-INFINITY)
+
+__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+    f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+    f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+// LPR: lanes per key row (power of two, 8 dims each, LPR * 8 >= head_dim).
+// GC: query heads handled together (power of two >= heads per kv head, at most 8).
+template <int LPR, int GC>
+__global__ void __launch_bounds__(64)
+attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
+                        const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+                        const int32_t* __restrict__ page_table, int table_stride, int page_size,
+                        int ring, const int32_t* __restrict__ seq_slot,
+                        const int32_t* __restrict__ slot_len, float* __restrict__ partial,
+                        int nsplit, int nh, int nkv, int hd, float scale, int window) {
+    constexpr int KPI = 64 / LPR;              // keys per load instruction
+    constexpr int NI = LPR < 16 ? LPR : 16;    // load instructions per tile
+    constexpr int TK = NI * KPI;               // keys per tile
+    const int lane = threadIdx.x, q = lane / LPR, c = lane % LPR;
+    const int G = nh / nkv;
+    const int kvh = blockIdx.x % nkv, g0 = (blockIdx.x / nkv) * GC;
+    const int b = blockIdx.y, sp = blockIdx.z;
+    const int slot = seq_slot[b];
+    const int len = slot_len[slot];
+    const int kf = window > 0 ? max(0, len - window) : 0;
+    const bool dim_ok = c * 8 < hd;
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * hd;
+
+    float qr[GC][8];
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        const bool ok = dim_ok && (g0 + g < G);
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (ok) v = *(const uint4*)(qkv + (size_t)b * rowlen + (size_t)(kvh * G + g0 + g) * hd + c * 8);
+        unpack8(v, qr[g]);
+    }
+    float m[GC], l[GC], acc[GC][8];
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        m[g] = NEG_INF;
+        l[g] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+    }
+
+    const int t_first = kf / TK;
+    const int n_tiles = (len + TK - 1) / TK - t_first;
+    const int per = (n_tiles + nsplit - 1) / nsplit;
+    const int t_lo = t_first + sp * per;
+    const int t_hi = min(t_first + n_tiles, t_lo + per);
+
+    for (int t = t_lo; t < t_hi; ++t) {
+        const int k0 = t * TK;
+        int lp = k0 / page_size;
+        if (ring > 0) lp %= ring;
+        const int phys = page_table[(size_t)slot * table_stride + lp];
+        const size_t base = (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)hd +
+                            (size_t)q * hd + c * 8;
+        uint4 kreg[NI], vreg[NI];
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            kreg[j] = dim_ok ? *(const uint4*)(kcache + base + (size_t)j * KPI * hd)
+                             : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            vreg[j] = dim_ok ? *(const uint4*)(vcache + base + (size_t)j * KPI * hd)
+                             : make_uint4(0, 0, 0, 0);
+
+        // scores: lane (q, c) ends up owning key k0 + c * KPI + q (if c < NI)
+        float s_own[GC];
+#pragma unroll
+        for (int g = 0; g < GC; ++g) s_own[g] = NEG_INF;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            float kf8[8];
+            unpack8(kreg[j], kf8);
+#pragma unroll
+            for (int g = 0; g < GC; ++g) {
+                float part = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) part = fmaf(qr[g][i], kf8[i], part);
+#pragma unroll
+                for (int o = 1; o < LPR; o <<= 1) part += __shfl_xor(part, o, ILLM_WAVE);
+                if (c == j) s_own[g] = part * scale;
+            }
+        }
+        const int key_own = k0 + c * KPI + q;
+        const bool own_ok = (c < NI) && key_own < len && key_own >= kf;
+        float p_own[GC];
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            const float s = own_ok ? s_own[g] : NEG_INF;
+            const float m_new = fmaxf(m[g], wave_max(s));
+            const float alpha = (m_new == NEG_INF) ? 1.f : expf(m[g] - m_new);
+            const float p = own_ok ? expf(s - m_new) : 0.f;
+            p_own[g] = p;
+            l[g] = l[g] * alpha + wave_sum(p);
+            m[g] = m_new;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] *= alpha;
+        }
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int key = k0 + j * KPI + q;
+            const bool ok = key < len && key >= kf;
+            float vf8[8];
+            unpack8(vreg[j], vf8);
+#pragma unroll
+            for (int g = 0; g < GC; ++g) {
+                float pj = __shfl(p_own[g], q * LPR + j, ILLM_WAVE);
+                pj = ok ? pj : 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(pj, ok ? vf8[i] : 0.f, acc[g][i]);
+            }
+        }
+    }
+    // add the row groups' shares
+#pragma unroll
+    for (int g = 0; g < GC; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float a = acc[g][i];
+#pragma unroll
+            for (int o = LPR; o < 64; o <<= 1) a += __shfl_xor(a, o, ILLM_WAVE);
+            acc[g][i] = a;
+        }
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        if (g0 + g >= G) continue;
+        const int h = kvh * G + g0 + g;
+        if (nsplit == 1) {
+            if (q == 0 && dim_ok) {
+                const float inv = 1.0f / l[g];
+                uint4 o;
+                o.x = (uint32_t)f32_to_bf16(acc[g][0] * inv) | ((uint32_t)f32_to_bf16(acc[g][1] * inv) << 16);
+                o.y = (uint32_t)f32_to_bf16(acc[g][2] * inv) | ((uint32_t)f32_to_bf16(acc[g][3] * inv) << 16);
+                o.z = (uint32_t)f32_to_bf16(acc[g][4] * inv) | ((uint32_t)f32_to_bf16(acc[g][5] * inv) << 16);
+                o.w = (uint32_t)f32_to_bf16(acc[g][6] * inv) | ((uint32_t)f32_to_bf16(acc[g][7] * inv) << 16);
+                *(uint4*)(out + ((size_t)b * nh + h) * hd + c * 8) = o;
+            }
+        } else {
+            float* pp = partial + (((size_t)b * nh + h) * nsplit + sp) * (size_t)(hd + 2);
+            if (q == 0 && dim_ok) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pp[c * 8 + i] = acc[g][i];
+            }
+            if (lane == 0) {
+                pp[hd] = m[g];
+                pp[hd + 1] = l[g];
+            }
+        }
+    }
+}
+
+// grid (heads, sequences): combine the splits (same as the generic path's merge)
+__global__ void attn_decode_bf16_merge_kernel(const float* __restrict__ partial,
+                                              bf16_t* __restrict__ out, int nsplit, int nh, int hd) {
+    const int h = blockIdx.x, b = blockIdx.y;
+    const float* pp = partial + ((size_t)b * nh + h) * nsplit * (size_t)(hd + 2);
+    float m = NEG_INF;
+    for (int s = 0; s < nsplit; ++s) m = fmaxf(m, pp[(size_t)s * (hd + 2) + hd]);
+    float L = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = pp[(size_t)s * (hd + 2) + hd];
+        if (ms != NEG_INF) L += expf(ms - m) * pp[(size_t)s * (hd + 2) + hd + 1];
+    }
+    const float inv = 1.0f / L;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float ms = pp[(size_t)s * (hd + 2) + hd];
+            if (ms != NEG_INF) a += expf(ms - m) * pp[(size_t)s * (hd + 2) + d];
+        }
+        out[((size_t)b * nh + h) * hd + d] = f32_to_bf16(a * inv);
+    }
+}
+
+template <int LPR, int GC>
+static int launch_decode(const void* qkv, void* out, const void* kcache, const void* vcache,
+                         const int32_t* page_table, int table_stride, int page_size, int ring,
+                         const int32_t* seq_slot, const int32_t* slot_len, float* partial,
+                         int nsplit, int B, int nh, int nkv, int hd, float scale, int window,
+                         hipStream_t stream) {
+    const int G = nh / nkv;
+    const int chunks = (G + GC - 1) / GC;
+    hipLaunchKernelGGL((attn_decode_bf16_kernel<LPR, GC>), dim3(nkv * chunks, B, nsplit), dim3(64),
+                       0, stream, (const bf16_t*)qkv, (bf16_t*)out, (const bf16_t*)kcache,
+                       (const bf16_t*)vcache, page_table, table_stride, page_size, ring, seq_slot,
+                       slot_len, partial, nsplit, nh, nkv, hd, scale, window);
+    if (nsplit > 1)
+        hipLaunchKernelGGL(attn_decode_bf16_merge_kernel, dim3(nh, B), dim3(64), 0, stream,
+                           (const float*)partial, (bf16_t*)out, nsplit, nh, hd);
+    return illm_launch_status();
+}
+
+template <int LPR>
+static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcache,
+                           const void* vcache, const int32_t* page_table, int table_stride,
+                           int page_size, int ring, const int32_t* seq_slot,
+                           const int32_t* slot_len, float* partial, int nsplit, int B, int nh,
+                           int nkv, int hd, float scale, int window, hipStream_t stream) {
+#define GO(GC_)                                                                                   \
+    return launch_decode<LPR, GC_>(qkv, out, kcache, vcache, page_table, table_stride, page_size, \
+                                   ring, seq_slot, slot_len, partial, nsplit, B, nh, nkv, hd,     \
+                                   scale, window, stream)
+    switch (gc) {
+        case 1: GO(1);
+        case 2: GO(2);
+        case 4: GO(4);
+        default: GO(8);
+    }
+#undef GO
+}
+
+// Sizes this kernel takes: bfloat16, head_dim a multiple of 8 up to 256, a page size that
+// is a multiple of 64.  Anything else: ILLM_ERR_ARG (the caller uses the generic kernel).
+extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache,
+                                     const void* vcache, const int32_t* page_table,
+                                     int table_stride, int page_size, int ring,
+                                     const int32_t* seq_slot, const int32_t* slot_len,
+                                     float* partial, int nsplit, int B, int nh, int nkv, int hd,
+                                     float scale, int window, void* stream) {
+    if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 || hd % 8 ||
+        page_size <= 0 || page_size % 64 || nsplit <= 0 || nsplit > 65535 || B > 65535 ||
+        table_stride <= 0 || (nsplit > 1 && !partial))
+        return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    const int G = nh / nkv;
+    int gc = 1;
+    while (gc < G && gc < 8) gc <<= 1;
+    int lpr = 1;
+    while (lpr * 8 < hd) lpr <<= 1;
+    hipStream_t st = (hipStream_t)stream;
+#define GO(LPR_)                                                                                   \
+    return launch_decode_g<LPR_>(gc, qkv, out, kcache, vcache, page_table, table_stride, page_size, \
+                                 ring, seq_slot, slot_len, partial, nsplit, B, nh, nkv, hd, scale, \
+                                 window, st)
+    switch (lpr) {
+        case 1: GO(1);
+        case 2: GO(2);
+        case 4: GO(4);
+        case 8: GO(8);
+        case 16: GO(16);
+        default: GO(32);
+    }
+#undef GO
+}

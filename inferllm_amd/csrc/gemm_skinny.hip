@@ -1,0 +1,148 @@
+// Y[M, N] = X[M, K] . W[N, K]^T for few rows (M <= 64, decoding), bfloat16 operands,
+// float32 accumulation on the matrix cores.  The product is bound by reading W once.
+//
+// MFMA 16x16x32: the A operand is a 16-row tile of W, the B operand 16 rows of X.
+// Both are read straight from global memory: lane (r = lane % 16, q = lane / 16)
+// needs 8 consecutive k of row r at k0 + 8 q, which is one 16-byte load; no LDS
+// staging is needed because W is used once and X is small enough to stay in
+// cache.  A wave owns NTB tiles of 16 W rows and all MT tiles of 16 X rows.  The
+// waves of a block split K in interleaved pieces of U k-steps (U * 64 bytes of
+// each W row at a time) and add their results through LDS in wave order, so the
+// sum has a fixed order.  Lanes of X rows >= M read row M - 1 and their results
+// are dropped.
+//
+// The reference calls cublasSgemm with M = 1 here (src/kern/gpu/kernel_gpu.cu:420-435).
+#include "api.h"
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+#define SK_U 4   // k-steps (of 32) per wave iteration
+
+template <int MT, int NTB>
+__global__ void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                   void* __restrict__ Y, int y_dt, int M, int N, int K) {
+    extern __shared__ float red[];   // [waves][NTB * MT * 64 * 4]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int waves = blockDim.x >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int n_base = blockIdx.x * (16 * NTB);
+
+    const bf16_t* wrow[NTB];
+#pragma unroll
+    for (int nt = 0; nt < NTB; ++nt) {
+        int n = n_base + nt * 16 + r;
+        n = n < N ? n : N - 1;
+        wrow[nt] = W + (size_t)n * K;
+    }
+    const bf16_t* xrow[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int mm = mt * 16 + r;
+        mm = mm < M ? mm : M - 1;
+        xrow[mt] = X + (size_t)mm * K;
+    }
+    f32x4_t acc[NTB][MT];
+#pragma unroll
+    for (int nt = 0; nt < NTB; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+    const int ksteps = (K + 31) / 32;
+    for (int s0 = wave * SK_U; s0 < ksteps; s0 += waves * SK_U) {
+        uint4 a[NTB][SK_U], b[MT][SK_U];
+#pragma unroll
+        for (int u = 0; u < SK_U; ++u) {
+            const int k = (s0 + u) * 32 + q * 8;
+            const bool ok = k < K;           // K is a multiple of 8: a lane's 8 values are all in or all out
+#pragma unroll
+            for (int nt = 0; nt < NTB; ++nt)
+                a[nt][u] = ok ? *(const uint4*)(wrow[nt] + k) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                b[mt][u] = ok ? *(const uint4*)(xrow[mt] + k) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < SK_U; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NTB; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        *(bf16x8_t*)&a[nt][u], *(bf16x8_t*)&b[mt][u], acc[nt][mt], 0, 0, 0);
+    }
+    // acc[nt][mt][i] = Y[m = mt*16 + r][n = n_base + nt*16 + q*4 + i]
+    constexpr int PER_WAVE = NTB * MT * 64 * 4;
+    if (waves > 1) {
+#pragma unroll
+        for (int nt = 0; nt < NTB; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                *(f32x4_t*)(red + (size_t)wave * PER_WAVE + ((nt * MT + mt) * 64 + lane) * 4) =
+                    acc[nt][mt];
+        __syncthreads();
+    }
+    // every thread of the block sums some of the (nt, mt, lane) groups over the waves
+    for (int grp = threadIdx.x; grp < NTB * MT * 64; grp += blockDim.x) {
+        f32x4_t v;
+        int l2, nt, mt;
+        if (waves > 1) {
+            v = *(f32x4_t*)(red + grp * 4);
+            for (int w = 1; w < waves; ++w) {
+                const f32x4_t o = *(f32x4_t*)(red + (size_t)w * PER_WAVE + grp * 4);
+                v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3];
+            }
+            l2 = grp & 63; mt = (grp >> 6) % MT; nt = (grp >> 6) / MT;
+        } else {
+            // one wave: thread == lane; walk this lane's own tiles
+            l2 = lane; mt = (grp >> 6) % MT; nt = (grp >> 6) / MT;
+            v = acc[0][0];
+#pragma unroll
+            for (int a2 = 0; a2 < NTB; ++a2)
+#pragma unroll
+                for (int b2 = 0; b2 < MT; ++b2)
+                    if (a2 == nt && b2 == mt) v = acc[a2][b2];
+        }
+        const int mrow = mt * 16 + (l2 & 15);
+        const int n0 = n_base + nt * 16 + (l2 >> 4) * 4;
+        if (mrow >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[i]);
+    }
+}
+
+template <int MT, int NTB>
+static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
+                         int waves, hipStream_t st) {
+    const int blocks = (N + 16 * NTB - 1) / (16 * NTB);
+    const size_t smem = waves > 1 ? (size_t)waves * NTB * MT * 64 * 4 * sizeof(float) : 0;
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB>), dim3(blocks), dim3(64 * waves), smem, st,
+                       (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K);
+    return illm_launch_status();
+}
+
+// Takes bfloat16 X and W, M in 1..64, K a multiple of 8.  Otherwise ILLM_ERR_ARG.
+extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int y_dt, int M,
+                                     int N, int K, void* stream) {
+    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
+        return ILLM_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int ksteps = (K + 31) / 32;
+    const int max_by_k = (ksteps + SK_U - 1) / SK_U;     // more waves than k pieces would idle
+    auto pick = [&](int ntb, int mt) {
+        const int blocks = (N + 16 * ntb - 1) / (16 * ntb);
+        int w = (2048 + blocks - 1) / blocks;            // aim at ~2048 waves on the chip
+        const int lds_cap = (64 * 1024) / (ntb * mt * 1024);
+        w = w < 1 ? 1 : w;
+        w = w > 16 ? 16 : w;
+        w = w > lds_cap ? lds_cap : w;
+        w = w > max_by_k ? max_by_k : w;
+        return w < 1 ? 1 : w;
+    };
+    if (M <= 16) return launch_skinny<1, 2>(X, W, Y, y_dt, M, N, K, pick(2, 1), st);
+    if (M <= 32) return launch_skinny<2, 2>(X, W, Y, y_dt, M, N, K, pick(2, 2), st);
+    if (M <= 48) return launch_skinny<3, 2>(X, W, Y, y_dt, M, N, K, pick(2, 3), st);
+    return launch_skinny<4, 2>(X, W, Y, y_dt, M, N, K, pick(2, 4), st);
+}

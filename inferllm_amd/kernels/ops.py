@@ -178,22 +178,41 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     if x.dtype == torch.float32 or w.dtype == torch.float32:
         return gemm_generic(x, w, out_dtype)
     M, K = x.shape
-    if M <= SKINNY_MAX_ROWS and skinny_fits(M, w.shape[0], K):
+    if M == 0:
+        return torch.empty((0, w.shape[0]), dtype=out_dtype, device=x.device)
+    if skinny_fits(M, w.shape[0], K):
         return gemm_skinny_bf16(x, w, out_dtype)
+    if out_dtype == torch.float32 and K % 8 == 0:
+        # float32 results (logits) keep the accumulator's precision: 64 rows at a time
+        return torch.cat([gemm_skinny_bf16(x[i:i + SKINNY_MAX_ROWS], w, out_dtype)
+                          for i in range(0, M, SKINNY_MAX_ROWS)], dim=0)
+    if out_dtype == torch.float32:
+        return gemm_generic(x, w, out_dtype)
     _gpu(x, w)
-    y = torch.matmul(x, w.t())
-    return y if out_dtype == y.dtype else y.to(out_dtype)
+    return torch.matmul(x, w.t())
 
 
 SKINNY_MAX_ROWS = 64
 
 
 def skinny_fits(M: int, N: int, K: int) -> bool:
-    return False
+    """Shapes the few-rows MFMA kernel takes (csrc/gemm_skinny.hip)."""
+    return 1 <= M <= SKINNY_MAX_ROWS and K % 8 == 0
 
 
-def gemm_skinny_bf16(x, w, out_dtype):
-    raise KernelError("no skinny kernel in this build")
+def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M <= 64, K] . w [N, K]^T, both bfloat16, float32 accumulation on the matrix cores."""
+    _gpu(x, w)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands")
+    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1],
+          f"linear: x {tuple(x.shape)} against w {tuple(w.shape)}")
+    M, K = x.shape
+    N = w.shape[0]
+    _need(skinny_fits(M, N, K), f"gemm_skinny: M={M} K={K} not taken")
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_gemm_skinny_bf16(_p(x), _p(w), _p(y), _code(y), M, N, K, _stream()),
+           "gemm_skinny")
+    return y
 
 
 # ------------------------------------------------------------------ attention
@@ -215,9 +234,9 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
 def decode_splits(B: int, nh: int, max_len: int) -> int:
     """How many ways to cut the keys of a decode step so that the launch fills the chip."""
     blocks = max(1, B * nh)
-    want = max(1, 1024 // blocks)
-    tiles = max(1, (max_len + 255) // 256)
-    return max(1, min(want, tiles, 64))
+    want = max(1, -(-1024 // blocks))
+    tiles = max(1, (max_len + 63) // 64)
+    return max(1, min(want, tiles, 32))
 
 
 def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
@@ -233,6 +252,14 @@ def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
           kcache.shape[1:] == (nkv, page_size, hd), "attn_decode: cache shape or dtype")
     _need(nh % nkv == 0, "attn_decode: heads must be a multiple of kv heads")
     out = torch.empty((B, nh * hd), dtype=qkv.dtype, device=qkv.device)
+    if qkv.dtype == torch.bfloat16 and hd % 8 == 0 and page_size % 64 == 0:
+        partial = (torch.empty((B, nh, nsplit, hd + 2), dtype=torch.float32, device=qkv.device)
+                   if nsplit > 1 else None)
+        _check(_lib().illm_attn_decode_bf16(
+            _p(qkv), _p(out), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
+            page_size, ring, _p(seq_slot), _p(slot_len), _p(partial), nsplit, B, nh, nkv, hd,
+            ctypes.c_float(scale), window, _stream()), f"attn_decode_bf16 (head_dim {hd})")
+        return out
     partial = torch.empty((B, nh, nsplit, hd + 2), dtype=torch.float32, device=qkv.device)
     _check(_lib().illm_attn_decode_generic(
         _p(qkv), _p(out), _code(qkv), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],

@@ -85,7 +85,7 @@ class Attention(Mixer):
             o = ops.attn_prefill(qkv, ctx.cu_seqlens, ctx.n_seqs, ctx.max_len, nh, nkv, hd,
                                  self.scale, window)
         else:
-            nsplit = ops.decode_splits(ctx.n_seqs, nh, ctx.max_len if not window else min(ctx.max_len, window))
+            nsplit = ops.decode_splits(ctx.n_seqs, nkv, ctx.max_len if not window else min(ctx.max_len, window))
             o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
                                 ctx.seq_slot, ctx.cache.slot_len, nh, nkv, hd, self.scale, window,
                                 nsplit)

@@ -210,6 +210,45 @@ def test_attn_decode(dtype, nh, nkv, hd, lens, window, nsplit):
     close(got, want, dtype, scale=2)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,lens,window,nsplit", [
+    (32, 32, 128, [600, 1, 64, 65], 0, 1), (32, 8, 128, [300, 70], 0, 3), (4, 4, 16, [7, 200], 0, 2),
+    (8, 1, 64, [1000], 0, 32), (6, 2, 24, [5, 11, 130], 0, 2), (16, 1, 256, [257, 31], 0, 2),
+    (5, 5, 96, [130, 520], 70, 5), (12, 4, 32, [90, 17, 700], 13, 2), (3, 3, 8, [129], 0, 1),
+    (20, 2, 48, [333], 0, 4)])
+def test_attn_decode_bf16_pages_of_64(nh, nkv, hd, lens, window, nsplit):
+    """The fast bfloat16 kernel (pages of 64 rows, as the engine's cache has them); stale rows
+    of the pages are NaN and must not leak into the result."""
+    dtype, page = torch.bfloat16, 64
+    ring = (window + page - 2) // page + 1 if window else 0
+    pt, kc, vc, slots, slot_len = paged_case(dtype, nkv, hd, lens, page, ring)
+    for b, s in enumerate(slots.tolist()):
+        n = lens[b]
+        if not ring:
+            lp, r = divmod(n, page)
+            if r:
+                kc[int(pt[s, lp]), :, r:] = float("nan"); vc[int(pt[s, lp]), :, r:] = float("nan")
+    kc[-1] = float("nan"); vc[-1] = float("nan")
+    B = len(lens)
+    qkv = rnd(B, (nh + 2 * nkv) * hd, dtype=dtype, seed=11)
+    scale = 1.0 / math.sqrt(hd)
+    got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring, slots.to(DEV),
+                            slot_len.to(DEV), nh, nkv, hd, scale, window, nsplit)
+    want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, slot_len, nh, nkv, hd, scale, window, nsplit)
+    close(got, want, dtype, scale=2)
+
+
+@pytest.mark.parametrize("ydt", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 2, 128), (4, 128, 128), (8, 4096, 4096), (1, 32000, 4096), (16, 411, 80),
+                                   (17, 100, 1000), (33, 64, 1008), (48, 31, 8), (64, 4096, 11008), (7, 12288, 4096),
+                                   (64, 33, 40)])
+def test_gemm_skinny(ydt, M, N, K):
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+    got = ops().gemm_skinny_bf16(x.to(DEV), w.to(DEV), ydt)
+    close(got, R.linear(x, w, ydt), ydt, scale=math.sqrt(K))
+    if ydt == torch.float32:       # float32 out keeps the accumulator: far tighter than bfloat16
+        torch.testing.assert_close(got.double().cpu(), R.linear(x, w, torch.float64), atol=2e-4 * math.sqrt(K), rtol=1e-4)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attn_decode_finds_one_far_key(dtype):
     """One key among hundreds is made to stand out: the output must be its value."""
