@@ -162,6 +162,7 @@ class CacheManager:
             line: torch.zeros((max_slots + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
             for line, s in state_lines.items()}
         self.len_host = torch.zeros(max_slots + 1, dtype=torch.int32)
+        self.len_host[self.spare_slot] = 1      # padding rows attend to one (spare) key, not to none
         self.slot_len = self.len_host.to(device)
         self._len_dirty = False
 

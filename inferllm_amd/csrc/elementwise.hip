@@ -60,6 +60,77 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict
     }
 }
 
+// The same with every element of the row held in registers: each thread owns NV
+// groups of 4 consecutive floats, all loads are issued before the first use, and x is
+// read once.  Needs E % 4 == 0 and E <= 1024 * NV.
+__device__ __forceinline__ float4 ld4_f(const void* p, int dt, size_t i4) {
+    if (dt == ILLM_BF16) {
+        const uint2 u = ((const uint2*)p)[i4];
+        return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                           __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+    }
+    return ((const float4*)p)[i4];
+}
+
+__device__ __forceinline__ void st4_f(void* p, int dt, size_t i4, float4 v) {
+    if (dt == ILLM_BF16) {
+        uint2 u;
+        u.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+        u.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+        ((uint2*)p)[i4] = u;
+    } else {
+        ((float4*)p)[i4] = v;
+    }
+}
+
+template <int NV>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, int delta_dt,
+                       const void* __restrict__ w, int w_dt, void* __restrict__ out, int out_dt,
+                       const int32_t* __restrict__ row_idx, int E, float eps) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const int in_row = row_idx ? row_idx[r] : r;
+    const int E4 = E >> 2;
+    const size_t ib = (size_t)in_row * E4, ob = (size_t)r * E4;
+    float4 v[NV], wv[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        wv[j] = v[j];
+        if (i < E4) {
+            v[j] = ((const float4*)x)[ib + i];
+            wv[j] = ld4_f(w, w_dt, i);
+        }
+    }
+    if (delta) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < E4) {
+                const float4 d = ld4_f(delta, delta_dt, ib + i);
+                v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
+                if (!row_idx) ((float4*)x)[ib + i] = v[j];
+            }
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+        ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)E + eps);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < E4)
+            st4_f(out, out_dt, ob + i,
+                  make_float4((v[j].x * scale) * wv[j].x, (v[j].y * scale) * wv[j].y,
+                              (v[j].z * scale) * wv[j].z, (v[j].w * scale) * wv[j].w));
+    }
+}
+
 extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const void* w,
                                 int w_dt, void* out, int out_dt, const int32_t* row_idx,
                                 int rows, int E, float eps, void* stream) {
@@ -67,8 +138,18 @@ extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const
         (delta && !illm_dtype_ok(delta_dt)))
         return ILLM_ERR_ARG;
     if (rows == 0) return ILLM_OK;
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x,
-                       delta, delta_dt, w, w_dt, out, out_dt, row_idx, E, eps);
+    hipStream_t st = (hipStream_t)stream;
+#define VEC(NV_)                                                                              \
+    hipLaunchKernelGGL(add_rmsnorm_vec_kernel<NV_>, dim3(rows), dim3(256), 0, st, x, delta,   \
+                       delta_dt, w, w_dt, out, out_dt, row_idx, E, eps)
+    if (E % 4 == 0 && E <= 1024) VEC(1);
+    else if (E % 4 == 0 && E <= 2048) VEC(2);
+    else if (E % 4 == 0 && E <= 4096) VEC(4);
+    else if (E % 4 == 0 && E <= 8192) VEC(8);
+    else
+        hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, delta, delta_dt, w,
+                           w_dt, out, out_dt, row_idx, E, eps);
+#undef VEC
     return illm_launch_status();
 }
 

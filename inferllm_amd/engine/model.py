@@ -43,6 +43,10 @@ class DecoderModel:
             elif e.cache_line not in writers:
                 raise ValueError(f"schedule: cache line {e.cache_line} is read before any run writes it")
         self.loaded = False
+        every = [self.embedding, self.final_norm, self.head]
+        for layer in self.layers:
+            every.extend([layer] + layer.parts())
+        self.graph_safe = all(getattr(p, "graph_safe", True) for p in every)
 
     # ------------------------------------------------------------ weights
     def wants(self) -> Dict[str, TensorWant]:

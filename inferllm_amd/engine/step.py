@@ -73,7 +73,8 @@ class StepRunner:
         self.model, self.cache = model, cache
         self.act_dtype, self.device = act_dtype, device
         self.vocab_size = model.spec.vocab_size
-        self.use_graphs = use_graphs and os.environ.get("INFERLLM_NO_GRAPH", "0") != "1"
+        self.use_graphs = (use_graphs and model.graph_safe
+                           and os.environ.get("INFERLLM_NO_GRAPH", "0") != "1")
         self._graphs: Dict[int, _DecodeGraph] = {}
 
     # ------------------------------------------------------------ checks

@@ -48,7 +48,13 @@ class StepContext:
 
 
 class Part:
-    """Base of all parts: parameter names -> checkpoint names in `self.tensors`."""
+    """Base of all parts: parameter names -> checkpoint names in `self.tensors`.
+
+    `graph_safe`: the part's forward only launches work on the current stream (no host
+    synchronisation, no host reads of device data), so decode steps that contain it may
+    be captured into a HIP graph.  A part that reads device data on the host sets it False.
+    """
+    graph_safe = True
 
     def __init__(self, tensors: Optional[Dict[str, str]] = None):
         self.tensors: Dict[str, str] = dict(tensors or {})

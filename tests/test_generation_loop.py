@@ -1,0 +1,149 @@
+"""The generation loop's decisions, with a fake model in place of the GPU:
+batches, stop tokens, sequences that end earlier, limits, slots given back."""
+import pytest
+
+from inferllm_amd.engine import GenerationLoop, StepEntry
+from inferllm_amd.sampling import SamplingParams, request_seed, uniform
+
+
+class FakeModel:
+    """next token = (sum of the sequence so far) % 50; keeps its own view of each slot."""
+
+    def __init__(self, n_slots):
+        self.free = list(range(n_slots - 1, -1, -1))
+        self.seq = {}
+        self.steps = []
+        self.max_live = 0
+
+    def alloc(self):
+        s = self.free.pop()
+        self.seq[s] = []
+        return s
+
+    def release(self, s):
+        assert s in self.seq, "slot freed twice"
+        del self.seq[s]
+        self.free.append(s)
+
+    def step(self, entries):
+        first = [len(self.seq[e.slot]) == 0 for e in entries]
+        assert all(first) or (not any(first) and all(len(e.tokens) == 1 for e in entries))
+        for e in entries:
+            self.seq[e.slot].extend(e.tokens)
+        self.steps.append([(e.slot, len(e.tokens)) for e in entries])
+        self.max_live = max(self.max_live, len(self.seq))
+        return [sum(self.seq[e.slot]) % 50 for e in entries]
+
+    @staticmethod
+    def sample(logits, seeds, counters, histories):
+        return list(logits)
+
+
+def expected(prompt, n, stops=(), include_stop=False, limit=10**9):
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = sum(seq) % 50
+        if t in stops:
+            if include_stop:
+                out.append(t)
+            break
+        out.append(t)
+        seq.append(t)
+        if len(seq) > limit:      # the token could not be fed back
+            break
+    return out
+
+
+def loop_for(model, max_batch=3, max_tokens=64 * 12, max_seq_len=256):
+    return GenerationLoop(model.step, model.sample, model.alloc, model.release, max_batch,
+                          max_tokens, max_seq_len)
+
+
+PROMPTS = [[1, 2, 3], [7], [4, 4, 4, 4, 9], [10, 11], [3, 3], [8, 1, 1, 1, 1, 1, 2], [5]]
+
+
+def test_every_request_gets_its_own_continuation_in_batches_of_three():
+    m = FakeModel(3)
+    loop = loop_for(m)
+    out = loop.run(PROMPTS, SamplingParams(), 6)
+    assert out == [expected(p, 6) for p in PROMPTS]
+    assert m.max_live <= 3 and not m.seq                    # slots all given back
+    assert loop.stats.batches == 3 and loop.stats.prompt_tokens == sum(map(len, PROMPTS))
+    # first step of each batch carries whole prompts, later ones single tokens
+    assert m.steps[0] == [(0, 3), (1, 1), (2, 5)]
+    assert all(n == 1 for s in m.steps[1:6] for _, n in s)
+
+
+def test_stop_tokens_end_a_sequence_early_and_the_rest_goes_on():
+    stops = {expected(PROMPTS[0], 6)[2], expected(PROMPTS[2], 6)[0]}
+    m = FakeModel(3)
+    out = loop_for(m).run(PROMPTS[:3], SamplingParams(), 6, stops)
+    assert out == [expected(p, 6, stops) for p in PROMPTS[:3]]
+    assert out[2] == [] and len(out[0]) == 2 and len(out[1]) > 2
+    sizes = [len(s) for s in m.steps]
+    assert sizes[0] == 3 and sizes[1] == 2 and sizes[-1] == 1   # the batch shrinks
+    out = loop_for(FakeModel(3)).run(PROMPTS[:3], SamplingParams(), 6, stops, include_stop=True)
+    assert out == [expected(p, 6, stops, True) for p in PROMPTS[:3]]
+
+
+def test_context_limit_ends_a_sequence():
+    m = FakeModel(2)
+    out = loop_for(m, max_batch=2, max_seq_len=6).run([[1, 2, 3], [9, 9, 9, 9, 9, 9]], SamplingParams(), 10)
+    assert out == [expected([1, 2, 3], 10, limit=6), expected([9] * 6, 10, limit=6)]
+    assert len(out[0]) == 4 and len(out[1]) == 1
+    with pytest.raises(ValueError, match="longer than"):
+        loop_for(FakeModel(2), max_seq_len=6).run([[1] * 7], SamplingParams(), 1)
+    with pytest.raises(ValueError, match="empty prompt"):
+        loop_for(FakeModel(2)).run([[]], SamplingParams(), 1)
+
+
+def test_batches_respect_cache_room():
+    loop = loop_for(FakeModel(8), max_batch=8, max_tokens=64 * 4)
+    lens = [60, 10, 70, 5, 5]
+    assert loop.room_needed(60, 6) == 128 and loop.room_needed(10, 6) == 64
+    assert loop.next_batch([0, 1, 2, 3, 4], lens, 6) == [0, 1]           # 128 + 64, then 128 does not fit
+    assert loop.next_batch([2, 3, 4], lens, 6) == [2, 3, 4]
+    big = loop_for(FakeModel(8), max_batch=8, max_tokens=64 * 4, max_seq_len=2048)
+    with pytest.raises(ValueError, match="more cache room"):
+        big.next_batch([0], [1000], 6)
+    m = FakeModel(8)
+    loop = loop_for(m, max_batch=8, max_tokens=64 * 4)
+    prompts = [[1] * n for n in lens]
+    assert loop.run(prompts, SamplingParams(), 6) == [expected(p, 6) for p in prompts]
+    assert loop.stats.batches == 2
+
+
+def test_zero_new_tokens_and_slots_returned_on_error():
+    m = FakeModel(2)
+    assert loop_for(m).run(PROMPTS[:2], SamplingParams(), 0) == [[], []]
+
+    def broken(entries):
+        raise RuntimeError("boom")
+    loop = GenerationLoop(broken, m.sample, m.alloc, m.release, 2, 640, 64)
+    with pytest.raises(RuntimeError, match="boom"):
+        loop.run(PROMPTS[:2], SamplingParams(), 3)
+    assert not m.seq and len(m.free) == 2
+
+
+def test_draws_depend_on_request_and_count_only():
+    calls = []
+
+    def sample(logits, seeds, counters, histories):
+        calls.append((list(seeds), list(counters)))
+        return list(logits)
+    m = FakeModel(3)
+    GenerationLoop(m.step, sample, m.alloc, m.release, 2, 6400, 64).run(PROMPTS[:3], SamplingParams(seed=9), 3)
+    assert calls[0] == ([request_seed(9, 0), request_seed(9, 1)], [0, 0])
+    assert calls[1][1] == [1, 1] and calls[3] == ([request_seed(9, 2)], [0])
+    us = [uniform(request_seed(9, i), c) for i in range(3) for c in range(50)]
+    assert all(0.0 <= u < 1.0 for u in us) and len(set(us)) == len(us)
+    assert abs(sum(us) / len(us) - 0.5) < 0.1
+
+
+def test_sampling_params_validation():
+    SamplingParams(temperature=0.8, top_k=40, top_p=0.95, repeat_penalty=1.1).validate()
+    for bad in (dict(temperature=-1), dict(top_p=0.0), dict(top_p=1.5), dict(repeat_penalty=0),
+                dict(repeat_last_n=1000)):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad).validate()
+    assert SamplingParams().greedy and not SamplingParams(temperature=0.1).greedy

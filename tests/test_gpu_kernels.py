@@ -45,7 +45,7 @@ def test_embed(dtype, V, E, ids):
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("T,E,eps", [(4, 4096, 1e-5), (3, 80, 1e-6), (1, 1001, 3e-2), (70, 96, 1e-5)])
+@pytest.mark.parametrize("T,E,eps", [(4, 4096, 1e-5), (3, 80, 1e-6), (1, 1001, 3e-2), (70, 96, 1e-5), (2, 6000, 1e-5), (2, 9000, 1e-5), (5, 1536, 1e-6)])
 def test_add_rmsnorm(out_dtype, w_dtype, T, E, eps):
     x = rnd(T, E, seed=1) * 0.05            # small rows: eps matters
     w = (1 + rnd(E, seed=2) * 0.1).to(w_dtype)

@@ -1,0 +1,243 @@
+"""Each part alone on the GPU against the plain functions; HIP graph replays against
+eager steps; and a toy mixer with state of its own, defined here, registered, built
+and stepped without a change to the framework's files."""
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def rnd(*shape, seed=0, std=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * std).to(dtype)
+
+
+def make_ctx(lens_before, new_tokens, kv_lines, dtype, state_lines=None, max_slots=4, max_seq_len=512):
+    """A cache and the context of one step: sequence i holds lens_before[i] tokens and gets
+    new_tokens[i] more.  Returns (ctx, cache, slots)."""
+    from inferllm_amd.cache import CacheManager
+    from inferllm_amd.parts import StepContext
+    cache = CacheManager(kv_lines, state_lines or {}, 64 * 16, max_slots, max_seq_len, dtype, DEV)
+    slots = [cache.alloc_slot() for _ in lens_before]
+    for s, n in zip(slots, lens_before):
+        if n:
+            cache.extend(s, 0, n)
+    return cache, slots
+
+
+def step_ctx(cache, slots, starts, counts, dtype, prefill):
+    from inferllm_amd.parts import StepContext
+    for s, a, n in zip(slots, starts, counts):
+        cache.extend(s, a, n)
+    cache.upload()
+    pos = [a + j for a, n in zip(starts, counts) for j in range(n)]
+    slot = [s for s, n in zip(slots, counts) for _ in range(n)]
+    cu = [0]
+    for n in counts:
+        cu.append(cu[-1] + n)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    return StepContext(device=DEV, act_dtype=dtype, prefill=prefill, n_rows=len(pos), n_seqs=len(slots),
+                       tokens=i32([0] * len(pos)), row_pos=i32(pos), row_slot=i32(slot), cu_seqlens=i32(cu),
+                       seq_slot=i32(slots), max_len=max(a + n for a, n in zip(starts, counts)), cache=cache)
+
+
+TOL = {torch.float32: 2e-5, torch.bfloat16: 3e-2}
+
+
+def rel(got, want):
+    return float((got.double().cpu() - want).abs().max() / want.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,E,theta,window", [(4, 2, 24, 96, 500000.0, None), (6, 6, 16, 40, 10000.0, None),
+                                                        (8, 2, 64, 72, 1234.5, 21)])
+def test_attention_part_whole_then_token_by_token(dtype, nh, nkv, hd, E, theta, window):
+    from inferllm_amd.parts import build_part
+    from inferllm_amd.config import PartSpec
+    names = {"q": "q", "k": "k", "v": "v", "o": "o"}
+    att = build_part("mixer", PartSpec("attention", {"hidden_size": E, "num_heads": nh, "num_kv_heads": nkv,
+                                                       "head_dim": hd, "window": window, "softmax_scale": None}, names))
+    rot = build_part("position", PartSpec("rotary", {"head_dim": hd, "rotary_dim": hd, "theta": theta,
+                                                       "pairing": "half", "max_positions": 512}))
+    w = {"q": rnd(nh * hd, E, seed=1, std=0.2), "k": rnd(nkv * hd, E, seed=2, std=0.2),
+         "v": rnd(nkv * hd, E, seed=3, std=0.2), "o": rnd(E, nh * hd, seed=4, std=0.2)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    assert {k: tuple(v.shape) for k, v in w.items()} == {k: tuple(t.shape) for k, t in att.wants().items()}
+    att.load({k: v.to(DEV) for k, v in w.items()})
+    lens = [70, 5]
+    hs = [rnd(n, E, seed=10 + i).to(dtype) for i, n in enumerate(lens)]
+
+    def plain(h):
+        S = h.shape[0]
+        q = P.linear(h, w["q"]).reshape(S, nh, hd); k = P.linear(h, w["k"]).reshape(S, nkv, hd)
+        v = P.linear(h, w["v"]).reshape(S, nkv, hd)
+        q, k = P.rope_rotate_half(q, range(S), theta), P.rope_rotate_half(k, range(S), theta)
+        return P.linear(P.causal_attention(q, k, v, window=window), w["o"])
+    want = [plain(h) for h in hs]
+    cache, slots = make_ctx([0, 0], None, {0: att.kv_spec()}, dtype)
+    head = [n - 3 for n in lens]
+    ctx = step_ctx(cache, slots, [0, 0], head, dtype, True)
+    out = att.forward(torch.cat([h[:n] for h, n in zip(hs, head)]).to(DEV), ctx, 0, True, rot)
+    assert rel(out[:head[0]], want[0][:head[0]]) < TOL[dtype] and rel(out[head[0]:], want[1][:head[1]]) < TOL[dtype]
+    for j in range(3):
+        ctx = step_ctx(cache, slots, [n + j for n in head], [1, 1], dtype, False)
+        out = att.forward(torch.stack([h[n + j] for h, n in zip(hs, head)]).to(DEV), ctx, 0, True, rot)
+        for b in range(2):
+            assert rel(out[b], want[b][head[b] + j]) < TOL[dtype], (b, j)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_feed_forward_and_block_parts(dtype):
+    from inferllm_amd.parts import build_part, part_class
+    from inferllm_amd.config import PartSpec
+    E, F, eps = 72, 200, 3e-4
+    norm = build_part("norm", PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": "n"}))
+    ffn = build_part("feed_forward", PartSpec("swiglu", {"hidden_size": E, "intermediate_size": F},
+                                              {"gate": "g", "up": "u", "down": "d"}))
+    w = {"n": (1 + rnd(E, seed=1, std=0.1)).to(dtype), "g": rnd(F, E, seed=2, std=0.2).to(dtype),
+         "u": rnd(F, E, seed=3, std=0.2).to(dtype), "d": rnd(E, F, seed=4, std=0.2).to(dtype)}
+    for p in (norm, ffn):
+        p.load({k: v.to(DEV) for k, v in w.items()})
+    cache, slots = make_ctx([0], None, {}, dtype)
+    ctx = step_ctx(cache, slots, [0], [9], dtype, True)
+    x, delta = rnd(9, E, seed=5, std=0.05), rnd(9, E, seed=6, std=0.05).to(dtype)
+    xg = x.to(DEV)
+    h = norm.forward(xg, delta.to(DEV), ctx)
+    want_x = x.double() + delta.double()
+    assert rel(xg, want_x) < 1e-6 and h.dtype == dtype                      # the residual stays float32
+    assert rel(h, P.rms_norm(want_x, w["n"], eps)) < TOL[dtype]
+    out = ffn.forward(h, ctx)
+    assert rel(out, P.swiglu_ffn(h.cpu(), w["g"], w["u"], w["d"])) < TOL[dtype]
+
+
+def test_decode_graph_replays_equal_eager_steps(tmp_path):
+    """The same decode steps through the captured HIP graph (replayed many times, with other
+    work and synchronisations between) and eagerly: every replay equals its eager step."""
+    import inferllm_amd as I
+    from tiny import TINY_B, make_model_dir, random_ids
+    d = make_model_dir(tmp_path, TINY_B, seed=3, dtype=torch.bfloat16)
+    reqs = [random_ids(n, 320, n) for n in (30, 12, 50)]
+    outs = []
+    for graphs in (True, False):
+        eng = I.Engine.from_pretrained(d, dtype="bfloat16", max_batch=4, use_graphs=graphs)
+        slots = [eng.alloc_slot() for _ in reqs]
+        eng.step([I.StepEntry(s, r[:10], []) for s, r in zip(slots, reqs)])
+        seq = []
+        for j in range(10, 30):
+            live = [(s, r) for s, r in zip(slots, reqs) if j < len(r)]
+            seq.append(eng.step([I.StepEntry(s, [r[j]], [0]) for s, r in live]).clone())
+            torch.cuda.synchronize()
+            junk = torch.randn(256, 256, device="cuda:0") @ torch.randn(256, 256, device="cuda:0")
+            junk.sum().item()
+        outs.append(seq)
+    for a, b in zip(*outs):
+        assert a.shape == b.shape and torch.equal(a, b)
+
+
+# ---------------------------------------------------------------- a toy mixer with state
+def register_toy():
+    from inferllm_amd.cache import StateSpec
+    from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from inferllm_amd.parts import Mixer, register_part
+    from inferllm_amd.weights import TensorWant
+
+    @register_part("mixer", "toy_running_mean")
+    class RunningMean(Mixer):
+        """delta_t = W . mean(h_0 .. h_t): the sum and the count live in per-sequence state."""
+        graph_safe = False          # reads lengths on the host
+
+        def __init__(self, hidden_size, tensors=None):
+            super().__init__(tensors)
+            self.E = hidden_size
+
+        def shapes(self):
+            return {"w": TensorWant((self.E, self.E))}
+
+        def state_spec(self):
+            return StateSpec((self.E + 1,), torch.float32)
+
+        def load(self, tensors):
+            self.w = self._take(tensors, "w").float()
+
+        def forward(self, h, ctx, line, writes_cache, position):
+            state = ctx.cache.state_line(line)
+            cu, slots = ctx.cu_seqlens.tolist(), ctx.seq_slot.tolist()
+            out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+            for b, s in enumerate(slots):
+                rows = h[cu[b]:cu[b + 1]].float()
+                sums = state[s, :self.E] + torch.cumsum(rows, 0)
+                counts = state[s, self.E] + torch.arange(1, rows.shape[0] + 1, device=h.device)
+                out[cu[b]:cu[b + 1]] = sums / counts[:, None]
+                state[s, :self.E] = sums[-1]
+                state[s, self.E] = counts[-1]
+            return (out @ self.w.t()).to(h.dtype)
+
+    @register_architecture("ToyRunningMeanForTests")
+    class ToyConfig:
+        def __init__(self, hidden_size, vocab_size, layers, eps):
+            self.E, self.V, self.L, self.eps = hidden_size, vocab_size, layers, eps
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["hidden_size"], d["vocab_size"], d["layers"], d["eps"])
+
+        def to_dict(self):
+            return {"architectures": ["ToyRunningMeanForTests"], "hidden_size": self.E,
+                    "vocab_size": self.V, "layers": self.L, "eps": self.eps}
+
+        def to_spec(self):
+            norm = lambda n: PartSpec("rms_norm", {"size": self.E, "eps": self.eps}, {"weight": n})
+            layers = [LayerSpec("pre_norm", PartSpec("toy_running_mean", {"hidden_size": self.E}, {"w": f"l{i}.mix"}),
+                                PartSpec("swiglu", {"hidden_size": self.E, "intermediate_size": 2 * self.E},
+                                         {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+                                norm(f"l{i}.n1"), norm(f"l{i}.n2"), None) for i in range(self.L)]
+            return ModelSpec("ToyRunningMeanForTests", self.V, self.E, 4096,
+                             PartSpec("token_embedding", {"vocab_size": self.V, "hidden_size": self.E}, {"weight": "emb"}),
+                             layers, [ScheduleEntry(i, i) for i in range(self.L)], norm("nf"),
+                             PartSpec("lm_head", {"hidden_size": self.E, "vocab_size": self.V}, {"weight": "head"}))
+    return ToyConfig
+
+
+def toy_plain(w, cfg, ids):
+    x = P.embedding(w["emb"], ids)
+    for i in range(cfg["layers"]):
+        h = P.rms_norm(x, w[f"l{i}.n1"], cfg["eps"])
+        mean = torch.cumsum(h, 0) / torch.arange(1, len(ids) + 1, dtype=torch.float64)[:, None]
+        x = x + P.linear(mean, w[f"l{i}.mix"])
+        x = x + P.swiglu_ffn(P.rms_norm(x, w[f"l{i}.n2"], cfg["eps"]), w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+    return P.linear(P.rms_norm(x, w["nf"], cfg["eps"]), w["head"])
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    import inferllm_amd as I
+    from tiny import random_ids, read_weights
+    register_toy()
+    cfg = {"architectures": ["ToyRunningMeanForTests"], "hidden_size": 48, "vocab_size": 100, "layers": 2, "eps": 1e-5}
+    d = I.write_random_model(str(tmp_path / "toy"), I.config_from_dict(cfg), seed=4)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="float32", max_batch=2, max_seq_len=256)
+    assert not eng.cache.groups and set(eng.cache.states) == {0, 1}          # state, and no keys at all
+    reqs = [random_ids(n, 100, n) for n in (20, 7, 33)]
+    want = [toy_plain(w, cfg, r) for r in reqs]
+    for order in ([0, 1], [2, 1]):                                           # slots are used again: state starts at zero
+        slots = {i: eng.alloc_slot() for i in order}
+        head = {i: len(reqs[i]) - 4 for i in order}
+        out = eng.step([I.StepEntry(slots[i], reqs[i][:head[i]], [head[i] - 1]) for i in order])
+        for j, i in enumerate(order):
+            assert rel(out[j], want[i][head[i] - 1]) < 2e-5
+        for t in range(4):
+            out = eng.step([I.StepEntry(slots[i], [reqs[i][head[i] + t]], [0]) for i in order])
+            for j, i in enumerate(order):
+                assert rel(out[j], want[i][head[i] + t]) < 2e-5
+        for i in order:
+            eng.free_slot(slots[i])
+    got = eng.generate([reqs[1]], max_new_tokens=3, stop_token_ids=[])
+    seq = list(reqs[1])
+    for _ in range(3):
+        seq.append(int(torch.argmax(toy_plain(w, cfg, seq)[-1])))
+    assert got == [seq[len(reqs[1]):]]
