@@ -1,0 +1,231 @@
+// Causal attention of whole prompts for bfloat16 on the matrix cores (MFMA 32x32x16),
+// head sizes that are multiples of 32 up to 256, any number of heads and groups,
+// ragged batches.
+//
+// A block of 4 waves takes 128 consecutive query rows of one (sequence, head); a
+// wave owns 32 of them.  Everything is computed transposed, so that a lane owns one
+// query column: S^T = K . Q^T puts 32 keys of one query in a lane's accumulator, the
+// running max and sum of the softmax need no reduction across lanes beyond one
+// exchange between the two half-waves, and the accumulator layout of P^T is already
+// the B-operand layout of the second product O^T = V^T . P^T: P never leaves
+// registers.  K tiles (64 keys) go through LDS as they are; V tiles are transposed on
+// their way into LDS so that 8 consecutive keys of one head dim are contiguous.  Q is
+// read once into registers.  Scores and statistics are float32; exponentials are
+// base 2 with log2(e) folded into the scale.
+//
+// Blocks are numbered so that the query blocks of one (sequence, head) run on the
+// same XCD (consecutive block ids go round the 8 XCDs) and share K and V in its L2,
+// heaviest (last) query blocks first.
+//
+// The chain is src/core/op.cpp:485-498 (scores, scale + mask, softmax, context) with
+// grouped heads as src/kern/naive/naive.cpp:576-604.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+#define PF_BN 64      // keys per tile
+#define PF_BM 128     // query rows per block
+#define NEG_INF (-INFINITY)
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+template <int HD>
+__global__ void __launch_bounds__(256)
+attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
+                         const int32_t* __restrict__ cu, int n_qblk, int nh, int nkv,
+                         float scale_log2, int window, int total_work) {
+    constexpr int KLD = HD + 8;        // K tile row stride: 16 bytes of padding
+    constexpr int VLD = PF_BN + 4;     // V^T row stride
+    constexpr int KS = HD / 16;        // k-steps of the first product
+    constexpr int DB = HD / 32;        // 32-row blocks of O^T
+    __shared__ __attribute__((aligned(16))) bf16_t ks[PF_BN * KLD];
+    __shared__ __attribute__((aligned(16))) bf16_t vts[HD * VLD];
+
+    const int per_xcd = (total_work + 7) / 8;
+    const int w = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (w >= total_work) return;
+    const int qb = n_qblk - 1 - (w % n_qblk);
+    const int hb = w / n_qblk;
+    const int h = hb % nh, b = hb / nh;
+    const int start = cu[b], len = cu[b + 1] - start;
+    const int q0 = qb * PF_BM;
+    if (q0 >= len) return;
+    const int kvh = h / (nh / nkv);
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int lq = lane & 31, half = lane >> 5;
+    const int q_row0 = q0 + wave * 32;
+    const int q = q_row0 + lq;
+    const int qc = q < len ? q : len - 1;
+
+    uint4 qf[KS];
+    {
+        const bf16_t* qp = qkv + (size_t)(start + qc) * rowlen + (size_t)h * HD + half * 8;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) qf[s] = *(const uint4*)(qp + s * 16);
+    }
+    f32x16_t o[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[d][i] = 0.f;
+    float m = NEG_INF, l = 0.f;
+
+    const int k_end = min(len, q0 + PF_BM);
+    int k_begin = window > 0 ? max(0, q0 - window + 1) : 0;
+    k_begin = (k_begin / PF_BN) * PF_BN;
+    const int wk_end = min(len, q_row0 + 32);                       // this wave's last key + 1
+    const int wk_begin = window > 0 ? max(0, q_row0 - window + 1) : 0;
+
+    for (int k0 = k_begin; k0 < k_end; k0 += PF_BN) {
+        __syncthreads();
+        // K tile as it is, V tile transposed; a wave instruction covers 16 keys x 4 chunks
+#pragma unroll
+        for (int it = 0; it < (PF_BN * HD / 8) / 256; ++it) {
+            const int u = tid + it * 256;
+            const int key = ((u >> 6) & 3) * 16 + (u & 15);
+            const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
+            const int krow = min(k0 + key, len - 1);
+            const bf16_t* src = qkv + (size_t)(start + krow) * rowlen;
+            const uint4 kv = *(const uint4*)(src + (size_t)(nh + kvh) * HD + ch * 8);
+            const uint4 vv = *(const uint4*)(src + (size_t)(nh + nkv + kvh) * HD + ch * 8);
+            *(uint4*)(ks + key * KLD + ch * 8) = kv;
+            bf16_t* vd = vts + (ch * 8) * VLD + key;
+            vd[0 * VLD] = (bf16_t)(vv.x & 0xffffu); vd[1 * VLD] = (bf16_t)(vv.x >> 16);
+            vd[2 * VLD] = (bf16_t)(vv.y & 0xffffu); vd[3 * VLD] = (bf16_t)(vv.y >> 16);
+            vd[4 * VLD] = (bf16_t)(vv.z & 0xffffu); vd[5 * VLD] = (bf16_t)(vv.z >> 16);
+            vd[6 * VLD] = (bf16_t)(vv.w & 0xffffu); vd[7 * VLD] = (bf16_t)(vv.w >> 16);
+        }
+        __syncthreads();
+        if (k0 >= wk_end || k0 + PF_BN <= wk_begin) continue;       // nothing visible to this wave
+
+        // S^T[key][q] for two sub-tiles of 32 keys
+        f32x16_t s[2];
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[sub][i] = 0.f;
+            const bf16_t* kp = ks + (sub * 32 + lq) * KLD + half * 8;
+#pragma unroll
+            for (int st = 0; st < KS; ++st) {
+                const uint4 a = *(const uint4*)(kp + st * 16);
+                s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&a,
+                                                                 *(const bf16x8_t*)&qf[st], s[sub],
+                                                                 0, 0, 0);
+            }
+        }
+        const bool need_mask = (k0 + PF_BN > q_row0 + 1) || (k0 + PF_BN > len) || (window > 0);
+        float mx = NEG_INF;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float v = s[sub][i] * scale_log2;
+                if (need_mask) {
+                    const int key = k0 + sub * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
+                    const bool ok = key <= q && key < len && (window <= 0 || key > q - window);
+                    v = ok ? v : NEG_INF;
+                }
+                s[sub][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+        float rs = 0.f;
+        uint4 pb[2][2];
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            float p[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                p[i] = __builtin_amdgcn_exp2f(s[sub][i] - m_use);
+                rs += p[i];
+            }
+#pragma unroll
+            for (int mf = 0; mf < 2; ++mf) {
+                pb[sub][mf].x = pack_bf16x2(p[8 * mf + 0], p[8 * mf + 1]);
+                pb[sub][mf].y = pack_bf16x2(p[8 * mf + 2], p[8 * mf + 3]);
+                pb[sub][mf].z = pack_bf16x2(p[8 * mf + 4], p[8 * mf + 5]);
+                pb[sub][mf].w = pack_bf16x2(p[8 * mf + 6], p[8 * mf + 7]);
+            }
+        }
+        l = l * alpha + rs;
+        m = m_new;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+        // O^T[d][q] += V^T[d][keys] . P^T[keys][q]
+#pragma unroll
+        for (int d = 0; d < DB; ++d) {
+            const bf16_t* vp = vts + (d * 32 + lq) * VLD + 4 * half;
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int mf = 0; mf < 2; ++mf) {
+                    const uint2 lo = *(const uint2*)(vp + sub * 32 + 16 * mf);
+                    const uint2 hi = *(const uint2*)(vp + sub * 32 + 16 * mf + 8);
+                    const uint4 a = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&a,
+                                                                   *(const bf16x8_t*)&pb[sub][mf],
+                                                                   o[d], 0, 0, 0);
+                }
+        }
+    }
+    l += __shfl_xor(l, 32, ILLM_WAVE);
+    if (q < len) {
+        const float inv = 1.0f / l;
+        bf16_t* op = out + (size_t)(start + q) * nh * HD + (size_t)h * HD + 4 * half;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; ++b4) {
+                uint2 v;
+                v.x = pack_bf16x2(o[d][4 * b4 + 0] * inv, o[d][4 * b4 + 1] * inv);
+                v.y = pack_bf16x2(o[d][4 * b4 + 2] * inv, o[d][4 * b4 + 3] * inv);
+                *(uint2*)(op + d * 32 + 8 * b4) = v;
+            }
+    }
+}
+
+template <int HD>
+static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_seqs, int max_len,
+                          int nh, int nkv, float scale, int window, hipStream_t st) {
+    const int n_qblk = (max_len + PF_BM - 1) / PF_BM;
+    const long long total = (long long)n_qblk * nh * n_seqs;
+    if (total > 0x7fffffffLL - 8) return ILLM_ERR_ARG;
+    const int blocks = (int)(((total + 7) / 8) * 8);
+    hipLaunchKernelGGL(attn_prefill_mfma_kernel<HD>, dim3(blocks), dim3(256), 0, st,
+                       (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
+                       scale * 1.44269504088896340736f, window, (int)total);
+    return illm_launch_status();
+}
+
+// Takes bfloat16 and head_dim in {32, 64, 96, 128, 160, 192, 224, 256}; else ILLM_ERR_ARG.
+extern "C" int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
+                                      int n_seqs, int max_len, int nh, int nkv, int hd,
+                                      float scale, int window, void* stream) {
+    if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
+        hd % 32)
+        return ILLM_ERR_ARG;
+    if (n_seqs == 0 || max_len == 0) return ILLM_OK;
+    hipStream_t st = (hipStream_t)stream;
+    switch (hd) {
+        case 32: return launch_prefill<32>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 64: return launch_prefill<64>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 96: return launch_prefill<96>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 128: return launch_prefill<128>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+    }
+}

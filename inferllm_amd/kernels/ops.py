@@ -225,6 +225,11 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
     _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_prefill: packed qkv rows")
     _need(nh % nkv == 0, "attn_prefill: heads must be a multiple of kv heads")
     out = torch.empty((T, nh * hd), dtype=qkv.dtype, device=qkv.device)
+    if qkv.dtype == torch.bfloat16 and hd % 32 == 0:
+        _check(_lib().illm_attn_prefill_bf16(
+            _p(qkv), _p(out), _p(cu_seqlens), n_seqs, max_len, nh, nkv, hd,
+            ctypes.c_float(scale), window, _stream()), f"attn_prefill_bf16 (head_dim {hd})")
+        return out
     _check(_lib().illm_attn_prefill_generic(
         _p(qkv), _p(out), _code(qkv), _p(cu_seqlens), n_seqs, max_len, nh, nkv, hd,
         ctypes.c_float(scale), window, _stream()), f"attn_prefill (head_dim {hd})")

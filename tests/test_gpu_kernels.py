@@ -172,6 +172,34 @@ def test_attn_prefill(dtype, nh, nkv, hd, lens, window):
     close(got, want, dtype, scale=2)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,lens,window", [
+    (4, 4, 128, [300, 129, 128, 1], 0), (8, 1, 64, [257, 64], 0), (3, 3, 96, [200], 0), (6, 2, 32, [127, 130], 0),
+    (2, 1, 160, [70], 0), (4, 2, 128, [400], 100), (2, 2, 64, [333, 5], 64), (5, 5, 224, [66], 0), (2, 2, 192, [129], 7)])
+def test_attn_prefill_mfma(nh, nkv, hd, lens, window):
+    """The matrix-core kernel over several blocks of 128 query rows and tiles of 64 keys."""
+    dtype = torch.bfloat16
+    T = sum(lens)
+    qkv = rnd(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=17)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    scale = 1.0 / math.sqrt(hd)
+    got = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), len(lens), max(lens), nh, nkv, hd, scale, window)
+    want = R.attn_prefill(qkv, cu, len(lens), max(lens), nh, nkv, hd, scale, window)
+    close(got, want, dtype, scale=2)
+
+
+def test_attn_prefill_finds_one_far_key():
+    """One early key is made to stand out for a late query: the output is that key's value."""
+    nh, nkv, hd, n = 2, 1, 128, 700
+    dtype = torch.bfloat16
+    qkv = rnd(n, (nh + 2 * nkv) * hd, dtype=dtype, seed=3)
+    view = qkv.view(n, nh + 2 * nkv, hd)
+    view[37, nh] = view[650, 1].float().mul(30).to(dtype)          # key 37 matches query row 650, head 1
+    cu = torch.tensor([0, n], dtype=torch.int32)
+    got = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), 1, n, nh, nkv, hd, 1.0, 0).cpu().view(n, nh, hd)
+    close(got[650, 1], view[37, nh + nkv], dtype)
+    assert not torch.allclose(got[30, 1].float(), view[37, nh + nkv].float(), atol=0.1)   # hidden from row 30
+
+
 def paged_case(dtype, nkv, hd, lens, page, ring=0, seed=3):
     """Random cache contents laid out through a shuffled page table."""
     B = len(lens)
