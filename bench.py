@@ -60,6 +60,8 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill (for profiles); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
@@ -117,6 +119,27 @@ def main() -> int:
             eng.free_slot(s)
         return batch * steps / dt, dt / steps * 1e3, mean_ctx
 
+    def prefill_run(T=2048, reps=3):
+        ids = torch.randint(0, cfg["vocab_size"], (T,), generator=g).tolist()
+        times = []
+        for i in range(reps):
+            s = eng.alloc_slot()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            logits = eng.step([StepEntry(s, ids, [T - 1])])
+            ops.argmax(logits).tolist()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            eng.free_slot(s)
+        pt = min(times[1:])
+        fl = prefill_flops(cfg, layers, T)
+        return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill_run(reps=max(3, args.steps))}), flush=True)
+        return 0
+
     tps, ms, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
     step_bytes = weight_bytes_per_step(cfg, layers, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, layers, esz)
     achieved = step_bytes / (ms * 1e-3) / 1e9
@@ -136,22 +159,7 @@ def main() -> int:
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
     if not args.no_points:
-        T = 2048
-        ids = torch.randint(0, cfg["vocab_size"], (T,), generator=g).tolist()
-        times = []
-        for i in range(3):
-            s = eng.alloc_slot()
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            logits = eng.step([StepEntry(s, ids, [T - 1])])
-            ops.argmax(logits).tolist()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t)
-            eng.free_slot(s)
-        pt = min(times[1:])
-        fl = prefill_flops(cfg, layers, T)
-        out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                          "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
+        out["prefill"] = prefill_run()
         b1, _, _ = decode_run(1, min(args.steps, 64), 4)
         b64, _, _ = decode_run(64, min(args.steps, 32), 4)
         out["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}

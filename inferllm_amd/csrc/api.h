@@ -70,6 +70,11 @@ int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache, const 
 int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
                           void* stream);
 
+// Tuning entry of the same product: rows of W per block 16 * ntb (ntb 1, 2, 4), u * 64 bytes
+// of a W row per wave iteration (u 4, 8), waves per block.
+int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M, int N,
+                              int K, int ntb, int u, int waves, void* stream);
+
 // out[b] = index of the largest logit of row b (lowest index on ties).
 int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream);
 

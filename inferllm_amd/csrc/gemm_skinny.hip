@@ -18,10 +18,10 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-#define SK_U 4   // k-steps (of 32) per wave iteration
-
-template <int MT, int NTB>
-__global__ void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+// U: k-steps (of 32) per wave iteration, i.e. U * 64 contiguous bytes of each W row.
+// MAXW: most waves a block may have (register budget: 512 / (MAXW / 4) per lane).
+template <int MT, int NTB, int SK_U, int MAXW>
+__global__ void __launch_bounds__(64 * MAXW) gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                    void* __restrict__ Y, int y_dt, int M, int N, int K) {
     extern __shared__ float red[];   // [waves][NTB * MT * 64 * 4]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -50,19 +50,28 @@ __global__ void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* _
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
     const int ksteps = (K + 31) / 32;
-    for (int s0 = wave * SK_U; s0 < ksteps; s0 += waves * SK_U) {
-        uint4 a[NTB][SK_U], b[MT][SK_U];
+    const int stride = waves * SK_U;
+    uint4 a[NTB][SK_U], b[MT][SK_U];
+    auto load = [&](int s0, uint4 (&aa)[NTB][SK_U], uint4 (&bb)[MT][SK_U]) {
 #pragma unroll
         for (int u = 0; u < SK_U; ++u) {
             const int k = (s0 + u) * 32 + q * 8;
             const bool ok = k < K;           // K is a multiple of 8: a lane's 8 values are all in or all out
 #pragma unroll
             for (int nt = 0; nt < NTB; ++nt)
-                a[nt][u] = ok ? *(const uint4*)(wrow[nt] + k) : make_uint4(0, 0, 0, 0);
+                aa[nt][u] = ok ? *(const uint4*)(wrow[nt] + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
-                b[mt][u] = ok ? *(const uint4*)(xrow[mt] + k) : make_uint4(0, 0, 0, 0);
+                bb[mt][u] = ok ? *(const uint4*)(xrow[mt] + k) : make_uint4(0, 0, 0, 0);
         }
+    };
+    int s0 = wave * SK_U;
+    if (s0 < ksteps) load(s0, a, b);
+    for (; s0 < ksteps; s0 += stride) {
+        // the next piece is on its way while this one is multiplied
+        uint4 an[NTB][SK_U], bn[MT][SK_U];
+        const bool more = s0 + stride < ksteps;
+        if (more) load(s0 + stride, an, bn);
 #pragma unroll
         for (int u = 0; u < SK_U; ++u)
 #pragma unroll
@@ -71,6 +80,15 @@ __global__ void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* _
                 for (int mt = 0; mt < MT; ++mt)
                     acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                         *(bf16x8_t*)&a[nt][u], *(bf16x8_t*)&b[mt][u], acc[nt][mt], 0, 0, 0);
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < SK_U; ++u) {
+#pragma unroll
+                for (int nt = 0; nt < NTB; ++nt) a[nt][u] = an[nt][u];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) b[mt][u] = bn[mt][u];
+            }
+        }
     }
     // acc[nt][mt][i] = Y[m = mt*16 + r][n = n_base + nt*16 + q*4 + i]
     constexpr int PER_WAVE = NTB * MT * 64 * 4;
@@ -113,14 +131,48 @@ __global__ void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* _
     }
 }
 
-template <int MT, int NTB>
+template <int MT, int NTB, int U>
 static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
                          int waves, hipStream_t st) {
+    // registers a lane needs: operands of two pieces in flight and the accumulators
+    constexpr int REGS = 2 * (NTB + MT) * U * 4 + NTB * MT * 4 + 40;
+    constexpr int MAXW = REGS <= 128 ? 16 : (REGS <= 256 ? 8 : 4);
+    waves = waves > MAXW ? MAXW : waves;
     const int blocks = (N + 16 * NTB - 1) / (16 * NTB);
     const size_t smem = waves > 1 ? (size_t)waves * NTB * MT * 64 * 4 * sizeof(float) : 0;
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB>), dim3(blocks), dim3(64 * waves), smem, st,
-                       (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW>), dim3(blocks), dim3(64 * waves), smem,
+                       st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K);
     return illm_launch_status();
+}
+
+static int clamp_waves(int w, int ntb, int mt, int u, int K) {
+    const int ksteps = (K + 31) / 32;
+    const int max_by_k = (ksteps + u - 1) / u;           // more waves than k pieces would idle
+    const int lds_cap = (64 * 1024) / (ntb * mt * 1024);
+    w = w > 16 ? 16 : w;
+    w = w > lds_cap ? lds_cap : w;
+    w = w > max_by_k ? max_by_k : w;
+    return w < 1 ? 1 : w;
+}
+
+// Tuning entry: the same product with the tile shape given: ntb in {1, 2, 4}, u in {4, 8},
+// waves per block (clamped to what LDS and K allow).  Used to choose the defaults below.
+extern "C" int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M,
+                                         int N, int K, int ntb, int u, int waves, void* stream) {
+    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
+        return ILLM_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int mt = (M + 15) / 16;
+    waves = clamp_waves(waves, ntb, mt, u, K);
+#define GO(MT_, NTB_, U_)                                                                     \
+    if (mt == MT_ && ntb == NTB_ && u == U_)                                                  \
+        return launch_skinny<MT_, NTB_, U_>(X, W, Y, y_dt, M, N, K, waves, st)
+    GO(1, 1, 4); GO(1, 2, 4); GO(1, 4, 4); GO(1, 1, 8); GO(1, 2, 8); GO(1, 4, 8);
+    GO(2, 1, 4); GO(2, 2, 4); GO(2, 4, 4); GO(2, 2, 8);
+    GO(3, 2, 4); GO(3, 4, 4);
+    GO(4, 1, 4); GO(4, 2, 4); GO(4, 4, 4);
+#undef GO
+    return ILLM_ERR_ARG;
 }
 
 // Takes bfloat16 X and W, M in 1..64, K a multiple of 8.  Otherwise ILLM_ERR_ARG.
@@ -128,21 +180,11 @@ extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int 
                                      int N, int K, void* stream) {
     if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
         return ILLM_ERR_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    const int ksteps = (K + 31) / 32;
-    const int max_by_k = (ksteps + SK_U - 1) / SK_U;     // more waves than k pieces would idle
-    auto pick = [&](int ntb, int mt) {
-        const int blocks = (N + 16 * ntb - 1) / (16 * ntb);
-        int w = (2048 + blocks - 1) / blocks;            // aim at ~2048 waves on the chip
-        const int lds_cap = (64 * 1024) / (ntb * mt * 1024);
-        w = w < 1 ? 1 : w;
-        w = w > 16 ? 16 : w;
-        w = w > lds_cap ? lds_cap : w;
-        w = w > max_by_k ? max_by_k : w;
-        return w < 1 ? 1 : w;
-    };
-    if (M <= 16) return launch_skinny<1, 2>(X, W, Y, y_dt, M, N, K, pick(2, 1), st);
-    if (M <= 32) return launch_skinny<2, 2>(X, W, Y, y_dt, M, N, K, pick(2, 2), st);
-    if (M <= 48) return launch_skinny<3, 2>(X, W, Y, y_dt, M, N, K, pick(2, 3), st);
-    return launch_skinny<4, 2>(X, W, Y, y_dt, M, N, K, pick(2, 4), st);
+    // measured on MI355X at the LLaMA-2-7B shapes: 16 W rows per block and about 1536 waves
+    // on the chip are best for M <= 16; wider row tiles only pay when X has many rows
+    const int ntb = M <= 16 ? 1 : 2, u = 4;
+    const int blocks = (N + 16 * ntb - 1) / (16 * ntb);
+    int waves = (1536 + blocks / 2) / blocks;
+    waves = waves < 1 ? 1 : waves;
+    return illm_gemm_skinny_bf16_cfg(X, W, Y, y_dt, M, N, K, ntb, u, waves, stream);
 }

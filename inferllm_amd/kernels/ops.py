@@ -180,7 +180,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     M, K = x.shape
     if M == 0:
         return torch.empty((0, w.shape[0]), dtype=out_dtype, device=x.device)
-    if skinny_fits(M, w.shape[0], K):
+    if skinny_fits(M, w.shape[0], K) and (M <= SKINNY_BEST_ROWS or out_dtype == torch.float32):
         return gemm_skinny_bf16(x, w, out_dtype)
     if out_dtype == torch.float32 and K % 8 == 0:
         # float32 results (logits) keep the accumulator's precision: 64 rows at a time
@@ -192,7 +192,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     return torch.matmul(x, w.t())
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64     # rows the few-rows kernel takes
+SKINNY_BEST_ROWS = 16    # up to here it beats the vendor GEMM (measured at the 7B shapes)
 
 
 def skinny_fits(M: int, N: int, K: int) -> bool:

@@ -115,16 +115,17 @@ def test_norm_feed_forward_and_block_parts(dtype):
     assert rel(out, P.swiglu_ffn(h.cpu(), w["g"], w["u"], w["d"])) < TOL[dtype]
 
 
-def test_decode_graph_replays_equal_eager_steps(tmp_path):
+@pytest.mark.parametrize("n_reqs", [3, 20])
+def test_decode_graph_replays_equal_eager_steps(tmp_path, n_reqs):
     """The same decode steps through the captured HIP graph (replayed many times, with other
     work and synchronisations between) and eagerly: every replay equals its eager step."""
     import inferllm_amd as I
     from tiny import TINY_B, make_model_dir, random_ids
     d = make_model_dir(tmp_path, TINY_B, seed=3, dtype=torch.bfloat16)
-    reqs = [random_ids(n, 320, n) for n in (30, 12, 50)]
+    reqs = [random_ids(n, 320, n) for n in ([30, 12, 50] + list(range(13, 30)))[:n_reqs]]
     outs = []
     for graphs in (True, False):
-        eng = I.Engine.from_pretrained(d, dtype="bfloat16", max_batch=4, use_graphs=graphs)
+        eng = I.Engine.from_pretrained(d, dtype="bfloat16", max_batch=n_reqs, use_graphs=graphs)
         slots = [eng.alloc_slot() for _ in reqs]
         eng.step([I.StepEntry(s, r[:10], []) for s, r in zip(slots, reqs)])
         seq = []
