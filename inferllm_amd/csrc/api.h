@@ -75,6 +75,10 @@ int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int y_dt, int M
 int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M, int N,
                               int K, int ntb, int u, int waves, void* stream);
 
+// Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny product.
+int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* Y, int y_dt, int M, int F,
+                                 int K, void* stream);
+
 // out[b] = index of the largest logit of row b (lowest index on ties).
 int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream);
 

@@ -20,21 +20,24 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // U: k-steps (of 32) per wave iteration, i.e. U * 64 contiguous bytes of each W row.
 // MAXW: most waves a block may have (register budget: 512 / (MAXW / 4) per lane).
-template <int MT, int NTB, int SK_U, int MAXW>
-__global__ void __launch_bounds__(64 * MAXW) gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                                   void* __restrict__ Y, int y_dt, int M, int N, int K) {
+// DUAL (with NTB == 2): W is [gate rows (N) | up rows (N)]; the block's two tiles are the same
+// 16 rows of each half and the result is silu(gate) * up, Y[M, N].
+template <int MT, int NTB, int SK_U, int MAXW, bool DUAL>
+__global__ void __launch_bounds__(64 * MAXW)
+gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                   void* __restrict__ Y, int y_dt, int M, int N, int K) {
     extern __shared__ float red[];   // [waves][NTB * MT * 64 * 4]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
     const int r = lane & 15, q = lane >> 4;
-    const int n_base = blockIdx.x * (16 * NTB);
+    const int n_base = blockIdx.x * (DUAL ? 16 : 16 * NTB);
 
     const bf16_t* wrow[NTB];
 #pragma unroll
     for (int nt = 0; nt < NTB; ++nt) {
-        int n = n_base + nt * 16 + r;
+        int n = n_base + (DUAL ? 0 : nt * 16) + r;
         n = n < N ? n : N - 1;
-        wrow[nt] = W + (size_t)n * K;
+        wrow[nt] = W + ((size_t)n + (DUAL ? (size_t)nt * N : 0)) * K;
     }
     const bf16_t* xrow[MT];
 #pragma unroll
@@ -101,47 +104,61 @@ __global__ void __launch_bounds__(64 * MAXW) gemm_skinny_kernel(const bf16_t* __
                     acc[nt][mt];
         __syncthreads();
     }
-    // every thread of the block sums some of the (nt, mt, lane) groups over the waves
-    for (int grp = threadIdx.x; grp < NTB * MT * 64; grp += blockDim.x) {
-        f32x4_t v;
-        int l2, nt, mt;
-        if (waves > 1) {
-            v = *(f32x4_t*)(red + grp * 4);
-            for (int w = 1; w < waves; ++w) {
-                const f32x4_t o = *(f32x4_t*)(red + (size_t)w * PER_WAVE + grp * 4);
-                v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3];
+    // every thread of the block sums some of the (mt, lane) groups over the waves, tile by tile
+    for (int grp = threadIdx.x; grp < MT * 64; grp += blockDim.x) {
+        const int l2 = grp & 63, mt = grp >> 6;
+        f32x4_t v[NTB];
+#pragma unroll
+        for (int nt = 0; nt < NTB; ++nt) {
+            if (waves > 1) {
+                const int e = ((nt * MT + mt) * 64 + l2) * 4;
+                v[nt] = *(f32x4_t*)(red + e);
+                for (int w = 1; w < waves; ++w) {
+                    const f32x4_t o = *(f32x4_t*)(red + (size_t)w * PER_WAVE + e);
+                    v[nt][0] += o[0]; v[nt][1] += o[1]; v[nt][2] += o[2]; v[nt][3] += o[3];
+                }
+            } else {
+                // one wave: thread == lane, and grp walks this lane's own mt tiles
+                v[nt] = acc[nt][0];
+#pragma unroll
+                for (int b2 = 1; b2 < MT; ++b2)
+                    if (b2 == mt) v[nt] = acc[nt][b2];
             }
-            l2 = grp & 63; mt = (grp >> 6) % MT; nt = (grp >> 6) / MT;
-        } else {
-            // one wave: thread == lane; walk this lane's own tiles
-            l2 = lane; mt = (grp >> 6) % MT; nt = (grp >> 6) / MT;
-            v = acc[0][0];
-#pragma unroll
-            for (int a2 = 0; a2 < NTB; ++a2)
-#pragma unroll
-                for (int b2 = 0; b2 < MT; ++b2)
-                    if (a2 == nt && b2 == mt) v = acc[a2][b2];
         }
         const int mrow = mt * 16 + (l2 & 15);
-        const int n0 = n_base + nt * 16 + (l2 >> 4) * 4;
         if (mrow >= M) continue;
+        if (DUAL) {
+            const int n0 = n_base + (l2 >> 4) * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[i]);
+            for (int i = 0; i < 4; ++i)
+                if (n0 + i < N) {
+                    const float g = v[0][i];
+                    st_f(Y, y_dt, (size_t)mrow * N + n0 + i, (g / (1.0f + expf(-g))) * v[NTB - 1][i]);
+                }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NTB; ++nt) {
+                const int n0 = n_base + nt * 16 + (l2 >> 4) * 4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[nt][i]);
+            }
+        }
     }
 }
 
-template <int MT, int NTB, int U>
+template <int MT, int NTB, int U, bool DUAL = false>
 static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
                          int waves, hipStream_t st) {
     // registers a lane needs: operands of two pieces in flight and the accumulators
     constexpr int REGS = 2 * (NTB + MT) * U * 4 + NTB * MT * 4 + 40;
     constexpr int MAXW = REGS <= 128 ? 16 : (REGS <= 256 ? 8 : 4);
     waves = waves > MAXW ? MAXW : waves;
-    const int blocks = (N + 16 * NTB - 1) / (16 * NTB);
+    const int rows_per_block = DUAL ? 16 : 16 * NTB;
+    const int blocks = (N + rows_per_block - 1) / rows_per_block;
     const size_t smem = waves > 1 ? (size_t)waves * NTB * MT * 64 * 4 * sizeof(float) : 0;
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW>), dim3(blocks), dim3(64 * waves), smem,
-                       st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, DUAL>), dim3(blocks), dim3(64 * waves),
+                       smem, st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K);
     return illm_launch_status();
 }
 
@@ -187,4 +204,23 @@ extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int 
     int waves = (1536 + blocks / 2) / blocks;
     waves = waves < 1 ? 1 : waves;
     return illm_gemm_skinny_bf16_cfg(X, W, Y, y_dt, M, N, K, ntb, u, waves, stream);
+}
+
+// Y[M, F] = silu(X . Wg^T) * (X . Wu^T) with W = [Wg (F rows) | Wu (F rows)], [2F, K]:
+// the gate and up products and the SiLU-multiply in one kernel (src/core/graph.cpp:57-79).
+extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* Y, int y_dt, int M,
+                                            int F, int K, void* stream) {
+    if (M <= 0 || M > 64 || F <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
+        return ILLM_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int mt = (M + 15) / 16;
+    const int blocks = (F + 15) / 16;
+    int waves = (1536 + blocks / 2) / blocks;
+    waves = clamp_waves(waves < 1 ? 1 : waves, 2, mt, 4, K);
+    switch (mt) {
+        case 1: return launch_skinny<1, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 2: return launch_skinny<2, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 3: return launch_skinny<3, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
+        default: return launch_skinny<4, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
+    }
 }

@@ -216,6 +216,23 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -
     return y
 
 
+def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(x . Wg^T) * (x . Wu^T) for w_gate_up = [Wg | Wu] stacked as [2F, K].
+
+    Few bfloat16 rows: one fused MFMA kernel.  Otherwise the product and `silu_mul`."""
+    M, K = x.shape
+    F2 = w_gate_up.shape[0]
+    if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and F2 % 2 == 0
+            and 1 <= M <= SKINNY_BEST_ROWS and K % 8 == 0):
+        _gpu(x, w_gate_up)
+        _need(w_gate_up.dim() == 2 and w_gate_up.shape[1] == K, "gate_up_silu: shapes")
+        y = torch.empty((M, F2 // 2), dtype=x.dtype, device=x.device)
+        _check(_lib().illm_gemm_skinny_gateup_silu(_p(x), _p(w_gate_up), _p(y), _code(y), M,
+                                                   F2 // 2, K, _stream()), "gate_up_silu")
+        return y
+    return silu_mul(linear(x, w_gate_up))
+
+
 # ------------------------------------------------------------------ attention
 def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_len: int, nh: int,
                  nkv: int, hd: int, scale: float, window: int) -> torch.Tensor:
@@ -240,7 +257,7 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
 def decode_splits(B: int, nh: int, max_len: int) -> int:
     """How many ways to cut the keys of a decode step so that the launch fills the chip."""
     blocks = max(1, B * nh)
-    want = max(1, -(-1024 // blocks))
+    want = max(1, -(-2048 // blocks))
     tiles = max(1, (max_len + 63) // 64)
     return max(1, min(want, tiles, 32))
 

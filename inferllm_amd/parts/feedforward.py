@@ -35,5 +35,4 @@ class SwiGLU(FeedForward):
         self.w_down = self._take(tensors, "down").contiguous()
 
     def forward(self, h, ctx: StepContext):
-        gu = ops.linear(h, self.w_gate_up)
-        return ops.linear(ops.silu_mul(gu), self.w_down)
+        return ops.linear(ops.gate_up_silu(h, self.w_gate_up), self.w_down)

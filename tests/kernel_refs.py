@@ -83,6 +83,10 @@ def linear(x, w, out_dtype=None):
     return (x.to(F64) @ w.to(F64).t()).to(out_dtype or x.dtype)
 
 
+def gate_up_silu(x, w_gate_up):
+    return silu_mul(linear(x, w_gate_up))
+
+
 def gemm_generic(x, w, out_dtype):
     return linear(x, w, out_dtype)
 
@@ -187,6 +191,6 @@ def sample(logits, temperature, top_k, top_p, repeat_penalty, last_tokens, seeds
 def patch(monkeypatch):
     """Put these functions in place of the GPU ops (CPU tests only)."""
     from inferllm_amd.kernels import ops
-    for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic",
+    for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic", "gate_up_silu",
                  "attn_prefill", "decode_splits", "attn_decode", "argmax", "sample"):
         monkeypatch.setattr(ops, name, globals()[name])

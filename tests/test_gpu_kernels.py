@@ -277,6 +277,18 @@ def test_gemm_skinny(ydt, M, N, K):
         torch.testing.assert_close(got.double().cpu(), R.linear(x, w, torch.float64), atol=2e-4 * math.sqrt(K), rtol=1e-4)
 
 
+@pytest.mark.parametrize("M,F,K", [(1, 11008, 4096), (8, 172, 64), (16, 200, 80), (3, 33, 1000), (40, 50, 64)])
+def test_gate_up_silu(M, F, K):
+    x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * F, K, dtype=torch.bfloat16, seed=2, std=0.2)
+    got = ops().gate_up_silu(x.to(DEV), w.to(DEV))
+    g, u = R.linear(x, w[:F], torch.float64), R.linear(x, w[F:], torch.float64)
+    want = g / (1 + torch.exp(-g)) * u
+    close(got, want, torch.bfloat16, scale=max(1.0, float(want.abs().max())))
+    swapped = u / (1 + torch.exp(-u)) * g
+    assert not torch.allclose(got.double().cpu(), swapped, atol=0.1 * float(want.abs().max()))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attn_decode_finds_one_far_key(dtype):
     """One key among hundreds is made to stand out: the output must be its value."""
