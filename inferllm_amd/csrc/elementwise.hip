@@ -164,9 +164,38 @@ __global__ void silu_mul_kernel(const void* __restrict__ gu, void* __restrict__ 
     st_f(out, dt, t * F + f, (g / (1.0f + expf(-g))) * u);
 }
 
+// bfloat16 rows with F % 8 == 0: 8 values (16 bytes) of gate and of up per thread
+__global__ void __launch_bounds__(256)
+silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int F) {
+    const size_t t = blockIdx.y;
+    const int f = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (f >= F) return;
+    const uint4 g = *(const uint4*)(gu + t * 2 * F + f);
+    const uint4 u = *(const uint4*)(gu + t * 2 * F + F + f);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+        const float r0 = (g0 / (1.0f + expf(-g0))) * u0, r1 = (g1 / (1.0f + expf(-g1))) * u1;
+        ow[i] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+    }
+    *(uint4*)(out + t * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* stream) {
     if (T < 0 || F <= 0 || !illm_dtype_ok(dt)) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
+    if (dt == ILLM_BF16 && F % 8 == 0) {
+        for (int t0 = 0; t0 < T; t0 += 65535) {
+            const int rows = T - t0 < 65535 ? T - t0 : 65535;
+            hipLaunchKernelGGL(silu_mul_bf16x8_kernel, dim3((F / 8 + 255) / 256, rows), dim3(256), 0,
+                               (hipStream_t)stream, (const bf16_t*)gate_up + (size_t)t0 * 2 * F,
+                               (bf16_t*)out + (size_t)t0 * F, F);
+        }
+        return illm_launch_status();
+    }
     // gridDim.y is limited to 65535: rows beyond that go in further launches
     for (int t0 = 0; t0 < T; t0 += 65535) {
         const int rows = T - t0 < 65535 ? T - t0 : 65535;
@@ -235,6 +264,59 @@ __global__ void rope_store_kernel(void* __restrict__ qkv, int dt,
     }
 }
 
+// bfloat16, pairs (i, i + hd/2), all of the head rotated (rot == hd), hd % 16 == 0: one block
+// per row; a thread rotates 8 pairs at a time with 16-byte loads, then the row's k and v
+// heads are copied to the cache 16 bytes at a time.
+__global__ void __launch_bounds__(256)
+rope_store_bf16_kernel(bf16_t* __restrict__ qkv, const float* __restrict__ cos_sin,
+                       const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_slot,
+                       const int32_t* __restrict__ slot_len, bf16_t* __restrict__ kcache,
+                       bf16_t* __restrict__ vcache, const int32_t* __restrict__ page_table,
+                       int table_stride, int page_size, int ring, int nh, int nkv, int hd) {
+    const int t = blockIdx.x;
+    const int pos = row_pos[t];
+    bf16_t* row = qkv + (size_t)t * (size_t)(nh + 2 * nkv) * hd;
+    const int half = hd / 2, cpu8 = half / 8;             // chunks of 8 pairs per head
+    if (cos_sin) {
+        const float* cs = cos_sin + (size_t)pos * hd;     // [hd/2][2]
+        for (int u = threadIdx.x; u < (nh + nkv) * cpu8; u += 256) {
+            const int h = u / cpu8, i0 = (u - h * cpu8) * 8;
+            bf16_t* p = row + (size_t)h * hd + i0;
+            const uint4 a = *(const uint4*)p, b = *(const uint4*)(p + half);
+            const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+            uint32_t ao[4], bo[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 c = *(const float4*)(cs + 2 * (i0 + 2 * j));   // cos, sin, cos, sin
+                const float x0 = __uint_as_float(aw[j] << 16), x1 = __uint_as_float(aw[j] & 0xffff0000u);
+                const float y0 = __uint_as_float(bw[j] << 16), y1 = __uint_as_float(bw[j] & 0xffff0000u);
+                ao[j] = (uint32_t)f32_to_bf16(x0 * c.x - y0 * c.y) |
+                        ((uint32_t)f32_to_bf16(x1 * c.z - y1 * c.w) << 16);
+                bo[j] = (uint32_t)f32_to_bf16(x0 * c.y + y0 * c.x) |
+                        ((uint32_t)f32_to_bf16(x1 * c.w + y1 * c.z) << 16);
+            }
+            *(uint4*)p = make_uint4(ao[0], ao[1], ao[2], ao[3]);
+            *(uint4*)(p + half) = make_uint4(bo[0], bo[1], bo[2], bo[3]);
+        }
+    }
+    if (kcache == nullptr) return;
+    const int slot = row_slot[t];
+    if (ring > 0) {
+        const int last_page = (slot_len[slot] - 1) / page_size;
+        if (pos / page_size + ring <= last_page) return;
+    }
+    __syncthreads();
+    const int c8 = hd / 8;
+    for (int u = threadIdx.x; u < 2 * nkv * c8; u += 256) {
+        const int which = u / (nkv * c8), r = u - which * nkv * c8;
+        const int kvh = r / c8, off = (r - kvh * c8) * 8;
+        const size_t dst = cache_row_offset(page_table, table_stride, slot, pos, page_size, ring, nkv,
+                                            kvh, hd) + off;
+        const bf16_t* src = row + (size_t)(nh + which * nkv + kvh) * hd + off;
+        *(uint4*)((which ? vcache : kcache) + dst) = *(const uint4*)src;
+    }
+}
+
 extern "C" int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_pos, int rot,
                                int pairing, const int32_t* row_pos, const int32_t* row_slot,
                                const int32_t* slot_len, void* kcache, void* vcache,
@@ -248,6 +330,12 @@ extern "C" int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_
     if (ring > 0 && !slot_len) return ILLM_ERR_ARG;
     if (nh + nkv > 65535) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
+    if (dt == ILLM_BF16 && hd % 16 == 0 && (!cos_sin || (pairing == 0 && rot == hd))) {
+        hipLaunchKernelGGL(rope_store_bf16_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream,
+                           (bf16_t*)qkv, cos_sin, row_pos, row_slot, slot_len, (bf16_t*)kcache,
+                           (bf16_t*)vcache, page_table, table_stride, page_size, ring, nh, nkv, hd);
+        return illm_launch_status();
+    }
     hipLaunchKernelGGL(rope_store_kernel, dim3(T, nh + nkv), dim3(64), 0, (hipStream_t)stream, qkv,
                        dt, cos_sin, rot, pairing, row_pos, row_slot, slot_len, kcache, vcache,
                        page_table, table_stride, page_size, ring, nh, nkv, hd);

@@ -67,7 +67,7 @@ def test_add_rmsnorm(out_dtype, w_dtype, T, E, eps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,F", [(4, 10), (5, 130), (3, 11008), (1, 173)])
+@pytest.mark.parametrize("T,F", [(4, 10), (5, 130), (3, 11008), (1, 173), (70, 64), (2, 2056)])
 def test_silu_mul(dtype, T, F):
     gu = rnd(T, 2 * F, dtype=dtype, std=3.0)
     gu[0, 0] = 0.0; gu[0, 1] = -60.0; gu[0, 2] = 40.0
@@ -81,7 +81,7 @@ def make_cache(n_pages, nkv, page, hd, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,hd,rot,pairing", [(4, 2, 24, 24, 0), (3, 3, 16, 16, 1), (8, 1, 128, 128, 0),
-                                                    (5, 5, 48, 32, 0), (2, 1, 256, 256, 1)])
+                                                    (5, 5, 48, 32, 0), (2, 1, 256, 256, 1), (32, 8, 64, 64, 0), (3, 1, 48, 48, 0), (2, 2, 32, 16, 0)])
 def test_rope_store(dtype, nh, nkv, hd, rot, pairing):
     from inferllm_amd.parts.position import rotary_table
     page, max_pos = 8, 64
