@@ -155,10 +155,10 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
             if (q == 0 && dim_ok) {
                 const float inv = 1.0f / l[g];
                 uint4 o;
-                o.x = (uint32_t)f32_to_bf16(acc[g][0] * inv) | ((uint32_t)f32_to_bf16(acc[g][1] * inv) << 16);
-                o.y = (uint32_t)f32_to_bf16(acc[g][2] * inv) | ((uint32_t)f32_to_bf16(acc[g][3] * inv) << 16);
-                o.z = (uint32_t)f32_to_bf16(acc[g][4] * inv) | ((uint32_t)f32_to_bf16(acc[g][5] * inv) << 16);
-                o.w = (uint32_t)f32_to_bf16(acc[g][6] * inv) | ((uint32_t)f32_to_bf16(acc[g][7] * inv) << 16);
+                o.x = pack_bf16x2(acc[g][0] * inv, acc[g][1] * inv);
+                o.y = pack_bf16x2(acc[g][2] * inv, acc[g][3] * inv);
+                o.z = pack_bf16x2(acc[g][4] * inv, acc[g][5] * inv);
+                o.w = pack_bf16x2(acc[g][6] * inv, acc[g][7] * inv);
                 *(uint4*)(out + ((size_t)b * nh + h) * hd + c * 8) = o;
             }
         } else {

@@ -13,9 +13,11 @@
 // read once into registers.  Scores and statistics are float32; exponentials are
 // base 2 with log2(e) folded into the scale.
 //
-// Blocks are numbered so that the query blocks of one (sequence, head) run on the
-// same XCD (consecutive block ids go round the 8 XCDs) and share K and V in its L2,
-// heaviest (last) query blocks first.
+// The next tile's K and V are on their way from global memory (into registers) while the
+// current tile is multiplied.  Blocks are numbered so that the query blocks of one
+// (sequence, head) run on the same XCD (consecutive block ids go round the 8 XCDs) and
+// share K and V in its L2, and so that every XCD starts with its heaviest (last) query
+// blocks and ends with the middle ones.
 //
 // The chain is src/core/op.cpp:485-498 (scores, scale + mask, softmax, context) with
 // grouped heads as src/kern/naive/naive.cpp:576-604.
@@ -31,15 +33,11 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 #define PF_BM 128     // query rows per block
 #define NEG_INF (-INFINITY)
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
-}
-
 template <int HD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, (HD <= 128 ? 2 : 1))
 attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
                          const int32_t* __restrict__ cu, int n_qblk, int nh, int nkv,
-                         float scale_log2, int window, int total_work) {
+                         float scale_log2, int window, int hb_per_xcd, int n_hb, int zigzag) {
     constexpr int KLD = HD + 8;        // K tile row stride: 16 bytes of padding
     constexpr int VLD = PF_BN + 4;     // V^T row stride
     constexpr int KS = HD / 16;        // k-steps of the first product
@@ -47,11 +45,16 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     __shared__ __attribute__((aligned(16))) bf16_t ks[PF_BN * KLD];
     __shared__ __attribute__((aligned(16))) bf16_t vts[HD * VLD];
 
-    const int per_xcd = (total_work + 7) / 8;
-    const int w = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (w >= total_work) return;
-    const int qb = n_qblk - 1 - (w % n_qblk);
-    const int hb = w / n_qblk;
+    // XCD x takes the (sequence, head) pairs [x * hb_per_xcd, (x + 1) * hb_per_xcd); within
+    // it, slots run over those pairs first and over query blocks, last block first, second
+    const int xcd = blockIdx.x % 8, slot_id = blockIdx.x / 8;
+    const int hb = xcd * hb_per_xcd + slot_id % hb_per_xcd;
+    if (hb >= n_hb) return;
+    // heavy half first (last query blocks, descending), then the light half ascending: when
+    // all blocks are resident at once, the blocks that share a CU add up to about the same
+    // (`zigzag`); with more blocks than fit at once, plain heaviest-first is better
+    const int qi = slot_id / hb_per_xcd, top = zigzag ? (n_qblk + 1) / 2 : n_qblk;
+    const int qb = qi < top ? n_qblk - 1 - qi : qi - top;
     const int h = hb % nh, b = hb / nh;
     const int start = cu[b], len = cu[b + 1] - start;
     const int q0 = qb * PF_BM;
@@ -83,18 +86,30 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     const int wk_end = min(len, q_row0 + 32);                       // this wave's last key + 1
     const int wk_begin = window > 0 ? max(0, q_row0 - window + 1) : 0;
 
-    for (int k0 = k_begin; k0 < k_end; k0 += PF_BN) {
-        __syncthreads();
-        // K tile as it is, V tile transposed; a wave instruction covers 16 keys x 4 chunks
+    constexpr int NLD = (PF_BN * HD / 8) / 256;     // 16-byte pieces of K (and of V) per thread
+    uint4 kpre[NLD], vpre[NLD];
+    auto fetch = [&](int k0) {
 #pragma unroll
-        for (int it = 0; it < (PF_BN * HD / 8) / 256; ++it) {
+        for (int it = 0; it < NLD; ++it) {
             const int u = tid + it * 256;
             const int key = ((u >> 6) & 3) * 16 + (u & 15);
             const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
             const int krow = min(k0 + key, len - 1);
             const bf16_t* src = qkv + (size_t)(start + krow) * rowlen;
-            const uint4 kv = *(const uint4*)(src + (size_t)(nh + kvh) * HD + ch * 8);
-            const uint4 vv = *(const uint4*)(src + (size_t)(nh + nkv + kvh) * HD + ch * 8);
+            kpre[it] = *(const uint4*)(src + (size_t)(nh + kvh) * HD + ch * 8);
+            vpre[it] = *(const uint4*)(src + (size_t)(nh + nkv + kvh) * HD + ch * 8);
+        }
+    };
+    if (k_begin < k_end) fetch(k_begin);
+    for (int k0 = k_begin; k0 < k_end; k0 += PF_BN) {
+        __syncthreads();
+        // K tile as it is, V tile transposed; a wave instruction covers 16 keys x 4 chunks
+#pragma unroll
+        for (int it = 0; it < NLD; ++it) {
+            const int u = tid + it * 256;
+            const int key = ((u >> 6) & 3) * 16 + (u & 15);
+            const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
+            const uint4 kv = kpre[it], vv = vpre[it];
             *(uint4*)(ks + key * KLD + ch * 8) = kv;
             bf16_t* vd = vts + (ch * 8) * VLD + key;
             vd[0 * VLD] = (bf16_t)(vv.x & 0xffffu); vd[1 * VLD] = (bf16_t)(vv.x >> 16);
@@ -103,6 +118,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
             vd[6 * VLD] = (bf16_t)(vv.w & 0xffffu); vd[7 * VLD] = (bf16_t)(vv.w >> 16);
         }
         __syncthreads();
+        if (k0 + PF_BN < k_end) fetch(k0 + PF_BN);
         if (k0 >= wk_end || k0 + PF_BN <= wk_begin) continue;       // nothing visible to this wave
 
         // S^T[key][q] for two sub-tiles of 32 keys
@@ -159,10 +175,12 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
         }
         l = l * alpha + rs;
         m = m_new;
+        if (__any(alpha != 1.f)) {          // the running max moved for some query of the wave
 #pragma unroll
-        for (int d = 0; d < DB; ++d)
+            for (int d = 0; d < DB; ++d)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+                for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+        }
         // O^T[d][q] += V^T[d][keys] . P^T[keys][q]
 #pragma unroll
         for (int d = 0; d < DB; ++d) {
@@ -200,12 +218,14 @@ template <int HD>
 static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_seqs, int max_len,
                           int nh, int nkv, float scale, int window, hipStream_t st) {
     const int n_qblk = (max_len + PF_BM - 1) / PF_BM;
-    const long long total = (long long)n_qblk * nh * n_seqs;
-    if (total > 0x7fffffffLL - 8) return ILLM_ERR_ARG;
-    const int blocks = (int)(((total + 7) / 8) * 8);
-    hipLaunchKernelGGL(attn_prefill_mfma_kernel<HD>, dim3(blocks), dim3(256), 0, st,
+    const long long n_hb = (long long)nh * n_seqs;
+    const long long hb_per_xcd = (n_hb + 7) / 8;
+    const long long blocks = 8 * hb_per_xcd * n_qblk;
+    if (blocks > 0x7fffffffLL) return ILLM_ERR_ARG;
+    hipLaunchKernelGGL(attn_prefill_mfma_kernel<HD>, dim3((unsigned)blocks), dim3(256), 0, st,
                        (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
-                       scale * 1.44269504088896340736f, window, (int)total);
+                       scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
+                       hb_per_xcd * n_qblk <= 64 ? 1 : 0);   // 32 CUs of an XCD, two blocks each
     return illm_launch_status();
 }
 

@@ -19,12 +19,19 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
 
-// round to nearest even; NaN stays NaN
+typedef __bf16 illm_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float illm_f32x2_t __attribute__((ext_vector_type(2)));
+
+// two floats to two bfloat16 (a in the low half), round to nearest even, by the
+// hardware's packed conversion (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    const illm_f32x2_t v = {a, b};
+    const illm_bf16x2_t r = __builtin_convertvector(v, illm_bf16x2_t);
+    return *(const uint32_t*)&r;
+}
+
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+    return (bf16_t)(pack_bf16x2(f, 0.f) & 0xffffu);
 }
 
 __device__ __forceinline__ float ld_f(const void* p, int dt, size_t i) {

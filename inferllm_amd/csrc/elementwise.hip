@@ -75,8 +75,8 @@ __device__ __forceinline__ float4 ld4_f(const void* p, int dt, size_t i4) {
 __device__ __forceinline__ void st4_f(void* p, int dt, size_t i4, float4 v) {
     if (dt == ILLM_BF16) {
         uint2 u;
-        u.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
-        u.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+        u.x = pack_bf16x2(v.x, v.y);
+        u.y = pack_bf16x2(v.z, v.w);
         ((uint2*)p)[i4] = u;
     } else {
         ((float4*)p)[i4] = v;
@@ -179,7 +179,7 @@ silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, 
         const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
         const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
         const float r0 = (g0 / (1.0f + expf(-g0))) * u0, r1 = (g1 / (1.0f + expf(-g1))) * u1;
-        ow[i] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+        ow[i] = pack_bf16x2(r0, r1);
     }
     *(uint4*)(out + t * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
 }
@@ -290,10 +290,8 @@ rope_store_bf16_kernel(bf16_t* __restrict__ qkv, const float* __restrict__ cos_s
                 const float4 c = *(const float4*)(cs + 2 * (i0 + 2 * j));   // cos, sin, cos, sin
                 const float x0 = __uint_as_float(aw[j] << 16), x1 = __uint_as_float(aw[j] & 0xffff0000u);
                 const float y0 = __uint_as_float(bw[j] << 16), y1 = __uint_as_float(bw[j] & 0xffff0000u);
-                ao[j] = (uint32_t)f32_to_bf16(x0 * c.x - y0 * c.y) |
-                        ((uint32_t)f32_to_bf16(x1 * c.z - y1 * c.w) << 16);
-                bo[j] = (uint32_t)f32_to_bf16(x0 * c.y + y0 * c.x) |
-                        ((uint32_t)f32_to_bf16(x1 * c.w + y1 * c.z) << 16);
+                ao[j] = pack_bf16x2(x0 * c.x - y0 * c.y, x1 * c.z - y1 * c.w);
+                bo[j] = pack_bf16x2(x0 * c.y + y0 * c.x, x1 * c.w + y1 * c.z);
             }
             *(uint4*)p = make_uint4(ao[0], ao[1], ao[2], ao[3]);
             *(uint4*)(p + half) = make_uint4(bo[0], bo[1], bo[2], bo[3]);
