@@ -175,24 +175,26 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     }
 }
 
-// grid (heads, sequences): combine the splits (same as the generic path's merge)
-__global__ void attn_decode_bf16_merge_kernel(const float* __restrict__ partial,
-                                              bf16_t* __restrict__ out, int nsplit, int nh, int hd) {
-    const int h = blockIdx.x, b = blockIdx.y;
+// grid (heads, sequences), one wave: lane s holds split s's max and sum (nsplit <= 64), the
+// weights are formed once, and splits that saw no key are skipped.
+__global__ void __launch_bounds__(64)
+attn_decode_bf16_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
+                              int nsplit, int nh, int hd) {
+    const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
     const float* pp = partial + ((size_t)b * nh + h) * nsplit * (size_t)(hd + 2);
-    float m = NEG_INF;
-    for (int s = 0; s < nsplit; ++s) m = fmaxf(m, pp[(size_t)s * (hd + 2) + hd]);
-    float L = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float ms = pp[(size_t)s * (hd + 2) + hd];
-        if (ms != NEG_INF) L += expf(ms - m) * pp[(size_t)s * (hd + 2) + hd + 1];
+    float ms = NEG_INF, ls = 0.f;
+    if (lane < nsplit) {
+        ms = pp[(size_t)lane * (hd + 2) + hd];
+        ls = pp[(size_t)lane * (hd + 2) + hd + 1];
     }
-    const float inv = 1.0f / L;
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    const float m = wave_max(ms);
+    const float w = (ms == NEG_INF) ? 0.f : expf(ms - m);
+    const float inv = 1.0f / wave_sum(w * ls);
+    for (int d = lane; d < hd; d += 64) {
         float a = 0.f;
         for (int s = 0; s < nsplit; ++s) {
-            const float ms = pp[(size_t)s * (hd + 2) + hd];
-            if (ms != NEG_INF) a += expf(ms - m) * pp[(size_t)s * (hd + 2) + d];
+            const float ws = __shfl(w, s, ILLM_WAVE);
+            if (ws != 0.f) a = fmaf(ws, pp[(size_t)s * (hd + 2) + d], a);
         }
         out[((size_t)b * nh + h) * hd + d] = f32_to_bf16(a * inv);
     }
@@ -244,7 +246,7 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
                                      float* partial, int nsplit, int B, int nh, int nkv, int hd,
                                      float scale, int window, void* stream) {
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 || hd % 8 ||
-        page_size <= 0 || page_size % 64 || nsplit <= 0 || nsplit > 65535 || B > 65535 ||
+        page_size <= 0 || page_size % 64 || nsplit <= 0 || nsplit > 64 || B > 65535 ||
         table_stride <= 0 || (nsplit > 1 && !partial))
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;

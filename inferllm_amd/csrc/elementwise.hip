@@ -83,8 +83,8 @@ __device__ __forceinline__ void st4_f(void* p, int dt, size_t i4, float4 v) {
     }
 }
 
-template <int NV>
-__global__ void __launch_bounds__(256)
+template <int NV, int TH>
+__global__ void __launch_bounds__(TH)
 add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, int delta_dt,
                        const void* __restrict__ w, int w_dt, void* __restrict__ out, int out_dt,
                        const int32_t* __restrict__ row_idx, int E, float eps) {
@@ -96,7 +96,7 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
     float4 v[NV], wv[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-        const int i = threadIdx.x + 256 * j;
+        const int i = threadIdx.x + TH * j;
         v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
         wv[j] = v[j];
         if (i < E4) {
@@ -107,7 +107,7 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
     if (delta) {
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
-            const int i = threadIdx.x + 256 * j;
+            const int i = threadIdx.x + TH * j;
             if (i < E4) {
                 const float4 d = ld4_f(delta, delta_dt, ib + i);
                 v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
@@ -123,7 +123,7 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
     const float scale = 1.0f / sqrtf(ss / (float)E + eps);
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-        const int i = threadIdx.x + 256 * j;
+        const int i = threadIdx.x + TH * j;
         if (i < E4)
             st4_f(out, out_dt, ob + i,
                   make_float4((v[j].x * scale) * wv[j].x, (v[j].y * scale) * wv[j].y,
@@ -139,13 +139,17 @@ extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const
         return ILLM_ERR_ARG;
     if (rows == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
-#define VEC(NV_)                                                                              \
-    hipLaunchKernelGGL(add_rmsnorm_vec_kernel<NV_>, dim3(rows), dim3(256), 0, st, x, delta,   \
-                       delta_dt, w, w_dt, out, out_dt, row_idx, E, eps)
-    if (E % 4 == 0 && E <= 1024) VEC(1);
-    else if (E % 4 == 0 && E <= 2048) VEC(2);
-    else if (E % 4 == 0 && E <= 4096) VEC(4);
-    else if (E % 4 == 0 && E <= 8192) VEC(8);
+#define VEC(NV_, TH_)                                                                         \
+    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV_, TH_>), dim3(rows), dim3(TH_), 0, st, x,   \
+                       delta, delta_dt, w, w_dt, out, out_dt, row_idx, E, eps)
+    // few rows (decoding): wide blocks, one group of 4 floats per thread, to shorten the row's
+    // critical path; many rows: narrow blocks so that more rows are in flight per CU
+    if (E % 4 == 0 && rows <= 128 && E > 1024 && E <= 4096) VEC(1, 1024);
+    else if (E % 4 == 0 && rows <= 128 && E > 4096 && E <= 8192) VEC(2, 1024);
+    else if (E % 4 == 0 && E <= 1024) VEC(1, 256);
+    else if (E % 4 == 0 && E <= 2048) VEC(2, 256);
+    else if (E % 4 == 0 && E <= 4096) VEC(4, 256);
+    else if (E % 4 == 0 && E <= 8192) VEC(8, 256);
     else
         hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, delta, delta_dt, w,
                            w_dt, out, out_dt, row_idx, E, eps);
