@@ -362,3 +362,43 @@ def test_sample_frequencies_match_probabilities():
     p = torch.softmax(row.double() / 0.9, 0)
     chi2 = float((n * (freq - p) ** 2 / p).sum())
     assert chi2 < 30.0, (chi2, freq, p)           # 6 degrees of freedom: far beyond any honest draw
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd", [32, 24])
+def test_window_edge_prefill_and_decode(dtype, hd):
+    """A key that stands out sits exactly at the window's edge: the query `window - 1` places
+    after it still sees it, the next query does not (prefill), and likewise for a single new
+    token over the cache (decode)."""
+    nh, nkv, n, window, edge = 2, 2, 150, 40, 70
+    qkv = rnd(n, (nh + 2 * nkv) * hd, dtype=dtype, seed=5, std=0.3)
+    view = qkv.view(n, nh + 2 * nkv, hd)
+    probe = rnd(hd, seed=6).to(dtype)
+    view[:, 0] = probe                                   # every query of head 0 looks for the probe
+    view[edge, nh] = probe.float().mul(25).to(dtype)     # and key `edge` answers it loudly
+    view[edge, nh + nkv] = 7.0                           # its value is unmistakable
+    cu = torch.tensor([0, n], dtype=torch.int32)
+    out = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), 1, n, nh, nkv, hd, 1.0, window).cpu().view(n, nh, hd).float()
+    last_seeing = edge + window - 1
+    assert float(out[last_seeing, 0].mean()) > 6.5       # still inside the window
+    assert float(out[last_seeing + 1, 0].mean()) < 3.0   # one step further: gone
+    assert float(out[edge - 1, 0].mean()) < 3.0          # and the future is hidden
+    want = R.attn_prefill(qkv, cu, 1, n, nh, nkv, hd, 1.0, window)
+    close(out.reshape(n, -1), want, dtype, scale=8)
+    # decode: cache holds keys 0..L-1 (the last one is the new token's)
+    page = 64
+    ring = (window + page - 2) // page + 1
+    for L, sees in ((edge + window, True), (edge + window + 1, False)):
+        pt = torch.tensor([[3, 1, 0][:ring] + [2] * max(0, ring - 3)], dtype=torch.int32)[:, :ring]
+        kc = torch.full((4, nkv, page, hd), float("nan"), dtype=dtype); vc = kc.clone()
+        for pos in range(max(0, L - ring * page), L):    # what a ring keeps
+            pg = int(pt[0, (pos // page) % ring])
+            if pos // page + ring > (L - 1) // page:
+                kc[pg, :, pos % page] = view[pos, nh:nh + nkv]; vc[pg, :, pos % page] = view[pos, nh + nkv:]
+        q = view[L - 1:L].reshape(1, -1).contiguous()
+        got = ops().attn_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring,
+                                torch.zeros(1, dtype=torch.int32, device=DEV),
+                                torch.tensor([L], dtype=torch.int32, device=DEV), nh, nkv, hd, 1.0, window, 2)
+        mean = float(got.cpu().view(nh, hd)[0].float().mean())
+        assert (mean > 6.5) == sees, (L, mean)
+        close(got.cpu().view(nh, hd), out[L - 1], dtype, scale=8)

@@ -186,3 +186,28 @@ def test_temperature_sampling_is_reproducible_and_batch_independent(tmp_path_fac
     assert a == b and a != c
     eng1, _, _ = setup(tmp_path_factory, "B", "float32", max_batch=1)     # one at a time
     assert eng1.generate(prompts, temperature=0.8, seed=42, max_new_tokens=6, stop_token_ids=[]) == a
+
+
+def test_command_line_generates_like_the_plain_model(tmp_path):
+    """`bin/chat` with token-id prompts, greedy: the same tokens as the plain implementation."""
+    import os
+    import subprocess
+    import sys
+    config = CONFIGS["A"]
+    d = make_model_dir(tmp_path, config, seed=7, dtype=torch.float32)
+    w = read_weights(d)
+    prompts = requests_for(config, [7, 3], seed=3)
+    ids_file = tmp_path / "prompts.txt"
+    ids_file.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "chat"), "-m", d, "-d", "float32", "--temp", "0",
+                        "-n", "9", "--prompt-ids-file", str(ids_file), "-c", "64", "--summary", "--type", "llama2"],
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    got = [[int(t) for t in line.split()] for line in r.stdout.strip().splitlines()]
+    want = [plain_llama.generate_greedy(config, w, p, 9, [2]) for p in prompts]
+    assert got == want
+    assert "token/s" in r.stderr
+    bad = subprocess.run([sys.executable, os.path.join(root, "bin", "chat"), "-m", d, "--type", "chatglm",
+                          "--prompt-ids", "1 2"], capture_output=True, text=True, timeout=110)
+    assert bad.returncode == 2 and "does not fit" in bad.stderr

@@ -242,3 +242,94 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     for _ in range(3):
         seq.append(int(torch.argmax(toy_plain(w, cfg, seq)[-1])))
     assert got == [seq[len(reqs[1]):]]
+
+
+def test_embedding_and_head_parts():
+    from inferllm_amd.parts import build_part
+    from inferllm_amd.config import PartSpec
+    V, E = 411, 80
+    emb = build_part("embedding", PartSpec("token_embedding", {"vocab_size": V, "hidden_size": E}, {"weight": "e"}))
+    head = build_part("head", PartSpec("lm_head", {"hidden_size": E, "vocab_size": V, "tied_fallback": "e"}, {"weight": "h"}))
+    w = rnd(V, E, seed=1, std=0.3).to(torch.bfloat16)
+    assert head.wants()["h"].optional and not head.wants()["e"].optional
+    emb.load({"e": w.to(DEV)}); head.load({"e": w.to(DEV)})
+    cache, slots = make_ctx([0], None, {}, torch.bfloat16)
+    ctx = step_ctx(cache, slots, [0], [4], torch.bfloat16, True)
+    ctx.tokens = torch.tensor([5, 0, 410, 5], dtype=torch.int32, device=DEV)
+    x = emb.forward(ctx)
+    assert x.dtype == torch.float32 and torch.equal(x.cpu(), w[[5, 0, 410, 5]].float())
+    h = rnd(4, E, seed=2).to(torch.bfloat16)
+    logits = head.forward(h.to(DEV), ctx)
+    assert logits.dtype == torch.float32 and rel(logits, P.linear(h, w)) < 1e-4     # float32 out of bfloat16 operands
+
+
+def test_schedule_runs_a_layer_twice_and_shares_a_cache_line(tmp_path):
+    """The order of layers is data: layer 0 runs twice (two cache lines), then layer 1 reads the
+    keys and values that layer 0's second run stored.  Whole, token by token and in a batch."""
+    import inferllm_amd as I
+    from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from tiny import random_ids, read_weights
+    E, V, nh, nkv, hd, F, eps, theta = 64, 90, 4, 2, 16, 100, 1e-5, 10000.0
+
+    @register_architecture("ToyScheduleForTests")
+    class Cfg:
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": ["ToyScheduleForTests"]}
+
+        def to_spec(self):
+            norm = lambda n: PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": n})
+            def layer(i):
+                return LayerSpec("pre_norm",
+                                 PartSpec("attention", {"hidden_size": E, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd},
+                                          {k: f"l{i}.{k}" for k in "qkvo"}),
+                                 PartSpec("swiglu", {"hidden_size": E, "intermediate_size": F},
+                                          {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+                                 norm(f"l{i}.n1"), norm(f"l{i}.n2"),
+                                 PartSpec("rotary", {"head_dim": hd, "rotary_dim": hd, "theta": theta, "pairing": "half",
+                                                     "max_positions": 256}))
+            sched = [ScheduleEntry(0, 0), ScheduleEntry(0, 1), ScheduleEntry(1, 1, writes_cache=False)]
+            return ModelSpec("ToyScheduleForTests", V, E, 256,
+                             PartSpec("token_embedding", {"vocab_size": V, "hidden_size": E}, {"weight": "emb"}),
+                             [layer(0), layer(1)], sched, norm("nf"),
+                             PartSpec("lm_head", {"hidden_size": E, "vocab_size": V}, {"weight": "head"}))
+
+    d = I.write_random_model(str(tmp_path / "sched"), Cfg(), seed=8)
+    w = read_weights(d)
+
+    def plain(ids):
+        S = len(ids)
+        pos = list(range(S))
+        def attn(i, h, kv=None):
+            q = P.rope_rotate_half(P.linear(h, w[f"l{i}.q"]).reshape(S, nh, hd), pos, theta)
+            if kv is None:
+                k = P.rope_rotate_half(P.linear(h, w[f"l{i}.k"]).reshape(S, nkv, hd), pos, theta)
+                v = P.linear(h, w[f"l{i}.v"]).reshape(S, nkv, hd)
+            else:
+                k, v = kv
+            return P.linear(P.causal_attention(q, k, v), w[f"l{i}.o"]), (k, v)
+        def block(i, x, kv=None):
+            d1, kv = attn(i, P.rms_norm(x, w[f"l{i}.n1"], eps), kv)
+            x = x + d1
+            return x + P.swiglu_ffn(P.rms_norm(x, w[f"l{i}.n2"], eps), w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"]), kv
+        x = P.embedding(w["emb"], ids)
+        x, _ = block(0, x)
+        x, kv = block(0, x)
+        x, _ = block(1, x, kv)
+        return P.linear(P.rms_norm(x, w["nf"], eps), w["head"])
+
+    eng = I.Engine.from_pretrained(d, dtype="float32", max_batch=2, max_seq_len=128)
+    assert len(eng.cache.groups) == 1 and eng.cache.groups[0].lines == [0, 1]
+    reqs = [random_ids(n, V, n) for n in (30, 9)]
+    want = [plain(r) for r in reqs]
+    slots = [eng.alloc_slot(), eng.alloc_slot()]
+    head = [len(r) - 3 for r in reqs]
+    out = eng.step([I.StepEntry(s, r[:n], list(range(n))) for s, r, n in zip(slots, reqs, head)])
+    assert rel(out[:head[0]], want[0][:head[0]]) < 2e-5 and rel(out[head[0]:], want[1][:head[1]]) < 2e-5
+    for j in range(3):
+        out = eng.step([I.StepEntry(s, [r[n + j]], [0]) for s, r, n in zip(slots, reqs, head)])
+        for b in range(2):
+            assert rel(out[b], want[b][head[b] + j]) < 2e-5, (b, j)
