@@ -175,6 +175,185 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     }
 }
 
+// Grouped heads (several query heads per kv head), head_dim % 32 == 0: the scores of all the
+// group's heads come from the matrix cores.  S^T[key][head] = K . Q^T with MFMA 16x16x32: the A
+// operand is 16 keys x 32 dims straight from the cache (16 bytes per lane), the B operand the
+// group's queries (kept in registers), and a lane ends up with 4 keys of one head, so the
+// softmax statistics need two exchanges per tile.  P goes through a small LDS array to the
+// lanes that own the V rows, which accumulate P.V as in the kernel above.
+typedef __bf16 dbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float df32x4_t __attribute__((ext_vector_type(4)));
+
+template <int HD, int GC>
+__global__ void __launch_bounds__(64)
+attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
+                            const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+                            const int32_t* __restrict__ page_table, int table_stride,
+                            int page_size, int ring, const int32_t* __restrict__ seq_slot,
+                            const int32_t* __restrict__ slot_len, float* __restrict__ partial,
+                            int nsplit, int nh, int nkv, float scale, int window) {
+    constexpr int LPR = HD <= 32 ? 4 : (HD <= 64 ? 8 : (HD <= 128 ? 16 : 32));
+    constexpr int KPI = 64 / LPR;
+    constexpr int NI = LPR < 16 ? LPR : 16;
+    constexpr int TK = NI * KPI;               // 64 keys (32 when a row needs 32 lanes)
+    constexpr int NSUB = TK / 16;              // MFMA sub-tiles of 16 keys
+    constexpr int KS = HD / 32;                // k-steps of 32 dims
+    constexpr int PLD = 20;                    // floats per key row of P in LDS (16 heads + pad)
+    __shared__ __attribute__((aligned(16))) float ps[64 * PLD];
+    const int lane = threadIdx.x;
+    const int r = lane & 15, q4 = lane >> 4;   // MFMA roles: key / head, and k group
+    const int q = lane / LPR, c = lane % LPR;  // V row roles
+    const int G = nh / nkv;
+    const int chunks = (G + GC - 1) / GC;
+    const int kvh = blockIdx.x / chunks, g0 = (blockIdx.x % chunks) * GC;
+    const int b = blockIdx.y, sp = blockIdx.z;
+    const int slot = seq_slot[b];
+    const int len = slot_len[slot];
+    const int kf = window > 0 ? max(0, len - window) : 0;
+    const bool dim_ok = c * 8 < HD;
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
+    const bool head_ok = (r < GC) && (g0 + r < G);
+
+    uint4 qf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        qf[s] = make_uint4(0, 0, 0, 0);
+        if (head_ok)
+            qf[s] = *(const uint4*)(qkv + (size_t)b * rowlen + (size_t)(kvh * G + g0 + r) * HD +
+                                    s * 32 + q4 * 8);
+    }
+    float m = NEG_INF, l = 0.f;                // of head r (the same in the four k groups)
+    float acc[GC][8];
+#pragma unroll
+    for (int g = 0; g < GC; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
+
+    const int t_first = kf / TK;
+    const int n_tiles = (len + TK - 1) / TK - t_first;
+    const int per = (n_tiles + nsplit - 1) / nsplit;
+    const int t_lo = t_first + sp * per;
+    const int t_hi = min(t_first + n_tiles, t_lo + per);
+
+    for (int t = t_lo; t < t_hi; ++t) {
+        const int k0 = t * TK;
+        int lp = k0 / page_size;
+        if (ring > 0) lp %= ring;
+        const int phys = page_table[(size_t)slot * table_stride + lp];
+        const size_t tile = (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)HD;
+        uint4 ka[NSUB][KS], vreg[NI];
+#pragma unroll
+        for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                ka[sub][s] = *(const uint4*)(kcache + tile + (size_t)(sub * 16 + r) * HD + s * 32 + q4 * 8);
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            vreg[j] = dim_ok ? *(const uint4*)(vcache + tile + (size_t)(j * KPI + q) * HD + c * 8)
+                             : make_uint4(0, 0, 0, 0);
+        // scores of 4 keys per sub-tile for head r
+        float sv[NSUB][4];
+        float mx = NEG_INF;
+#pragma unroll
+        for (int sub = 0; sub < NSUB; ++sub) {
+            df32x4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const dbf16x8_t*)&ka[sub][s],
+                                                            *(const dbf16x8_t*)&qf[s], a, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = k0 + sub * 16 + 4 * q4 + i;
+                const bool ok = key < len && key >= kf;
+                sv[sub][i] = ok ? a[i] * scale : NEG_INF;
+                mx = fmaxf(mx, sv[sub][i]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, ILLM_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
+        const float alpha = expf(m - m_use);             // m = -inf gives 0 (nothing summed yet)
+        float rs = 0.f;
+        __syncthreads();                                  // the last tile's P has been read
+#pragma unroll
+        for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float p = (sv[sub][i] == NEG_INF) ? 0.f : expf(sv[sub][i] - m_use);
+                rs += p;
+                ps[(sub * 16 + 4 * q4 + i) * PLD + r] = p;
+            }
+        rs += __shfl_xor(rs, 16, ILLM_WAVE);
+        rs += __shfl_xor(rs, 32, ILLM_WAVE);
+        l = l * alpha + rs;
+        m = m_new;
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            const float ag = __shfl(alpha, g, ILLM_WAVE);  // lane g holds head g's factor
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] *= ag;
+        }
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int kt = j * KPI + q;
+            const int key = k0 + kt;
+            const bool ok = key < len && key >= kf;
+            float vf8[8];
+            unpack8(vreg[j], vf8);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vf8[i] = ok ? vf8[i] : 0.f;
+#pragma unroll
+            for (int g4 = 0; g4 < GC; g4 += 4) {
+                const float4 pv = *(const float4*)(ps + kt * PLD + g4);
+                const float pg[4] = {pv.x, pv.y, pv.z, pv.w};
+#pragma unroll
+                for (int gg = 0; gg < 4 && g4 + gg < GC; ++gg)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        acc[g4 + gg][i] = fmaf(pg[gg], vf8[i], acc[g4 + gg][i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < GC; ++g)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float a = acc[g][i];
+#pragma unroll
+            for (int o = LPR; o < 64; o <<= 1) a += __shfl_xor(a, o, ILLM_WAVE);
+            acc[g][i] = a;
+        }
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        const float lg = __shfl(l, g, ILLM_WAVE), mg = __shfl(m, g, ILLM_WAVE);
+        if (g0 + g >= G) continue;
+        const int h = kvh * G + g0 + g;
+        if (nsplit == 1) {
+            if (q == 0 && dim_ok) {
+                const float inv = 1.0f / lg;
+                uint4 o;
+                o.x = pack_bf16x2(acc[g][0] * inv, acc[g][1] * inv);
+                o.y = pack_bf16x2(acc[g][2] * inv, acc[g][3] * inv);
+                o.z = pack_bf16x2(acc[g][4] * inv, acc[g][5] * inv);
+                o.w = pack_bf16x2(acc[g][6] * inv, acc[g][7] * inv);
+                *(uint4*)(out + ((size_t)b * nh + h) * HD + c * 8) = o;
+            }
+        } else {
+            float* pp = partial + (((size_t)b * nh + h) * nsplit + sp) * (size_t)(HD + 2);
+            if (q == 0 && dim_ok) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pp[c * 8 + i] = acc[g][i];
+            }
+            if (lane == 0) {
+                pp[HD] = mg;
+                pp[HD + 1] = lg;
+            }
+        }
+    }
+}
+
 // grid (heads, sequences), one wave: lane s holds split s's max and sum (nsplit <= 64), the
 // weights are formed once, and splits that saw no key are skipped.
 __global__ void __launch_bounds__(64)
@@ -251,6 +430,41 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
     const int G = nh / nkv;
+    if (G > 1 && hd % 32 == 0) {
+        int gcq = 2;
+        while (gcq < G && gcq < 16) gcq <<= 1;
+        const int chunks = (G + gcq - 1) / gcq;
+        const dim3 grid(nkv * chunks, B, nsplit);
+#define GQA(HD_, GC_)                                                                              \
+    hipLaunchKernelGGL((attn_decode_bf16_gqa_kernel<HD_, GC_>), grid, dim3(64), 0,                 \
+                       (hipStream_t)stream, (const bf16_t*)qkv, (bf16_t*)out,                      \
+                       (const bf16_t*)kcache, (const bf16_t*)vcache, page_table, table_stride,     \
+                       page_size, ring, seq_slot, slot_len, partial, nsplit, nh, nkv, scale, window)
+#define GQA_HD(HD_)                                                                                \
+    do {                                                                                           \
+        if (gcq == 2) GQA(HD_, 2);                                                                 \
+        else if (gcq == 4) GQA(HD_, 4);                                                            \
+        else if (gcq == 8) GQA(HD_, 8);                                                            \
+        else GQA(HD_, 16);                                                                         \
+    } while (0)
+        switch (hd) {
+            case 32: GQA_HD(32); break;
+            case 64: GQA_HD(64); break;
+            case 96: GQA_HD(96); break;
+            case 128: GQA_HD(128); break;
+            case 160: GQA_HD(160); break;
+            case 192: GQA_HD(192); break;
+            case 224: GQA_HD(224); break;
+            default: GQA_HD(256); break;
+        }
+#undef GQA_HD
+#undef GQA
+        if (nsplit > 1)
+            hipLaunchKernelGGL(attn_decode_bf16_merge_kernel, dim3(nh, B), dim3(64), 0,
+                               (hipStream_t)stream, (const float*)partial, (bf16_t*)out, nsplit, nh,
+                               hd);
+        return illm_launch_status();
+    }
     int gc = 1;
     while (gc < G && gc < 8) gc <<= 1;
     int lpr = 1;

@@ -242,7 +242,8 @@ def test_attn_decode(dtype, nh, nkv, hd, lens, window, nsplit):
     (32, 32, 128, [600, 1, 64, 65], 0, 1), (32, 8, 128, [300, 70], 0, 3), (4, 4, 16, [7, 200], 0, 2),
     (8, 1, 64, [1000], 0, 32), (6, 2, 24, [5, 11, 130], 0, 2), (16, 1, 256, [257, 31], 0, 2),
     (5, 5, 96, [130, 520], 70, 5), (12, 4, 32, [90, 17, 700], 13, 2), (3, 3, 8, [129], 0, 1),
-    (20, 2, 48, [333], 0, 4)])
+    (20, 2, 48, [333], 0, 4), (64, 8, 128, [1000, 63], 0, 5), (32, 8, 64, [129], 0, 1), (6, 3, 96, [70, 700], 0, 3),
+    (34, 2, 32, [200], 0, 2), (8, 2, 160, [90, 300], 50, 2), (10, 5, 224, [65], 0, 1)])
 def test_attn_decode_bf16_pages_of_64(nh, nkv, hd, lens, window, nsplit):
     """The fast bfloat16 kernel (pages of 64 rows, as the engine's cache has them); stale rows
     of the pages are NaN and must not leak into the result."""
