@@ -79,6 +79,16 @@ int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, i
 int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* Y, int y_dt, int M, int F,
                                  int K, void* stream);
 
+// Few bfloat16 rows (M <= 16, hd % 32 == 0): the q|k|v product, the rotation of q and k (pairs
+// (i, i + hd/2), all dims) at row_pos[m], q into Y[M, (nh + 2 nkv) hd] (k and v parts untouched),
+// k and v into the paged cache of row_slot[m], all in one kernel.  waves_wanted: waves per block
+// (0: the default choice).
+int illm_qkv_rope_store_skinny(const void* X, const void* W, void* Y, int M, int K,
+                               const float* cos_sin, int max_pos, const int32_t* row_pos,
+                               const int32_t* row_slot, void* kcache, void* vcache,
+                               const int32_t* page_table, int table_stride, int page_size, int ring,
+                               int nh, int nkv, int hd, int waves_wanted, void* stream);
+
 // out[b] = index of the largest logit of row b (lowest index on ties).
 int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream);
 

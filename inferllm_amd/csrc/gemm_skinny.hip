@@ -20,24 +20,84 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // U: k-steps (of 32) per wave iteration, i.e. U * 64 contiguous bytes of each W row.
 // MAXW: most waves a block may have (register budget: 512 / (MAXW / 4) per lane).
-// DUAL (with NTB == 2): W is [gate rows (N) | up rows (N)]; the block's two tiles are the same
-// 16 rows of each half and the result is silu(gate) * up, Y[M, N].
-template <int MT, int NTB, int SK_U, int MAXW, bool DUAL>
+// What a block's tiles are and what happens to the sums:
+//   SK_PLAIN     NTB consecutive tiles of 16 rows of W; Y = sums.
+//   SK_GATE_UP   (NTB == 2) W is [gate rows (N) | up rows (N)]; the two tiles are the same 16 rows
+//                of each half and Y[M, N] = silu(gate) * up.
+//   SK_QKV_ROPE  (NTB == 2) W is [q heads | k heads | v heads]; a block of a q or k head takes 16
+//                rows and their rotation partners (hd/2 further), rotates the pairs by the row's
+//                position and writes q to Y and k to the paged cache; a block of a v head takes 32
+//                consecutive rows and writes them to the cache.
+enum { SK_PLAIN = 0, SK_GATE_UP = 1, SK_QKV_ROPE = 2 };
+
+struct SkRope {
+    const float* cos_sin;        // [max_pos][hd/2][2]
+    const int32_t* row_pos;      // [M]
+    const int32_t* row_slot;     // [M]
+    bf16_t* kcache;
+    bf16_t* vcache;
+    const int32_t* page_table;
+    int table_stride, page_size, ring, nh, nkv, hd;
+};
+
+template <int MT, int NTB, int SK_U, int MAXW, int MODE>
 __global__ void __launch_bounds__(64 * MAXW)
 gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                   void* __restrict__ Y, int y_dt, int M, int N, int K) {
+                   void* __restrict__ Y, int y_dt, int M, int N, int K, SkRope rope) {
+    constexpr bool DUAL = MODE == SK_GATE_UP;
     extern __shared__ float red[];   // [waves][NTB * MT * 64 * 4]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
     const int r = lane & 15, q = lane >> 4;
     const int n_base = blockIdx.x * (DUAL ? 16 : 16 * NTB);
+    int tile_row[NTB];           // first W row of each of the block's tiles
+#pragma unroll
+    for (int nt = 0; nt < NTB; ++nt) tile_row[nt] = n_base + (DUAL ? nt * N : nt * 16);
+    int rot_head = -1, rot_j = 0;
+    if (MODE == SK_QKV_ROPE) {
+        const int pph = rope.hd / 32, n_rot = (rope.nh + rope.nkv) * pph;
+        if ((int)blockIdx.x < n_rot) {
+            rot_head = blockIdx.x / pph;
+            rot_j = blockIdx.x % pph;
+            tile_row[0] = rot_head * rope.hd + 16 * rot_j;
+            tile_row[NTB - 1] = tile_row[0] + rope.hd / 2;
+        } else {
+            tile_row[0] = (rope.nh + rope.nkv) * rope.hd + 32 * ((int)blockIdx.x - n_rot);
+            tile_row[NTB - 1] = tile_row[0] + 16;
+        }
+    }
+
+    // SK_QKV_ROPE: the threads that will write the results fetch what that needs (position,
+    // angles, the cache row's address) now, so that it arrives while W is streamed
+    float pre_cs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    size_t pre_off = 0;
+    if (MODE == SK_QKV_ROPE && threadIdx.x < 64 && (int)(threadIdx.x & 15) < M) {
+        const int mrow = threadIdx.x & 15, ro = (threadIdx.x >> 4) * 4;
+        const int pos = rope.row_pos[mrow], slot = rope.row_slot[mrow];
+        if (rot_head >= 0) {
+            const float4* cs = (const float4*)(rope.cos_sin + (size_t)pos * rope.hd + 2 * (16 * rot_j + ro));
+            const float4 c0 = cs[0], c1 = cs[1];
+            pre_cs[0] = c0.x; pre_cs[1] = c0.y; pre_cs[2] = c0.z; pre_cs[3] = c0.w;
+            pre_cs[4] = c1.x; pre_cs[5] = c1.y; pre_cs[6] = c1.z; pre_cs[7] = c1.w;
+            if (rot_head >= rope.nh)
+                pre_off = cache_row_offset(rope.page_table, rope.table_stride, slot, pos,
+                                           rope.page_size, rope.ring, rope.nkv, rot_head - rope.nh,
+                                           rope.hd) + 16 * rot_j + ro;
+        } else {
+            const int vrow = tile_row[0] - (rope.nh + rope.nkv) * rope.hd;
+            pre_off = cache_row_offset(rope.page_table, rope.table_stride, slot, pos, rope.page_size,
+                                       rope.ring, rope.nkv, vrow / rope.hd, rope.hd) + vrow % rope.hd + ro;
+        }
+    }
 
     const bf16_t* wrow[NTB];
 #pragma unroll
     for (int nt = 0; nt < NTB; ++nt) {
-        int n = n_base + (DUAL ? 0 : nt * 16) + r;
-        n = n < N ? n : N - 1;
-        wrow[nt] = W + ((size_t)n + (DUAL ? (size_t)nt * N : 0)) * K;
+        int n = tile_row[nt] + r;
+        const int last = DUAL ? 2 * N - 1 : N - 1;
+        if (DUAL) n = (n - nt * N < N) ? n : nt * N + N - 1;
+        else n = n < last ? n : last;
+        wrow[nt] = W + (size_t)n * K;
     }
     const bf16_t* xrow[MT];
 #pragma unroll
@@ -127,7 +187,29 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
         }
         const int mrow = mt * 16 + (l2 & 15);
         if (mrow >= M) continue;
-        if (DUAL) {
+        if (MODE == SK_QKV_ROPE) {
+            // MT == 1 and at least 64 threads: grp == threadIdx.x, the thread that prefetched
+            const int ro = (l2 >> 4) * 4;                 // this lane's 4 rows within a tile
+            if (rot_head >= 0) {
+                float y0[4], y1[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float c = pre_cs[2 * i], sn = pre_cs[2 * i + 1];
+                    y0[i] = v[0][i] * c - v[NTB - 1][i] * sn;
+                    y1[i] = v[0][i] * sn + v[NTB - 1][i] * c;
+                }
+                bf16_t* dst = rot_head < rope.nh ? (bf16_t*)Y + (size_t)mrow * N + tile_row[0] + ro
+                                                 : rope.kcache + pre_off;
+                *(uint2*)dst = make_uint2(pack_bf16x2(y0[0], y0[1]), pack_bf16x2(y0[2], y0[3]));
+                *(uint2*)(dst + rope.hd / 2) =
+                    make_uint2(pack_bf16x2(y1[0], y1[1]), pack_bf16x2(y1[2], y1[3]));
+            } else {
+                bf16_t* dst = rope.vcache + pre_off;
+                *(uint2*)dst = make_uint2(pack_bf16x2(v[0][0], v[0][1]), pack_bf16x2(v[0][2], v[0][3]));
+                *(uint2*)(dst + 16) = make_uint2(pack_bf16x2(v[NTB - 1][0], v[NTB - 1][1]),
+                                                 pack_bf16x2(v[NTB - 1][2], v[NTB - 1][3]));
+            }
+        } else if (DUAL) {
             const int n0 = n_base + (l2 >> 4) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -138,7 +220,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
         } else {
 #pragma unroll
             for (int nt = 0; nt < NTB; ++nt) {
-                const int n0 = n_base + nt * 16 + (l2 >> 4) * 4;
+                const int n0 = tile_row[nt] + (l2 >> 4) * 4;
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[nt][i]);
@@ -147,9 +229,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     }
 }
 
-template <int MT, int NTB, int U, bool DUAL = false>
+template <int MT, int NTB, int U, int MODE = SK_PLAIN>
 static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
-                         int waves, hipStream_t st) {
+                         int waves, hipStream_t st, SkRope rope = SkRope()) {
+    constexpr bool DUAL = MODE == SK_GATE_UP;
     // registers a lane needs: operands of two pieces in flight and the accumulators
     constexpr int REGS = 2 * (NTB + MT) * U * 4 + NTB * MT * 4 + 40;
     constexpr int MAXW = REGS <= 128 ? 16 : (REGS <= 256 ? 8 : 4);
@@ -157,8 +240,8 @@ static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M,
     const int rows_per_block = DUAL ? 16 : 16 * NTB;
     const int blocks = (N + rows_per_block - 1) / rows_per_block;
     const size_t smem = waves > 1 ? (size_t)waves * NTB * MT * 64 * 4 * sizeof(float) : 0;
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, DUAL>), dim3(blocks), dim3(64 * waves),
-                       smem, st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K);
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, MODE>), dim3(blocks), dim3(64 * waves),
+                       smem, st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K, rope);
     return illm_launch_status();
 }
 
@@ -218,9 +301,34 @@ extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* 
     int waves = (1536 + blocks / 2) / blocks;
     waves = clamp_waves(waves < 1 ? 1 : waves, 2, mt, 4, K);
     switch (mt) {
-        case 1: return launch_skinny<1, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
-        case 2: return launch_skinny<2, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
-        case 3: return launch_skinny<3, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
-        default: return launch_skinny<4, 2, 4, true>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 1: return launch_skinny<1, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 2: return launch_skinny<2, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 3: return launch_skinny<3, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        default: return launch_skinny<4, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
     }
+}
+
+// Decode step of an attention layer's input side in one kernel: Y = X . Wqkv^T, the q and k heads
+// rotated (pairs (i, i + hd/2), all hd dims) by the angles at row_pos[m], q written to
+// Y[M, (nh + 2 nkv) hd] (its k and v parts are left untouched), k and v written to the paged cache
+// of row_slot[m].  M <= 16, hd % 32 == 0, K % 8 == 0, bfloat16.
+extern "C" int illm_qkv_rope_store_skinny(const void* X, const void* W, void* Y, int M, int K,
+                                          const float* cos_sin, int max_pos,
+                                          const int32_t* row_pos, const int32_t* row_slot,
+                                          void* kcache, void* vcache, const int32_t* page_table,
+                                          int table_stride, int page_size, int ring, int nh, int nkv,
+                                          int hd, int waves_wanted, void* stream) {
+    if (M <= 0 || M > 16 || K <= 0 || (K % 8) || nh <= 0 || nkv <= 0 || hd <= 0 || (hd % 32) ||
+        !cos_sin || max_pos <= 0 || !row_pos || !row_slot || !kcache || !vcache || !page_table ||
+        table_stride <= 0 || page_size <= 0)
+        return ILLM_ERR_ARG;
+    SkRope rope = {cos_sin, row_pos, row_slot, (bf16_t*)kcache, (bf16_t*)vcache, page_table,
+                   table_stride, page_size, ring, nh, nkv, hd};
+    const int N = (nh + 2 * nkv) * hd;
+    const int blocks = N / 32;
+    // measured at the 7B shape: about 1152 waves on the chip are best for 32-row blocks
+    int waves = waves_wanted > 0 ? waves_wanted : (1152 + blocks / 2) / blocks;
+    waves = clamp_waves(waves < 1 ? 1 : waves, 2, 1, 4, K);
+    return launch_skinny<1, 2, 4, SK_QKV_ROPE>(X, W, Y, ILLM_BF16, M, N, K, waves,
+                                               (hipStream_t)stream, rope);
 }

@@ -216,6 +216,40 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -
     return y
 
 
+QKV_ROPE_WAVES = 0       # waves per block of the fused kernel; 0: the kernel's own choice
+
+
+def qkv_rope_store_fits(x: torch.Tensor, w_qkv: torch.Tensor, hd: int) -> bool:
+    """Whether the one-kernel q|k|v product + rotation + cache store takes these operands."""
+    return (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and
+            1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0 and hd % 32 == 0)
+
+
+def qkv_rope_store(x: torch.Tensor, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
+                   row_pos: torch.Tensor, row_slot: torch.Tensor, kcache: torch.Tensor,
+                   vcache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
+                   nh: int, nkv: int, hd: int) -> torch.Tensor:
+    """Decode only: x . Wqkv^T, q and k rotated (pairs (i, i + hd/2), all dims) at row_pos, q
+    returned in rows [q | k | v] whose k and v parts are NOT filled, k and v stored in the cache."""
+    _gpu(x, w_qkv, cos_sin, row_pos, row_slot, kcache, vcache, page_table)
+    _i32(row_pos, x.shape[0]); _i32(row_slot, x.shape[0]); _i32(page_table)
+    M, K = x.shape
+    N = (nh + 2 * nkv) * hd
+    _need(qkv_rope_store_fits(x, w_qkv, hd), "qkv_rope_store: operands not taken")
+    _need(w_qkv.shape == (N, K), f"qkv_rope_store: weight {tuple(w_qkv.shape)} vs ({N}, {K})")
+    _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[1] * 2 == hd and
+          cos_sin.shape[2] == 2, "qkv_rope_store: angle table must be float32 [max_pos, hd/2, 2]")
+    _need(kcache.dtype == torch.bfloat16 and kcache.shape[1:] == (nkv, page_size, hd) and
+          vcache.shape == kcache.shape and vcache.dtype == torch.bfloat16 and page_table.dim() == 2,
+          "qkv_rope_store: cache shape or dtype")
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    _check(_lib().illm_qkv_rope_store_skinny(
+        _p(x), _p(w_qkv), _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
+        _p(kcache), _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, nh, nkv, hd,
+        QKV_ROPE_WAVES, _stream()), "qkv_rope_store")
+    return y
+
+
 def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     """silu(x . Wg^T) * (x . Wu^T) for w_gate_up = [Wg | Wu] stacked as [2F, K].
 

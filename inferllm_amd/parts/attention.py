@@ -62,10 +62,10 @@ class Attention(Mixer):
         kc, vc, group = ctx.cache.kv_line(line)
         window = self.window or 0
         if writes_cache:
-            qkv = ops.linear(h, self.w_qkv)
             if position is not None:
-                position.on_qkv(qkv, ctx, nh, nkv, hd, kc, vc, group)
+                qkv = position.project_qkv(h, self.w_qkv, ctx, nh, nkv, hd, kc, vc, group)
             else:
+                qkv = ops.linear(h, self.w_qkv)
                 ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot, ctx.cache.slot_len, kc,
                                vc, group.table, group.page_size, group.ring, nh, nkv, hd)
             if ctx.prefill:

@@ -111,6 +111,16 @@ class PositionEncoding(Part):
         """Encode q and k of packed rows in place and store k, v in the cache (if given)."""
         raise NotImplementedError
 
+    def project_qkv(self, h: torch.Tensor, w_qkv: torch.Tensor, ctx: StepContext, nh: int,
+                    nkv: int, hd: int, kcache, vcache, group) -> torch.Tensor:
+        """Packed rows [q | k | v] = h . w_qkv^T, encoded, k and v stored.  An encoding may
+        override this with a fused kernel; in a step of single tokens the k and v parts of the
+        returned rows need not be filled (they are read from the cache)."""
+        from ..kernels import ops
+        qkv = ops.linear(h, w_qkv)
+        self.on_qkv(qkv, ctx, nh, nkv, hd, kcache, vcache, group)
+        return qkv
+
 
 class Block(Part):
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,

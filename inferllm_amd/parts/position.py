@@ -63,6 +63,16 @@ class Rotary(PositionEncoding):
                        group.ring if group is not None else 0, nh, nkv, hd)
 
 
+    def project_qkv(self, h, w_qkv, ctx: StepContext, nh, nkv, hd, kcache, vcache, group):
+        if (not ctx.prefill and kcache is not None and self.pairing == "half"
+                and self.rotary_dim == hd and ops.qkv_rope_store_fits(h, w_qkv, hd)
+                and kcache.dtype == torch.bfloat16):
+            return ops.qkv_rope_store(h, w_qkv, self.table(ctx.device), ctx.row_pos, ctx.row_slot,
+                                      kcache, vcache, group.table, group.page_size, group.ring,
+                                      nh, nkv, hd)
+        return super().project_qkv(h, w_qkv, ctx, nh, nkv, hd, kcache, vcache, group)
+
+
 @register_part("position", "none")
 class NoPosition(PositionEncoding):
     """No encoding: q and k stay as they are; k and v are still stored."""

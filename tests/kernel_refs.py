@@ -83,6 +83,10 @@ def linear(x, w, out_dtype=None):
     return (x.to(F64) @ w.to(F64).t()).to(out_dtype or x.dtype)
 
 
+def qkv_rope_store_fits(x, w_qkv, hd):
+    return False        # the CPU stand-in goes through linear + rope_store
+
+
 def gate_up_silu(x, w_gate_up):
     return silu_mul(linear(x, w_gate_up))
 
@@ -191,6 +195,6 @@ def sample(logits, temperature, top_k, top_p, repeat_penalty, last_tokens, seeds
 def patch(monkeypatch):
     """Put these functions in place of the GPU ops (CPU tests only)."""
     from inferllm_amd.kernels import ops
-    for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic", "gate_up_silu",
+    for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic", "gate_up_silu", "qkv_rope_store_fits",
                  "attn_prefill", "decode_splits", "attn_decode", "argmax", "sample"):
         monkeypatch.setattr(ops, name, globals()[name])

@@ -403,3 +403,30 @@ def test_window_edge_prefill_and_decode(dtype, hd):
         mean = float(got.cpu().view(nh, hd)[0].float().mean())
         assert (mean > 6.5) == sees, (L, mean)
         close(got.cpu().view(nh, hd), out[L - 1], dtype, scale=8)
+
+
+@pytest.mark.parametrize("M,nh,nkv,hd,K", [(1, 32, 32, 128, 4096), (8, 4, 2, 32, 64), (16, 6, 3, 64, 200), (3, 8, 1, 96, 72)])
+def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K):
+    """The fused decode kernel against product, then rotation and cache store."""
+    from inferllm_amd.parts.position import rotary_table
+    dtype, page = torch.bfloat16, 64
+    table = rotary_table(777.0, hd, 300, "cpu")
+    x = rnd(M, K, dtype=dtype, seed=1)
+    w = rnd((nh + 2 * nkv) * hd, K, dtype=dtype, seed=2, std=0.1)
+    pos = torch.tensor([(37 * i + 5) % 290 for i in range(M)], dtype=torch.int32)
+    slot = torch.randperm(M + 2, generator=torch.Generator().manual_seed(9))[:M].to(torch.int32)
+    assert len(set(slot.tolist())) == M
+    g = torch.Generator().manual_seed(4)
+    pt = torch.randperm((M + 2) * 5, generator=g).reshape(M + 2, 5).to(torch.int32)
+    kc, vc = make_cache((M + 2) * 5, nkv, page, hd, dtype)
+    # reference: float64 product, rounded to bfloat16 once (as the fused kernel rounds once)
+    qkv_ref = R.linear(x, w, torch.float64)
+    kr, vr = kc.clone().double(), vc.clone().double()
+    R.rope_store(qkv_ref, table, hd, 0, pos, slot, None, kr, vr, pt, page, 0, nh, nkv, hd)
+    got = ops().qkv_rope_store(x.to(DEV), w.to(DEV), table.to(DEV), pos.to(DEV), slot.to(DEV), kc_g := kc.to(DEV),
+                               vc_g := vc.to(DEV), pt.to(DEV), page, 0, nh, nkv, hd).cpu()
+    sc = math.sqrt(K) * 0.1
+    close(got[:, :nh * hd], qkv_ref[:, :nh * hd], dtype, scale=sc)
+    for gotc, wantc in ((kc_g.cpu(), kr), (vc_g.cpu(), vr)):
+        assert torch.equal(torch.isnan(gotc), torch.isnan(wantc))        # the same rows, nothing else
+        close(torch.nan_to_num(gotc), torch.nan_to_num(wantc), dtype, scale=sc)

@@ -211,3 +211,24 @@ def test_command_line_generates_like_the_plain_model(tmp_path):
     bad = subprocess.run([sys.executable, os.path.join(root, "bin", "chat"), "-m", d, "--type", "chatglm",
                           "--prompt-ids", "1 2"], capture_output=True, text=True, timeout=110)
     assert bad.returncode == 2 and "does not fit" in bad.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompt_then_decoding_at_head_size_128(tmp_path_factory, dtype):
+    """1,500 tokens in one step (many query blocks, key tiles and pages), then 40 tokens one by
+    one at positions beyond 1,500, with the head size and grouping of the large models."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "D", dtype, max_batch=2, max_seq_len=2048,
+                               max_tokens=2048 + 64)
+    ids = requests_for(config, [1540], seed=12)[0]
+    want = plain(ids)
+    s = eng.alloc_slot()
+    probe = [0, 1, 63, 64, 127, 128, 129, 700, 1023, 1024, 1499]
+    got = eng.step([StepEntry(s, ids[:1500], probe)]).clone()
+    per = (got.double().cpu() - want[probe]).abs().max(dim=1).values / want.abs().max()
+    assert float(per.max()) < BUDGET[dtype], f"prefill rows {[p for p, e in zip(probe, per) if e >= BUDGET[dtype]]}"
+    outs = [eng.step([StepEntry(s, [t], [0])]).clone() for t in ids[1500:]]
+    per = (torch.cat(outs).double().cpu() - want[1500:]).abs().max(dim=1).values / want.abs().max()
+    assert float(per.max()) < BUDGET[dtype], f"first bad decode position {1500 + int((per >= BUDGET[dtype]).nonzero()[0])}"
+    eng.free_slot(s)
+    eng.cache.check()

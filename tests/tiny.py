@@ -26,7 +26,13 @@ TINY_C = {"architectures": ["LlamaForCausalLM"], "hidden_size": 80, "intermediat
           "head_dim": 32, "vocab_size": 411, "rms_norm_eps": 3e-5, "rope_theta": 25000.0,
           "max_position_embeddings": 512, "tie_word_embeddings": True,
           "bos_token_id": 0, "eos_token_id": 5}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# the head size and group layout of the large models, long positions, few parameters
+TINY_D = {"architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermediate_size": 520,
+          "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 2,
+          "head_dim": 128, "vocab_size": 1000, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+          "max_position_embeddings": 4096, "tie_word_embeddings": False,
+          "bos_token_id": 1, "eos_token_id": 2}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def make_model_dir(tmp_path, config: dict, seed: int, dtype=torch.float32) -> str:
