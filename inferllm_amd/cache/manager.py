@@ -202,11 +202,13 @@ class CacheManager:
         self.len_host[slot] = new_len
         self._len_dirty = True
 
-    def upload(self) -> None:
-        """Bring page tables and lengths on the device up to date with the host."""
+    def upload(self, lengths: bool = True) -> None:
+        """Bring page tables (and, unless `lengths` is False, the per-slot lengths) on the
+        device up to date with the host.  Steps of single tokens carry their sequences'
+        lengths themselves and leave `slot_len` for the next step of whole prompts."""
         for g in self.groups:
             g.upload()
-        if self._len_dirty:
+        if lengths and self._len_dirty:
             self.slot_len.copy_(self.len_host)
             self._len_dirty = False
 

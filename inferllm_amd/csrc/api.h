@@ -28,7 +28,9 @@ int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* st
 // Rotate q and k of packed rows [q (nh*hd) | k (nkv*hd) | v (nkv*hd)] in place by the
 // angles of `cos_sin` ([max_pos][rot/2][2] float32; null: no rotation) at row_pos[t],
 // pairing 0 = (i, i + rot/2), 1 = (2i, 2i+1); then store k and v of each row in the
-// paged cache of row_slot[t] (skipped when kcache is null).
+// paged cache of row_slot[t] (skipped when kcache is null).  With a ring of pages, slot_len
+// (length of every slot after the step) lets rows that a later row of the same step would
+// overwrite be skipped; it may be null when no sequence brings more than one row.
 int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_pos, int rot, int pairing,
                     const int32_t* row_pos, const int32_t* row_slot, const int32_t* slot_len,
                     void* kcache, void* vcache, const int32_t* page_table, int table_stride,
@@ -50,18 +52,18 @@ int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens
                            void* stream);
 
 // One query row per sequence over the paged cache.  partial: float32
-// [B][nh][nsplit][hd + 2] scratch.  slot_len[slot] = keys of the sequence, the new one included.
+// [B][nh][nsplit][hd + 2] scratch.  seq_len[b] = keys of sequence b, the new one included.
 int illm_attn_decode_generic(const void* qkv, void* out, int dt, const void* kcache,
                              const void* vcache, const int32_t* page_table, int table_stride,
                              int page_size, int ring, const int32_t* seq_slot,
-                             const int32_t* slot_len, float* partial, int nsplit, int B, int nh,
+                             const int32_t* seq_len, float* partial, int nsplit, int B, int nh,
                              int nkv, int hd, float scale, int window, void* stream);
 
 // The same for bfloat16 with head_dim % 8 == 0 and page_size % 64 == 0 (anything else:
 // ILLM_ERR_ARG); nsplit == 1 needs no `partial`.
 int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache, const void* vcache,
                           const int32_t* page_table, int table_stride, int page_size, int ring,
-                          const int32_t* seq_slot, const int32_t* slot_len, float* partial,
+                          const int32_t* seq_slot, const int32_t* seq_len, float* partial,
                           int nsplit, int B, int nh, int nkv, int hd, float scale, int window,
                           void* stream);
 

@@ -34,7 +34,7 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
                         const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                         const int32_t* __restrict__ page_table, int table_stride, int page_size,
                         int ring, const int32_t* __restrict__ seq_slot,
-                        const int32_t* __restrict__ slot_len, float* __restrict__ partial,
+                        const int32_t* __restrict__ seq_len, float* __restrict__ partial,
                         int nsplit, int nh, int nkv, int hd, float scale, int window) {
     constexpr int KPI = 64 / LPR;              // keys per load instruction
     constexpr int NI = LPR < 16 ? LPR : 16;    // load instructions per tile
@@ -44,7 +44,7 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     const int kvh = blockIdx.x % nkv, g0 = (blockIdx.x / nkv) * GC;
     const int b = blockIdx.y, sp = blockIdx.z;
     const int slot = seq_slot[b];
-    const int len = slot_len[slot];
+    const int len = seq_len[b];
     const int kf = window > 0 ? max(0, len - window) : 0;
     const bool dim_ok = c * 8 < hd;
     const size_t rowlen = (size_t)(nh + 2 * nkv) * hd;
@@ -190,7 +190,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
                             const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                             const int32_t* __restrict__ page_table, int table_stride,
                             int page_size, int ring, const int32_t* __restrict__ seq_slot,
-                            const int32_t* __restrict__ slot_len, float* __restrict__ partial,
+                            const int32_t* __restrict__ seq_len, float* __restrict__ partial,
                             int nsplit, int nh, int nkv, float scale, int window) {
     constexpr int LPR = HD <= 32 ? 4 : (HD <= 64 ? 8 : (HD <= 128 ? 16 : 32));
     constexpr int KPI = 64 / LPR;
@@ -208,7 +208,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
     const int kvh = blockIdx.x / chunks, g0 = (blockIdx.x % chunks) * GC;
     const int b = blockIdx.y, sp = blockIdx.z;
     const int slot = seq_slot[b];
-    const int len = slot_len[slot];
+    const int len = seq_len[b];
     const int kf = window > 0 ? max(0, len - window) : 0;
     const bool dim_ok = c * 8 < HD;
     const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
@@ -382,7 +382,7 @@ attn_decode_bf16_merge_kernel(const float* __restrict__ partial, bf16_t* __restr
 template <int LPR, int GC>
 static int launch_decode(const void* qkv, void* out, const void* kcache, const void* vcache,
                          const int32_t* page_table, int table_stride, int page_size, int ring,
-                         const int32_t* seq_slot, const int32_t* slot_len, float* partial,
+                         const int32_t* seq_slot, const int32_t* seq_len, float* partial,
                          int nsplit, int B, int nh, int nkv, int hd, float scale, int window,
                          hipStream_t stream) {
     const int G = nh / nkv;
@@ -390,7 +390,7 @@ static int launch_decode(const void* qkv, void* out, const void* kcache, const v
     hipLaunchKernelGGL((attn_decode_bf16_kernel<LPR, GC>), dim3(nkv * chunks, B, nsplit), dim3(64),
                        0, stream, (const bf16_t*)qkv, (bf16_t*)out, (const bf16_t*)kcache,
                        (const bf16_t*)vcache, page_table, table_stride, page_size, ring, seq_slot,
-                       slot_len, partial, nsplit, nh, nkv, hd, scale, window);
+                       seq_len, partial, nsplit, nh, nkv, hd, scale, window);
     if (nsplit > 1)
         hipLaunchKernelGGL(attn_decode_bf16_merge_kernel, dim3(nh, B), dim3(64), 0, stream,
                            (const float*)partial, (bf16_t*)out, nsplit, nh, hd);
@@ -401,11 +401,11 @@ template <int LPR>
 static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcache,
                            const void* vcache, const int32_t* page_table, int table_stride,
                            int page_size, int ring, const int32_t* seq_slot,
-                           const int32_t* slot_len, float* partial, int nsplit, int B, int nh,
+                           const int32_t* seq_len, float* partial, int nsplit, int B, int nh,
                            int nkv, int hd, float scale, int window, hipStream_t stream) {
 #define GO(GC_)                                                                                   \
     return launch_decode<LPR, GC_>(qkv, out, kcache, vcache, page_table, table_stride, page_size, \
-                                   ring, seq_slot, slot_len, partial, nsplit, B, nh, nkv, hd,     \
+                                   ring, seq_slot, seq_len, partial, nsplit, B, nh, nkv, hd,     \
                                    scale, window, stream)
     switch (gc) {
         case 1: GO(1);
@@ -421,7 +421,7 @@ static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcach
 extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache,
                                      const void* vcache, const int32_t* page_table,
                                      int table_stride, int page_size, int ring,
-                                     const int32_t* seq_slot, const int32_t* slot_len,
+                                     const int32_t* seq_slot, const int32_t* seq_len,
                                      float* partial, int nsplit, int B, int nh, int nkv, int hd,
                                      float scale, int window, void* stream) {
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 || hd % 8 ||
@@ -439,7 +439,7 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
     hipLaunchKernelGGL((attn_decode_bf16_gqa_kernel<HD_, GC_>), grid, dim3(64), 0,                 \
                        (hipStream_t)stream, (const bf16_t*)qkv, (bf16_t*)out,                      \
                        (const bf16_t*)kcache, (const bf16_t*)vcache, page_table, table_stride,     \
-                       page_size, ring, seq_slot, slot_len, partial, nsplit, nh, nkv, scale, window)
+                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, scale, window)
 #define GQA_HD(HD_)                                                                                \
     do {                                                                                           \
         if (gcq == 2) GQA(HD_, 2);                                                                 \
@@ -472,7 +472,7 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
     hipStream_t st = (hipStream_t)stream;
 #define GO(LPR_)                                                                                   \
     return launch_decode_g<LPR_>(gc, qkv, out, kcache, vcache, page_table, table_stride, page_size, \
-                                 ring, seq_slot, slot_len, partial, nsplit, B, nh, nkv, hd, scale, \
+                                 ring, seq_slot, seq_len, partial, nsplit, B, nh, nkv, hd, scale, \
                                  window, st)
     switch (lpr) {
         case 1: GO(1);

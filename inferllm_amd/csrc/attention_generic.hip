@@ -148,7 +148,7 @@ attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __r
                            const void* __restrict__ vcache,
                            const int32_t* __restrict__ page_table, int table_stride,
                            int page_size, int ring, const int32_t* __restrict__ seq_slot,
-                           const int32_t* __restrict__ slot_len, float* __restrict__ partial,
+                           const int32_t* __restrict__ seq_len, float* __restrict__ partial,
                            int nsplit, int nh, int nkv, int hd, float scale, int window) {
     __shared__ float qs[256];
     __shared__ float ps[256];
@@ -156,7 +156,7 @@ attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __r
     const int h = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
     const int tid = threadIdx.x;
     const int slot = seq_slot[b];
-    const int len = slot_len[slot];
+    const int len = seq_len[b];
     const int kvh = h / (nh / nkv);
     const size_t rowlen = (size_t)(nh + 2 * nkv) * hd;
     const int k_first = window > 0 ? max(0, len - window) : 0;
@@ -234,7 +234,7 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ partial, void
 extern "C" int illm_attn_decode_generic(const void* qkv, void* out, int dt, const void* kcache,
                                         const void* vcache, const int32_t* page_table,
                                         int table_stride, int page_size, int ring,
-                                        const int32_t* seq_slot, const int32_t* slot_len,
+                                        const int32_t* seq_slot, const int32_t* seq_len,
                                         float* partial, int nsplit, int B, int nh, int nkv, int hd,
                                         float scale, int window, void* stream) {
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 || !illm_dtype_ok(dt) ||
@@ -243,7 +243,7 @@ extern "C" int illm_attn_decode_generic(const void* qkv, void* out, int dt, cons
     if (B == 0) return ILLM_OK;
     hipLaunchKernelGGL(attn_decode_generic_kernel, dim3(nh, B, nsplit), dim3(256), 0,
                        (hipStream_t)stream, qkv, dt, kcache, vcache, page_table, table_stride,
-                       page_size, ring, seq_slot, slot_len, partial, nsplit, nh, nkv, hd, scale,
+                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, hd, scale,
                        window);
     hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(nh, B), dim3(64), 0, (hipStream_t)stream,
                        (const float*)partial, out, dt, nsplit, nh, hd);

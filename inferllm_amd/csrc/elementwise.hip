@@ -243,7 +243,7 @@ __global__ void rope_store_kernel(void* __restrict__ qkv, int dt,
     if (h < nh || kcache == nullptr) return;
     const int kvh = h - nh;
     const int slot = row_slot[t];
-    if (ring > 0) {
+    if (ring > 0 && slot_len) {
         // a later row of this step lands on the same ring page: this one is already outside
         const int last_page = (slot_len[slot] - 1) / page_size;
         if (pos / page_size + ring <= last_page) return;
@@ -303,7 +303,7 @@ rope_store_bf16_kernel(bf16_t* __restrict__ qkv, const float* __restrict__ cos_s
     }
     if (kcache == nullptr) return;
     const int slot = row_slot[t];
-    if (ring > 0) {
+    if (ring > 0 && slot_len) {
         const int last_page = (slot_len[slot] - 1) / page_size;
         if (pos / page_size + ring <= last_page) return;
     }
@@ -329,7 +329,6 @@ extern "C" int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_
     if (pairing != 0 && pairing != 1) return ILLM_ERR_ARG;
     if (kcache && (!vcache || !page_table || !row_slot || page_size <= 0 || table_stride <= 0))
         return ILLM_ERR_ARG;
-    if (ring > 0 && !slot_len) return ILLM_ERR_ARG;
     if (nh + nkv > 65535) return ILLM_ERR_ARG;
     if (T == 0) return ILLM_OK;
     if (dt == ILLM_BF16 && hd % 16 == 0 && (!cos_sin || (pairing == 0 && rot == hd))) {

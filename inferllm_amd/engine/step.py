@@ -50,7 +50,12 @@ class _DecodeGraph:
     def __init__(self, runner: "StepRunner", size: int):
         self.size = size
         dev = runner.device
-        self.meta = torch.zeros(3 * size, dtype=torch.int32, device=dev)   # tokens | pos | slot
+        self.meta = torch.zeros(4 * size, dtype=torch.int32, device=dev)   # tokens | pos | slot | len
+        # host side of `meta`: pinned, so that one asynchronous copy brings a step's numbers over
+        self.stage = torch.zeros(4 * size, dtype=torch.int32, pin_memory=True)
+        self.stage_np = self.stage.numpy()
+        self.copied = torch.cuda.Event()
+        self.in_flight = False
         self.cu = torch.arange(size + 1, dtype=torch.int32, device=dev)
         self.rows = torch.arange(size, dtype=torch.int32, device=dev)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
@@ -60,9 +65,9 @@ class _DecodeGraph:
         n = self.size
         return StepContext(
             device=runner.device, act_dtype=runner.act_dtype, prefill=False, n_rows=n, n_seqs=n,
-            tokens=self.meta[:n], row_pos=self.meta[n:2 * n], row_slot=self.meta[2 * n:],
-            cu_seqlens=self.cu, seq_slot=self.meta[2 * n:], max_len=runner.cache.max_seq_len,
-            cache=runner.cache)
+            tokens=self.meta[:n], row_pos=self.meta[n:2 * n], row_slot=self.meta[2 * n:3 * n],
+            cu_seqlens=self.cu, seq_slot=self.meta[2 * n:3 * n], seq_len=self.meta[3 * n:],
+            max_len=runner.cache.max_seq_len, cache=runner.cache)
 
 
 class StepRunner:
@@ -113,7 +118,7 @@ class StepRunner:
         starts = [self.cache.length(e.slot) for e in entries]
         for e, s in zip(entries, starts):
             self.cache.extend(e.slot, s, len(e.tokens))
-        self.cache.upload()
+        self.cache.upload(lengths=prefill)
         if prefill:
             return self._prefill(entries)
         return self._decode(entries, starts)
@@ -132,42 +137,50 @@ class StepRunner:
             slot.extend([e.slot] * n)
             cu.append(cu[-1] + n)
         T, B = len(tokens), len(entries)
-        host = torch.tensor(tokens + pos + slot + cu + [e.slot for e in entries] + want,
-                            dtype=torch.int32)
+        host = torch.tensor(tokens + pos + slot + cu + [e.slot for e in entries]
+                            + [len(e.tokens) for e in entries] + want, dtype=torch.int32)
         meta = host.to(self.device)
         o = 0
         parts = []
-        for n in (T, T, T, B + 1, B, len(want)):
+        for n in (T, T, T, B + 1, B, B, len(want)):
             parts.append(meta[o:o + n])
             o += n
         ctx = StepContext(
             device=self.device, act_dtype=self.act_dtype, prefill=True, n_rows=T, n_seqs=B,
             tokens=parts[0], row_pos=parts[1], row_slot=parts[2], cu_seqlens=parts[3],
-            seq_slot=parts[4], max_len=max(len(e.tokens) for e in entries), cache=self.cache)
-        return self.model.forward(ctx, parts[5] if want else None)
+            seq_slot=parts[4], seq_len=parts[5], max_len=max(len(e.tokens) for e in entries),
+            cache=self.cache)
+        return self.model.forward(ctx, parts[6] if want else None)
 
     def _decode(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> Optional[torch.Tensor]:
         B = len(entries)
         size = _bucket(B) if self.use_graphs else B
         pad = size - B
         spare = self.cache.spare_slot
-        host = torch.tensor([int(e.tokens[0]) for e in entries] + [0] * pad
-                            + list(starts) + [0] * pad
-                            + [e.slot for e in entries] + [spare] * pad, dtype=torch.int32)
+        host = ([int(e.tokens[0]) for e in entries] + [0] * pad
+                + list(starts) + [0] * pad
+                + [e.slot for e in entries] + [spare] * pad
+                + [s + 1 for s in starts] + [1] * pad)          # a padding row sees one (spare) key
         wanted = [i for i, e in enumerate(entries) if len(e.want)]
         if not self.use_graphs:
-            meta = host.to(self.device)
+            meta = torch.tensor(host, dtype=torch.int32).to(self.device)
             ctx = StepContext(
                 device=self.device, act_dtype=self.act_dtype, prefill=False, n_rows=B, n_seqs=B,
-                tokens=meta[:B], row_pos=meta[B:2 * B], row_slot=meta[2 * B:],
+                tokens=meta[:B], row_pos=meta[B:2 * B], row_slot=meta[2 * B:3 * B],
                 cu_seqlens=torch.arange(B + 1, dtype=torch.int32, device=self.device),
-                seq_slot=meta[2 * B:], max_len=max(starts) + 1, cache=self.cache)
+                seq_slot=meta[2 * B:3 * B], seq_len=meta[3 * B:], max_len=max(starts) + 1,
+                cache=self.cache)
             rows = torch.tensor(wanted, dtype=torch.int32, device=self.device) if wanted else None
             return self.model.forward(ctx, rows)
         g = self._graphs.get(size)
         if g is None:
             g = self._graphs[size] = _DecodeGraph(self, size)
-        g.meta.copy_(host)
+        if g.in_flight:
+            g.copied.synchronize()          # the last step's copy has left the pinned buffer
+        g.stage_np[:] = host
+        g.meta.copy_(g.stage, non_blocking=True)
+        g.copied.record()
+        g.in_flight = True
         if g.graph is None:
             self._capture(g)
         g.graph.replay()

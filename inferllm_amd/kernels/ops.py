@@ -298,11 +298,12 @@ def decode_splits(B: int, nh: int, max_len: int) -> int:
 
 def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                 page_table: torch.Tensor, page_size: int, ring: int, seq_slot: torch.Tensor,
-                slot_len: torch.Tensor, nh: int, nkv: int, hd: int, scale: float, window: int,
+                seq_len: torch.Tensor, nh: int, nkv: int, hd: int, scale: float, window: int,
                 nsplit: int) -> torch.Tensor:
-    """One new token per sequence against the paged cache; returns [B, nh * hd]."""
-    _gpu(qkv, kcache, vcache, page_table, seq_slot, slot_len)
-    _i32(page_table); _i32(seq_slot, qkv.shape[0]); _i32(slot_len)
+    """One new token per sequence against the paged cache; returns [B, nh * hd].
+    seq_len[b]: keys of sequence b, the new one included."""
+    _gpu(qkv, kcache, vcache, page_table, seq_slot, seq_len)
+    _i32(page_table); _i32(seq_slot, qkv.shape[0]); _i32(seq_len, qkv.shape[0])
     B = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_decode: packed qkv rows")
     _need(kcache.dtype == qkv.dtype and vcache.shape == kcache.shape and
@@ -314,13 +315,13 @@ def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                    if nsplit > 1 else None)
         _check(_lib().illm_attn_decode_bf16(
             _p(qkv), _p(out), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
-            page_size, ring, _p(seq_slot), _p(slot_len), _p(partial), nsplit, B, nh, nkv, hd,
+            page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh, nkv, hd,
             ctypes.c_float(scale), window, _stream()), f"attn_decode_bf16 (head_dim {hd})")
         return out
     partial = torch.empty((B, nh, nsplit, hd + 2), dtype=torch.float32, device=qkv.device)
     _check(_lib().illm_attn_decode_generic(
         _p(qkv), _p(out), _code(qkv), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
-        page_size, ring, _p(seq_slot), _p(slot_len), _p(partial), nsplit, B, nh, nkv, hd,
+        page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh, nkv, hd,
         ctypes.c_float(scale), window, _stream()), f"attn_decode (head_dim {hd})")
     return out
 

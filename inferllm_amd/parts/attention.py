@@ -66,7 +66,7 @@ class Attention(Mixer):
                 qkv = position.project_qkv(h, self.w_qkv, ctx, nh, nkv, hd, kc, vc, group)
             else:
                 qkv = ops.linear(h, self.w_qkv)
-                ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot, ctx.cache.slot_len, kc,
+                ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot, ctx.cache.slot_len if ctx.prefill else None, kc,
                                vc, group.table, group.page_size, group.ring, nh, nkv, hd)
             if ctx.prefill:
                 ctx.exchange[("kv_rows", line)] = qkv
@@ -87,7 +87,7 @@ class Attention(Mixer):
         else:
             nsplit = ops.decode_splits(ctx.n_seqs, nkv, ctx.max_len if not window else min(ctx.max_len, window))
             o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
-                                ctx.seq_slot, ctx.cache.slot_len, nh, nkv, hd, self.scale, window,
+                                ctx.seq_slot, ctx.seq_len, nh, nkv, hd, self.scale, window,
                                 nsplit)
         return ops.linear(o, self.w_o)
 

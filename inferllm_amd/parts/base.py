@@ -42,6 +42,7 @@ class StepContext:
     row_slot: torch.Tensor            # [rows] cache slot of each row
     cu_seqlens: torch.Tensor          # [seqs + 1] row offsets of the sequences
     seq_slot: torch.Tensor            # [seqs]
+    seq_len: torch.Tensor             # [seqs] length of each sequence after this step
     max_len: int                      # longest sequence after this step (host number)
     cache: CacheManager
     exchange: Dict[Any, Any] = field(default_factory=dict)   # between runs of layers in one step

@@ -57,7 +57,7 @@ class Rotary(PositionEncoding):
     def on_qkv(self, qkv, ctx: StepContext, nh, nkv, hd, kcache, vcache, group) -> None:
         ops.rope_store(qkv, self.table(ctx.device), self.rotary_dim,
                        0 if self.pairing == "half" else 1, ctx.row_pos, ctx.row_slot,
-                       ctx.cache.slot_len, kcache, vcache,
+                       ctx.cache.slot_len if ctx.prefill else None, kcache, vcache,
                        group.table if group is not None else None,
                        group.page_size if group is not None else 1,
                        group.ring if group is not None else 0, nh, nkv, hd)
@@ -78,7 +78,8 @@ class NoPosition(PositionEncoding):
     """No encoding: q and k stay as they are; k and v are still stored."""
 
     def on_qkv(self, qkv, ctx: StepContext, nh, nkv, hd, kcache, vcache, group) -> None:
-        ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot, ctx.cache.slot_len, kcache,
+        ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot,
+                       ctx.cache.slot_len if ctx.prefill else None, kcache,
                        vcache, group.table if group is not None else None,
                        group.page_size if group is not None else 1,
                        group.ring if group is not None else 0, nh, nkv, hd)

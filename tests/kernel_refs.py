@@ -70,7 +70,7 @@ def rope_store(qkv, cos_sin, rot, pairing, row_pos, row_slot, slot_len, kcache, 
         return
     for t in range(T):
         slot, pos = int(row_slot[t]), int(row_pos[t])
-        if ring > 0:
+        if ring > 0 and slot_len is not None:
             last_page = (int(slot_len[slot]) - 1) // page_size
             if pos // page_size + ring <= last_page:
                 continue
@@ -128,14 +128,14 @@ def decode_splits(B, nh, max_len):
     return 2
 
 
-def attn_decode(qkv, kcache, vcache, page_table, page_size, ring, seq_slot, slot_len, nh, nkv, hd,
+def attn_decode(qkv, kcache, vcache, page_table, page_size, ring, seq_slot, seq_len, nh, nkv, hd,
                 scale, window, nsplit):
     B = qkv.shape[0]
     view = qkv.view(B, nh + 2 * nkv, hd)
     out = torch.zeros(B, nh * hd, dtype=qkv.dtype, device=qkv.device)
     for b in range(B):
         slot = int(seq_slot[b])
-        n = int(slot_len[slot])
+        n = int(seq_len[b])
         first = max(0, n - window) if window and window > 0 else 0
         ks, vs = [], []
         for pos in range(first, n):

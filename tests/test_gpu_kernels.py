@@ -212,10 +212,7 @@ def paged_case(dtype, nkv, hd, lens, page, ring=0, seed=3):
     for b, s in enumerate(slots):
         pt[s] = perm[b].to(torch.int32)
     kc, vc = rnd(n_pages, nkv, page, hd, dtype=dtype, seed=seed + 1), rnd(n_pages, nkv, page, hd, dtype=dtype, seed=seed + 2)
-    slot_len = torch.zeros(B + 2, dtype=torch.int32)
-    for b, s in enumerate(slots):
-        slot_len[s] = lens[b]
-    return pt, kc, vc, torch.tensor(slots, dtype=torch.int32), slot_len
+    return pt, kc, vc, torch.tensor(slots, dtype=torch.int32), torch.tensor(lens, dtype=torch.int32)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -228,13 +225,13 @@ def test_attn_decode(dtype, nh, nkv, hd, lens, window, nsplit):
     ring = 0
     if window:
         ring = (window + page - 2) // page + 1
-    pt, kc, vc, slots, slot_len = paged_case(dtype, nkv, hd, lens, page, ring)
+    pt, kc, vc, slots, seq_len = paged_case(dtype, nkv, hd, lens, page, ring)
     B = len(lens)
     qkv = rnd(B, (nh + 2 * nkv) * hd, dtype=dtype, seed=11)
     scale = 1.0 / math.sqrt(hd)
     got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring, slots.to(DEV),
-                            slot_len.to(DEV), nh, nkv, hd, scale, window, nsplit)
-    want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, slot_len, nh, nkv, hd, scale, window, nsplit)
+                            seq_len.to(DEV), nh, nkv, hd, scale, window, nsplit)
+    want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, seq_len, nh, nkv, hd, scale, window, nsplit)
     close(got, want, dtype, scale=2)
 
 
@@ -249,7 +246,7 @@ def test_attn_decode_bf16_pages_of_64(nh, nkv, hd, lens, window, nsplit):
     of the pages are NaN and must not leak into the result."""
     dtype, page = torch.bfloat16, 64
     ring = (window + page - 2) // page + 1 if window else 0
-    pt, kc, vc, slots, slot_len = paged_case(dtype, nkv, hd, lens, page, ring)
+    pt, kc, vc, slots, seq_len = paged_case(dtype, nkv, hd, lens, page, ring)
     for b, s in enumerate(slots.tolist()):
         n = lens[b]
         if not ring:
@@ -261,8 +258,8 @@ def test_attn_decode_bf16_pages_of_64(nh, nkv, hd, lens, window, nsplit):
     qkv = rnd(B, (nh + 2 * nkv) * hd, dtype=dtype, seed=11)
     scale = 1.0 / math.sqrt(hd)
     got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring, slots.to(DEV),
-                            slot_len.to(DEV), nh, nkv, hd, scale, window, nsplit)
-    want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, slot_len, nh, nkv, hd, scale, window, nsplit)
+                            seq_len.to(DEV), nh, nkv, hd, scale, window, nsplit)
+    want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, seq_len, nh, nkv, hd, scale, window, nsplit)
     close(got, want, dtype, scale=2)
 
 
@@ -294,7 +291,7 @@ def test_gate_up_silu(M, F, K):
 def test_attn_decode_finds_one_far_key(dtype):
     """One key among hundreds is made to stand out: the output must be its value."""
     nh, nkv, hd, page, n = 4, 2, 32, 16, 777
-    pt, kc, vc, slots, slot_len = paged_case(dtype, nkv, hd, [n], page)
+    pt, kc, vc, slots, seq_len = paged_case(dtype, nkv, hd, [n], page)
     qkv = rnd(1, (nh + 2 * nkv) * hd, dtype=dtype, seed=1)
     target = 5
     pg, r = R.cache_offsets(pt, int(slots[0]), target, page, 0)
@@ -302,7 +299,7 @@ def test_attn_decode_finds_one_far_key(dtype):
     for kvh in range(nkv):
         kc[pg, kvh, r] = q[0, kvh * (nh // nkv)].float().mul(40).to(dtype)   # huge score for head kvh*per
     got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, 0, slots.to(DEV),
-                            slot_len.to(DEV), nh, nkv, hd, 1.0, 0, 4).cpu().view(nh, hd)
+                            seq_len.to(DEV), nh, nkv, hd, 1.0, 0, 4).cpu().view(nh, hd)
     for kvh in range(nkv):
         close(got[kvh * (nh // nkv)], vc[pg, kvh, r], dtype)
 

@@ -43,7 +43,8 @@ def step_ctx(cache, slots, starts, counts, dtype, prefill):
     i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
     return StepContext(device=DEV, act_dtype=dtype, prefill=prefill, n_rows=len(pos), n_seqs=len(slots),
                        tokens=i32([0] * len(pos)), row_pos=i32(pos), row_slot=i32(slot), cu_seqlens=i32(cu),
-                       seq_slot=i32(slots), max_len=max(a + n for a, n in zip(starts, counts)), cache=cache)
+                       seq_slot=i32(slots), seq_len=i32([a + n for a, n in zip(starts, counts)]),
+                       max_len=max(a + n for a, n in zip(starts, counts)), cache=cache)
 
 
 TOL = {torch.float32: 2e-5, torch.bfloat16: 3e-2}
