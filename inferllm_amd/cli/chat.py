@@ -128,11 +128,19 @@ def main(argv=None) -> int:
     stops = parse_ids(args.stop_ids) if args.stop_ids else None
 
     def run(prompts: List[List[int]]) -> None:
+        stream = len(prompts) == 1 and text.tok is None     # one request of ids: print as they come
+
+        def show(i: int, tok: int) -> None:
+            print(tok, end=" ", flush=True)
         outs = eng.generate(prompts, temperature=args.temp, top_k=args.top_k, top_p=args.top_p,
                             repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n,
-                            seed=seed, max_new_tokens=args.n_predict, stop_token_ids=stops)
-        for o in outs:
-            print(text.show(o), flush=True)
+                            seed=seed, max_new_tokens=args.n_predict, stop_token_ids=stops,
+                            on_token=show if stream else None)
+        if stream:
+            print(flush=True)
+        else:
+            for o in outs:
+                print(text.show(o), flush=True)
         if args.summary:
             print(eng.last_stats.summary(), file=sys.stderr, flush=True)
 

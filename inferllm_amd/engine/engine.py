@@ -109,11 +109,13 @@ class Engine:
                  top_k: int = 0, top_p: float = 1.0, repeat_penalty: float = 1.0,
                  repeat_last_n: int = 64, seed: int = 0, max_new_tokens: int = 128,
                  stop_token_ids: Optional[Sequence[int]] = None,
-                 include_stop: bool = False) -> List[List[int]]:
+                 include_stop: bool = False, on_token=None) -> List[List[int]]:
         """Generated token ids for every prompt (lists of token ids).
 
         `stop_token_ids` defaults to the model's eos ids; a stop token ends its
-        sequence and is left out of the result unless `include_stop`."""
+        sequence and is left out of the result unless `include_stop`.  `on_token(request
+        index, token)` is called for every token as it is generated (the reference prints
+        tokens as they come, application/chat.cpp:232-236)."""
         params = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p,
                                 repeat_penalty=repeat_penalty, repeat_last_n=repeat_last_n,
                                 seed=seed)
@@ -127,7 +129,7 @@ class Engine:
         loop = GenerationLoop(self.step, sampler, self.alloc_slot, self.free_slot,
                               max_batch=self.max_batch, max_tokens=self.cache.max_tokens,
                               max_seq_len=self.max_seq_len, page_size=self.cache.page_size,
-                              sync=lambda: torch.cuda.synchronize(self.device))
+                              sync=lambda: torch.cuda.synchronize(self.device), on_token=on_token)
         out = loop.run(prompts, params, max_new_tokens, stops, include_stop)
         self.last_stats = loop.stats
         return out

@@ -60,12 +60,14 @@ class GenerationLoop:
 
     def __init__(self, step: Callable, sample: Callable, alloc_slot: Callable[[], int],
                  free_slot: Callable[[int], None], max_batch: int, max_tokens: int,
-                 max_seq_len: int, page_size: int = 64, sync: Optional[Callable[[], None]] = None):
+                 max_seq_len: int, page_size: int = 64, sync: Optional[Callable[[], None]] = None,
+                 on_token: Optional[Callable[[int, int], None]] = None):
         self.step, self.sample = step, sample
         self.alloc_slot, self.free_slot = alloc_slot, free_slot
         self.max_batch, self.max_tokens, self.max_seq_len = max_batch, max_tokens, max_seq_len
         self.page_size = page_size
         self.sync = sync or (lambda: None)
+        self.on_token = on_token            # called with (request index, token) as tokens are kept
         self.stats = GenerationStats()
 
     # ------------------------------------------------------------ decisions
@@ -153,6 +155,8 @@ class GenerationLoop:
                                      max_new_tokens, self.max_seq_len)
                     if why != "stop" or include_stop:
                         s.out.append(tok)
+                        if self.on_token is not None:
+                            self.on_token(s.index, tok)
                     s.history.append(tok)
                     if why is None:
                         going.append(s)

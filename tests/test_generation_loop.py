@@ -147,3 +147,15 @@ def test_sampling_params_validation():
         with pytest.raises(ValueError):
             SamplingParams(**bad).validate()
     assert SamplingParams().greedy and not SamplingParams(temperature=0.1).greedy
+
+
+def test_tokens_are_reported_as_they_are_kept():
+    seen = []
+    m = FakeModel(3)
+    loop = GenerationLoop(m.step, m.sample, m.alloc, m.release, 3, 6400, 256,
+                          on_token=lambda i, t: seen.append((i, t)))
+    stops = {expected(PROMPTS[0], 6)[2]}
+    out = loop.run(PROMPTS[:3], SamplingParams(), 4, stops)
+    for i in range(3):
+        assert [t for j, t in seen if j == i] == out[i]
+    assert [i for i, _ in seen[:3]] == [0, 1, 2]          # step by step, not request by request
