@@ -66,34 +66,28 @@ class Attention(Mixer):
                 qkv = position.project_qkv(h, self.w_qkv, ctx, nh, nkv, hd, kc, vc, group)
             else:
                 qkv = ops.linear(h, self.w_qkv)
-                ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot, ctx.cache.slot_len if ctx.prefill else None, kc,
-                               vc, group.table, group.page_size, group.ring, nh, nkv, hd)
+                ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot,
+                               ctx.cache.slot_len if ctx.prefill else None, kc, vc, group.table,
+                               group.page_size, group.ring, nh, nkv, hd)
             if ctx.prefill:
-                ctx.exchange[("kv_rows", line)] = qkv
+                ctx.exchange[("kv_rows", line)] = qkv      # for runs that read this cache line
         else:
-            # keys and values are those that an earlier run of this step stored on the line
+            # keys and values are those an earlier run of this step stored on the line: only q
+            # is projected and encoded (as packed rows with no kv heads)
             q = ops.linear(h, self.w_qkv[: nh * hd])
-            if ctx.prefill:
-                src = ctx.exchange[("kv_rows", line)]
-                qkv = torch.cat([q, src[:, nh * hd:]], dim=1)
-            else:
-                qkv = torch.cat([q, q.new_zeros((q.shape[0], 2 * nkv * hd))], dim=1)
             if position is not None:
-                # rotates q (and the copied k again is avoided by handing no k heads: see below)
-                self._encode_q_only(qkv, ctx, position)
+                position.on_qkv(q, ctx, nh, 0, hd, None, None, None)
+            if ctx.prefill:
+                kv = ctx.exchange[("kv_rows", line)][:, nh * hd:]
+            else:
+                kv = q.new_zeros((q.shape[0], 2 * nkv * hd))   # single tokens read the cache
+            qkv = torch.cat([q, kv], dim=1)
         if ctx.prefill:
             o = ops.attn_prefill(qkv, ctx.cu_seqlens, ctx.n_seqs, ctx.max_len, nh, nkv, hd,
                                  self.scale, window)
         else:
-            nsplit = ops.decode_splits(ctx.n_seqs, nkv, ctx.max_len if not window else min(ctx.max_len, window))
+            longest = min(ctx.max_len, window) if window else ctx.max_len
             o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
                                 ctx.seq_slot, ctx.seq_len, nh, nkv, hd, self.scale, window,
-                                nsplit)
+                                ops.decode_splits(ctx.n_seqs, nkv, longest))
         return ops.linear(o, self.w_o)
-
-    def _encode_q_only(self, qkv, ctx, position) -> None:
-        nh, nkv, hd = self.nh, self.nkv, self.hd
-        q = qkv[:, : nh * hd].contiguous()
-        # a q-only view: rows of nh heads and no kv heads
-        position.on_qkv(q, ctx, nh, 0, hd, None, None, None)
-        qkv[:, : nh * hd] = q
