@@ -60,12 +60,13 @@ int illm_attn_decode_generic(const void* qkv, void* out, int dt, const void* kca
                              int nkv, int hd, float scale, int window, void* stream);
 
 // The same for bfloat16 with head_dim % 8 == 0 and page_size % 64 == 0 (anything else:
-// ILLM_ERR_ARG); nsplit == 1 needs no `partial`.
+// ILLM_ERR_ARG); nsplit == 1 needs no `partial`.  `waves`: waves per block that share a key
+// range and combine through LDS (clamped to what the head group's registers and LDS allow).
 int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache, const void* vcache,
                           const int32_t* page_table, int table_stride, int page_size, int ring,
                           const int32_t* seq_slot, const int32_t* seq_len, float* partial,
-                          int nsplit, int B, int nh, int nkv, int hd, float scale, int window,
-                          void* stream);
+                          int nsplit, int waves, int B, int nh, int nkv, int hd, float scale,
+                          int window, void* stream);
 
 // Y[M, N] = X[M, K] . W[N, K]^T for bfloat16 X and W, 1 <= M <= 64, K % 8 == 0, on the
 // matrix cores with float32 accumulation; Y float32 or bfloat16.

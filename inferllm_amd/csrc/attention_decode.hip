@@ -7,8 +7,9 @@
 // instruction, and a tile's loads are all issued before any is used.  Scores are
 // reduced over the LPR lanes of a row, the running max / sum are wave-wide, and
 // each lane accumulates P.V for its 8 dims over the keys of its row group; the
-// groups are added once at the end.  Splits of the key range run as separate
-// one-wave blocks and leave (acc, max, sum) for the merge kernel.
+// groups are added once at the end.  The waves of a block take the tiles of their key range
+// in turn and combine their results through LDS; splits of the key range across blocks
+// (for few sequences) leave (acc, max, sum) for the merge kernel.
 //
 // Same chain as src/core/op.cpp:485-498 with S = 1, grouped as
 // src/kern/naive/naive.cpp:576-604.
@@ -29,7 +30,7 @@ __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
 // LPR: lanes per key row (power of two, 8 dims each, LPR * 8 >= head_dim).
 // GC: query heads handled together (power of two >= heads per kv head, at most 8).
 template <int LPR, int GC>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(GC <= 4 ? 512 : 256)
 attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
                         const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                         const int32_t* __restrict__ page_table, int table_stride, int page_size,
@@ -39,7 +40,9 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     constexpr int KPI = 64 / LPR;              // keys per load instruction
     constexpr int NI = LPR < 16 ? LPR : 16;    // load instructions per tile
     constexpr int TK = NI * KPI;               // keys per tile
-    const int lane = threadIdx.x, q = lane / LPR, c = lane % LPR;
+    extern __shared__ float wave_res[];        // [waves][GC][hd + 2], used when waves > 1
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int q = lane / LPR, c = lane % LPR;
     const int G = nh / nkv;
     const int kvh = blockIdx.x % nkv, g0 = (blockIdx.x / nkv) * GC;
     const int b = blockIdx.y, sp = blockIdx.z;
@@ -72,7 +75,7 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     const int t_lo = t_first + sp * per;
     const int t_hi = min(t_first + n_tiles, t_lo + per);
 
-    for (int t = t_lo; t < t_hi; ++t) {
+    for (int t = t_lo + wave; t < t_hi; t += waves) {
         const int k0 = t * TK;
         int lp = k0 / page_size;
         if (ring > 0) lp %= ring;
@@ -147,6 +150,47 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
             for (int o = LPR; o < 64; o <<= 1) a += __shfl_xor(a, o, ILLM_WAVE);
             acc[g][i] = a;
         }
+    if (waves > 1) {
+        // every wave leaves its result in LDS; wave 0 combines them
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            float* wr = wave_res + (size_t)(wave * GC + g) * (hd + 2);
+            if (q == 0 && dim_ok) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) wr[c * 8 + i] = acc[g][i];
+            }
+            if (lane == 0) {
+                wr[hd] = m[g];
+                wr[hd + 1] = l[g];
+            }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            float mm = NEG_INF;
+            for (int w = 0; w < waves; ++w)
+                mm = fmaxf(mm, wave_res[(size_t)(w * GC + g) * (hd + 2) + hd]);
+            float L = 0.f, a[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a[i] = 0.f;
+            for (int w = 0; w < waves; ++w) {
+                const float* wr = wave_res + (size_t)(w * GC + g) * (hd + 2);
+                const float mw = wr[hd];
+                if (mw == NEG_INF) continue;
+                const float wgt = expf(mw - mm);
+                L += wgt * wr[hd + 1];
+                if (q == 0 && dim_ok) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) a[i] = fmaf(wgt, wr[c * 8 + i], a[i]);
+                }
+            }
+            m[g] = mm;
+            l[g] = L;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] = a[i];
+        }
+    }
 #pragma unroll
     for (int g = 0; g < GC; ++g) {
         if (g0 + g >= G) continue;
@@ -185,7 +229,7 @@ typedef __bf16 dbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float df32x4_t __attribute__((ext_vector_type(4)));
 
 template <int HD, int GC>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(GC <= 4 ? 512 : (GC <= 8 ? 256 : 128))
 attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
                             const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                             const int32_t* __restrict__ page_table, int table_stride,
@@ -199,8 +243,10 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
     constexpr int NSUB = TK / 16;              // MFMA sub-tiles of 16 keys
     constexpr int KS = HD / 32;                // k-steps of 32 dims
     constexpr int PLD = 20;                    // floats per key row of P in LDS (16 heads + pad)
-    __shared__ __attribute__((aligned(16))) float ps[64 * PLD];
-    const int lane = threadIdx.x;
+    // per wave 64 * PLD floats of P; after the tiles the same memory holds the waves' results
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    float* ps = lds + (size_t)wave * 64 * PLD;
     const int r = lane & 15, q4 = lane >> 4;   // MFMA roles: key / head, and k group
     const int q = lane / LPR, c = lane % LPR;  // V row roles
     const int G = nh / nkv;
@@ -235,7 +281,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
     const int t_lo = t_first + sp * per;
     const int t_hi = min(t_first + n_tiles, t_lo + per);
 
-    for (int t = t_lo; t < t_hi; ++t) {
+    for (int t = t_lo + wave; t < t_hi; t += waves) {
         const int k0 = t * TK;
         int lp = k0 / page_size;
         if (ring > 0) lp %= ring;
@@ -275,7 +321,9 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
         const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
         const float alpha = expf(m - m_use);             // m = -inf gives 0 (nothing summed yet)
         float rs = 0.f;
-        __syncthreads();                                  // the last tile's P has been read
+        // P is private to the wave, whose LDS accesses run in program order: no barrier, only
+        // a fence for the compiler
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int sub = 0; sub < NSUB; ++sub)
 #pragma unroll
@@ -288,7 +336,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
         rs += __shfl_xor(rs, 32, ILLM_WAVE);
         l = l * alpha + rs;
         m = m_new;
-        __syncthreads();
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int g = 0; g < GC; ++g) {
             const float ag = __shfl(alpha, g, ILLM_WAVE);  // lane g holds head g's factor
@@ -325,14 +373,59 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
             for (int o = LPR; o < 64; o <<= 1) a += __shfl_xor(a, o, ILLM_WAVE);
             acc[g][i] = a;
         }
+    float lg[GC], mg[GC];
 #pragma unroll
     for (int g = 0; g < GC; ++g) {
-        const float lg = __shfl(l, g, ILLM_WAVE), mg = __shfl(m, g, ILLM_WAVE);
+        lg[g] = __shfl(l, g, ILLM_WAVE);
+        mg[g] = __shfl(m, g, ILLM_WAVE);
+    }
+    if (waves > 1) {
+        __syncthreads();                       // every wave is done with its P
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            float* wr = lds + (size_t)(wave * GC + g) * (HD + 2);
+            if (q == 0 && dim_ok) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) wr[c * 8 + i] = acc[g][i];
+            }
+            if (lane == 0) {
+                wr[HD] = mg[g];
+                wr[HD + 1] = lg[g];
+            }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            float mm = NEG_INF;
+            for (int w = 0; w < waves; ++w) mm = fmaxf(mm, lds[(size_t)(w * GC + g) * (HD + 2) + HD]);
+            float L = 0.f, a[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a[i] = 0.f;
+            for (int w = 0; w < waves; ++w) {
+                const float* wr = lds + (size_t)(w * GC + g) * (HD + 2);
+                const float mw = wr[HD];
+                if (mw == NEG_INF) continue;
+                const float wgt = expf(mw - mm);
+                L += wgt * wr[HD + 1];
+                if (q == 0 && dim_ok) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) a[i] = fmaf(wgt, wr[c * 8 + i], a[i]);
+                }
+            }
+            mg[g] = mm;
+            lg[g] = L;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[g][i] = a[i];
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
         if (g0 + g >= G) continue;
         const int h = kvh * G + g0 + g;
         if (nsplit == 1) {
             if (q == 0 && dim_ok) {
-                const float inv = 1.0f / lg;
+                const float inv = 1.0f / lg[g];
                 uint4 o;
                 o.x = pack_bf16x2(acc[g][0] * inv, acc[g][1] * inv);
                 o.y = pack_bf16x2(acc[g][2] * inv, acc[g][3] * inv);
@@ -347,8 +440,8 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
                 for (int i = 0; i < 8; ++i) pp[c * 8 + i] = acc[g][i];
             }
             if (lane == 0) {
-                pp[HD] = mg;
-                pp[HD + 1] = lg;
+                pp[HD] = mg[g];
+                pp[HD + 1] = lg[g];
             }
         }
     }
@@ -383,12 +476,15 @@ template <int LPR, int GC>
 static int launch_decode(const void* qkv, void* out, const void* kcache, const void* vcache,
                          const int32_t* page_table, int table_stride, int page_size, int ring,
                          const int32_t* seq_slot, const int32_t* seq_len, float* partial,
-                         int nsplit, int B, int nh, int nkv, int hd, float scale, int window,
-                         hipStream_t stream) {
+                         int nsplit, int waves, int B, int nh, int nkv, int hd, float scale,
+                         int window, hipStream_t stream) {
     const int G = nh / nkv;
     const int chunks = (G + GC - 1) / GC;
-    hipLaunchKernelGGL((attn_decode_bf16_kernel<LPR, GC>), dim3(nkv * chunks, B, nsplit), dim3(64),
-                       0, stream, (const bf16_t*)qkv, (bf16_t*)out, (const bf16_t*)kcache,
+    const int maxw = GC <= 4 ? 8 : 4;
+    waves = waves < 1 ? 1 : (waves > maxw ? maxw : waves);
+    const size_t smem = waves > 1 ? (size_t)waves * GC * (hd + 2) * sizeof(float) : 0;
+    hipLaunchKernelGGL((attn_decode_bf16_kernel<LPR, GC>), dim3(nkv * chunks, B, nsplit),
+                       dim3(64 * waves), smem, stream, (const bf16_t*)qkv, (bf16_t*)out, (const bf16_t*)kcache,
                        (const bf16_t*)vcache, page_table, table_stride, page_size, ring, seq_slot,
                        seq_len, partial, nsplit, nh, nkv, hd, scale, window);
     if (nsplit > 1)
@@ -401,12 +497,12 @@ template <int LPR>
 static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcache,
                            const void* vcache, const int32_t* page_table, int table_stride,
                            int page_size, int ring, const int32_t* seq_slot,
-                           const int32_t* seq_len, float* partial, int nsplit, int B, int nh,
-                           int nkv, int hd, float scale, int window, hipStream_t stream) {
+                           const int32_t* seq_len, float* partial, int nsplit, int waves, int B,
+                           int nh, int nkv, int hd, float scale, int window, hipStream_t stream) {
 #define GO(GC_)                                                                                   \
     return launch_decode<LPR, GC_>(qkv, out, kcache, vcache, page_table, table_stride, page_size, \
-                                   ring, seq_slot, seq_len, partial, nsplit, B, nh, nkv, hd,     \
-                                   scale, window, stream)
+                                   ring, seq_slot, seq_len, partial, nsplit, waves, B, nh, nkv,  \
+                                   hd, scale, window, stream)
     switch (gc) {
         case 1: GO(1);
         case 2: GO(2);
@@ -418,12 +514,14 @@ static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcach
 
 // Sizes this kernel takes: bfloat16, head_dim a multiple of 8 up to 256, a page size that
 // is a multiple of 64.  Anything else: ILLM_ERR_ARG (the caller uses the generic kernel).
+// `waves`: waves per block that share a key range (clamped to what registers and LDS allow);
+// `nsplit`: key ranges per sequence, combined by the merge kernel when > 1.
 extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache,
                                      const void* vcache, const int32_t* page_table,
                                      int table_stride, int page_size, int ring,
                                      const int32_t* seq_slot, const int32_t* seq_len,
-                                     float* partial, int nsplit, int B, int nh, int nkv, int hd,
-                                     float scale, int window, void* stream) {
+                                     float* partial, int nsplit, int waves, int B, int nh, int nkv,
+                                     int hd, float scale, int window, void* stream) {
     if (B < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 || hd % 8 ||
         page_size <= 0 || page_size % 64 || nsplit <= 0 || nsplit > 64 || B > 65535 ||
         table_stride <= 0 || (nsplit > 1 && !partial))
@@ -435,8 +533,19 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
         while (gcq < G && gcq < 16) gcq <<= 1;
         const int chunks = (G + gcq - 1) / gcq;
         const dim3 grid(nkv * chunks, B, nsplit);
+        // waves of a block: bounded by the registers a head group needs and by 64 KB of LDS
+        int wq = waves < 1 ? 1 : waves;
+        const int maxw = gcq <= 4 ? 8 : (gcq <= 8 ? 4 : 2);
+        wq = wq > maxw ? maxw : wq;
+        size_t smem = 0;
+        for (;; --wq) {
+            const size_t p_bytes = (size_t)wq * 64 * 20 * sizeof(float);
+            const size_t r_bytes = wq > 1 ? (size_t)wq * gcq * (hd + 2) * sizeof(float) : 0;
+            smem = p_bytes > r_bytes ? p_bytes : r_bytes;
+            if (smem <= 64 * 1024 || wq == 1) break;
+        }
 #define GQA(HD_, GC_)                                                                              \
-    hipLaunchKernelGGL((attn_decode_bf16_gqa_kernel<HD_, GC_>), grid, dim3(64), 0,                 \
+    hipLaunchKernelGGL((attn_decode_bf16_gqa_kernel<HD_, GC_>), grid, dim3(64 * wq), smem,         \
                        (hipStream_t)stream, (const bf16_t*)qkv, (bf16_t*)out,                      \
                        (const bf16_t*)kcache, (const bf16_t*)vcache, page_table, table_stride,     \
                        page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, scale, window)
@@ -472,8 +581,8 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
     hipStream_t st = (hipStream_t)stream;
 #define GO(LPR_)                                                                                   \
     return launch_decode_g<LPR_>(gc, qkv, out, kcache, vcache, page_table, table_stride, page_size, \
-                                 ring, seq_slot, seq_len, partial, nsplit, B, nh, nkv, hd, scale, \
-                                 window, st)
+                                 ring, seq_slot, seq_len, partial, nsplit, waves, B, nh, nkv, hd,  \
+                                 scale, window, st)
     switch (lpr) {
         case 1: GO(1);
         case 2: GO(2);

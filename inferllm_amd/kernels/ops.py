@@ -288,20 +288,24 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
     return out
 
 
-def decode_splits(B: int, nh: int, max_len: int) -> int:
-    """How many ways to cut the keys of a decode step so that the launch fills the chip."""
-    blocks = max(1, B * nh)
-    want = max(1, -(-2048 // blocks))
+def decode_splits(B: int, nkv: int, max_len: int):
+    """(nsplit, waves): how to cut the keys of a decode step so that about 2048 waves are at
+    work: first among the waves of a block (no second kernel), then among blocks."""
+    blocks = max(1, B * nkv)
     tiles = max(1, (max_len + 63) // 64)
-    return max(1, min(want, tiles, 32))
+    want = max(1, min(-(-2048 // blocks), tiles))
+    waves = min(8, want)
+    return max(1, min(-(-want // waves), 32)), waves
 
 
 def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                 page_table: torch.Tensor, page_size: int, ring: int, seq_slot: torch.Tensor,
                 seq_len: torch.Tensor, nh: int, nkv: int, hd: int, scale: float, window: int,
-                nsplit: int) -> torch.Tensor:
+                nsplit: int, waves: int = 1) -> torch.Tensor:
     """One new token per sequence against the paged cache; returns [B, nh * hd].
-    seq_len[b]: keys of sequence b, the new one included."""
+    seq_len[b]: keys of sequence b, the new one included.  The keys of a sequence are cut
+    into `nsplit` ranges (blocks, combined by a merge kernel) and each range is shared by
+    `waves` waves of a block (combined in LDS; the bfloat16 kernels only)."""
     _gpu(qkv, kcache, vcache, page_table, seq_slot, seq_len)
     _i32(page_table); _i32(seq_slot, qkv.shape[0]); _i32(seq_len, qkv.shape[0])
     B = qkv.shape[0]
@@ -315,7 +319,7 @@ def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                    if nsplit > 1 else None)
         _check(_lib().illm_attn_decode_bf16(
             _p(qkv), _p(out), _p(kcache), _p(vcache), _p(page_table), page_table.shape[1],
-            page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, B, nh, nkv, hd,
+            page_size, ring, _p(seq_slot), _p(seq_len), _p(partial), nsplit, waves, B, nh, nkv, hd,
             ctypes.c_float(scale), window, _stream()), f"attn_decode_bf16 (head_dim {hd})")
         return out
     partial = torch.empty((B, nh, nsplit, hd + 2), dtype=torch.float32, device=qkv.device)

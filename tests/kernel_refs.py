@@ -124,12 +124,12 @@ def attn_prefill(qkv, cu_seqlens, n_seqs, max_len, nh, nkv, hd, scale, window):
     return out
 
 
-def decode_splits(B, nh, max_len):
-    return 2
+def decode_splits(B, nkv, max_len):
+    return 2, 1
 
 
 def attn_decode(qkv, kcache, vcache, page_table, page_size, ring, seq_slot, seq_len, nh, nkv, hd,
-                scale, window, nsplit):
+                scale, window, nsplit, waves=1):
     B = qkv.shape[0]
     view = qkv.view(B, nh + 2 * nkv, hd)
     out = torch.zeros(B, nh * hd, dtype=qkv.dtype, device=qkv.device)

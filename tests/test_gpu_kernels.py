@@ -257,10 +257,11 @@ def test_attn_decode_bf16_pages_of_64(nh, nkv, hd, lens, window, nsplit):
     B = len(lens)
     qkv = rnd(B, (nh + 2 * nkv) * hd, dtype=dtype, seed=11)
     scale = 1.0 / math.sqrt(hd)
-    got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring, slots.to(DEV),
-                            seq_len.to(DEV), nh, nkv, hd, scale, window, nsplit)
     want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, seq_len, nh, nkv, hd, scale, window, nsplit)
-    close(got, want, dtype, scale=2)
+    for waves in (1, 2, 3, 8):                  # waves of a block that share a key range
+        got = ops().attn_decode(qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring, slots.to(DEV),
+                                seq_len.to(DEV), nh, nkv, hd, scale, window, nsplit, waves)
+        close(got, want, dtype, scale=2)
 
 
 @pytest.mark.parametrize("ydt", DTYPES)
