@@ -334,3 +334,140 @@ def test_schedule_runs_a_layer_twice_and_shares_a_cache_line(tmp_path):
         out = eng.step([I.StepEntry(s, [r[n + j]], [0]) for s, r, n in zip(slots, reqs, head)])
         for b in range(2):
             assert rel(out[b], want[b][head[b] + j]) < 2e-5, (b, j)
+
+
+def test_toy_routed_feed_forward_and_learned_positions(tmp_path):
+    """Two more toy parts defined here: a feed-forward that routes every row to one of three
+    experts (router logits in float32, top-1), and a position encoding that adds a learned table
+    to the embedded rows and leaves q and k alone.  Registered, built from a spec, stepped whole,
+    token by token and in a batch, against a plain computation."""
+    import inferllm_amd as I
+    from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from inferllm_amd.kernels import ops
+    from inferllm_amd.parts import FeedForward, PositionEncoding, register_part
+    from inferllm_amd.weights import TensorWant
+    from tiny import random_ids, read_weights
+    E, V, nh, hd, F, X, eps, P_MAX = 48, 70, 3, 16, 64, 3, 1e-5, 128
+
+    @register_part("feed_forward", "toy_top1_experts")
+    class Top1Experts(FeedForward):
+        graph_safe = False              # routes on the host
+
+        def __init__(self, hidden_size, intermediate_size, experts, tensors=None):
+            super().__init__(tensors)
+            self.E, self.F, self.X = hidden_size, intermediate_size, experts
+
+        def shapes(self):
+            out = {"router": TensorWant((self.X, self.E))}
+            for x in range(self.X):
+                out[f"gate_up{x}"] = TensorWant((2 * self.F, self.E))
+                out[f"down{x}"] = TensorWant((self.E, self.F))
+            return out
+
+        def load(self, tensors):
+            self.router = self._take(tensors, "router")
+            self.gu = [self._take(tensors, f"gate_up{x}") for x in range(self.X)]
+            self.down = [self._take(tensors, f"down{x}") for x in range(self.X)]
+
+        def forward(self, h, ctx):
+            logits = ops.linear(h, self.router, out_dtype=torch.float32)     # router in float32
+            choice = torch.argmax(logits, dim=-1)
+            out = torch.zeros_like(h)
+            for x in range(self.X):
+                rows = (choice == x).nonzero().flatten()
+                if rows.numel():
+                    hx = h[rows].contiguous()
+                    out[rows] = ops.linear(ops.gate_up_silu(hx, self.gu[x]), self.down[x])
+            return out
+
+    @register_part("position", "toy_learned_absolute")
+    class LearnedAbsolute(PositionEncoding):
+        def __init__(self, hidden_size, max_positions, tensors=None):
+            super().__init__(tensors)
+            self.E, self.P = hidden_size, max_positions
+
+        def shapes(self):
+            return {"table": TensorWant((self.P, self.E))}
+
+        def load(self, tensors):
+            self.table = self._take(tensors, "table").float()
+
+        def on_embedding(self, x, ctx):
+            x += self.table[ctx.row_pos.long()]
+
+        def on_qkv(self, qkv, ctx, nh, nkv, hd, kcache, vcache, group):
+            ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot,
+                           ctx.cache.slot_len if ctx.prefill else None, kcache, vcache,
+                           group.table if group is not None else None,
+                           group.page_size if group is not None else 1,
+                           group.ring if group is not None else 0, nh, nkv, hd)
+
+    @register_architecture("ToyRoutedForTests")
+    class Cfg:
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": ["ToyRoutedForTests"]}
+
+        def to_spec(self):
+            norm = lambda n: PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": n})
+            pos = PartSpec("toy_learned_absolute", {"hidden_size": E, "max_positions": P_MAX}, {"table": "pos"})
+            def ffn(i):
+                t = {"router": f"l{i}.router"}
+                for x in range(X):
+                    t[f"gate_up{x}"] = f"l{i}.x{x}.gu"; t[f"down{x}"] = f"l{i}.x{x}.d"
+                return PartSpec("toy_top1_experts", {"hidden_size": E, "intermediate_size": F, "experts": X}, t)
+            layers = [LayerSpec("pre_norm",
+                                PartSpec("attention", {"hidden_size": E, "num_heads": nh, "num_kv_heads": nh, "head_dim": hd},
+                                         {k: f"l{i}.{k}" for k in "qkvo"}),
+                                ffn(i) if i == 1 else PartSpec("swiglu", {"hidden_size": E, "intermediate_size": F},
+                                                                {"gate": "l0.g", "up": "l0.u", "down": "l0.d"}),
+                                norm(f"l{i}.n1"), norm(f"l{i}.n2"), pos) for i in range(2)]
+            return ModelSpec("ToyRoutedForTests", V, E, P_MAX,
+                             PartSpec("token_embedding", {"vocab_size": V, "hidden_size": E}, {"weight": "emb"}),
+                             layers, [ScheduleEntry(0, 0), ScheduleEntry(1, 1)], norm("nf"),
+                             PartSpec("lm_head", {"hidden_size": E, "vocab_size": V}, {"weight": "head"}))
+
+    d = I.write_random_model(str(tmp_path / "routed"), Cfg(), seed=6)
+    w = read_weights(d)
+    w["pos"] = w["pos"] * 20.0                                  # positions must matter
+    w["l1.router"] = w["l1.router"] * 50.0                      # clear choices, all experts used
+    from inferllm_amd.weights import write_safetensors
+    write_safetensors(str(tmp_path / "routed" / "model.safetensors"), w.items())
+
+    def plain(ids):
+        S = len(ids)
+        x = P.embedding(w["emb"], ids) + w["pos"][:S].double()
+        used = set()
+        for i in range(2):
+            h = P.rms_norm(x, w[f"l{i}.n1"], eps)
+            q, k, v = (P.linear(h, w[f"l{i}.{n}"]).reshape(S, nh, hd) for n in "qkv")
+            x = x + P.linear(P.causal_attention(q, k, v), w[f"l{i}.o"])
+            h = P.rms_norm(x, w[f"l{i}.n2"], eps)
+            if i == 0:
+                x = x + P.swiglu_ffn(h, w["l0.g"], w["l0.u"], w["l0.d"])
+            else:
+                choice = torch.argmax(P.linear(h, w["l1.router"]), dim=-1)
+                y = torch.zeros_like(x)
+                for r in range(S):
+                    e = int(choice[r]); used.add(e)
+                    gu = w[f"l1.x{e}.gu"]
+                    y[r] = P.swiglu_ffn(h[r:r + 1], gu[:F], gu[F:], w[f"l1.x{e}.d"])[0]
+                x = x + y
+        return P.linear(P.rms_norm(x, w["nf"], eps), w["head"]), used
+
+    eng = I.Engine.from_pretrained(d, dtype="float32", max_batch=2, max_seq_len=P_MAX)
+    assert not eng.runner.use_graphs                            # a part of the model reads on the host
+    reqs = [random_ids(n, V, 3 * n) for n in (40, 11)]
+    want = [plain(r) for r in reqs]
+    assert want[0][1] == {0, 1, 2}                              # every expert had rows
+    slots = [eng.alloc_slot(), eng.alloc_slot()]
+    head = [len(r) - 3 for r in reqs]
+    out = eng.step([I.StepEntry(s, r[:n], list(range(n))) for s, r, n in zip(slots, reqs, head)])
+    assert rel(out[:head[0]], want[0][0][:head[0]]) < 2e-5 and rel(out[head[0]:], want[1][0][:head[1]]) < 2e-5
+    for j in range(3):
+        out = eng.step([I.StepEntry(s, [r[n + j]], [0]) for s, r, n in zip(slots, reqs, head)])
+        for b in range(2):
+            assert rel(out[b], want[b][0][head[b] + j]) < 2e-5, (b, j)
