@@ -57,6 +57,9 @@ def build_parser() -> argparse.ArgumentParser:
                     help="config.json to build random weights from instead of --model")
     ap.add_argument("--weights-seed", type=int, default=0, help="seed of --random weights")
     ap.add_argument("--summary", action="store_true", help="print prefill and decode token/s at the end")
+    ap.add_argument("--profile", action="store_true",
+                    help="time every kernel call with HIP events (steps run without HIP graphs) and "
+                         "print a table per op at the end")
     return ap
 
 
@@ -110,7 +113,8 @@ def main(argv=None) -> int:
     from ..config import config_from_dict
 
     seed = args.seed if args.seed >= 0 else int(time.time())
-    kw = dict(dtype=args.dtype, max_batch=args.max_batch, max_seq_len=args.ctx_size)
+    kw = dict(dtype=args.dtype, max_batch=args.max_batch, max_seq_len=args.ctx_size,
+              use_graphs=not args.profile)
     if args.random_config:
         with open(args.random_config, "r", encoding="utf-8") as f:
             config = config_from_dict(json.load(f))
@@ -143,6 +147,14 @@ def main(argv=None) -> int:
                 print(text.show(o), flush=True)
         if args.summary:
             print(eng.last_stats.summary(), file=sys.stderr, flush=True)
+
+    if args.profile:
+        from ..kernels.profile import kernel_timing
+        timing = kernel_timing()
+        times = timing.__enter__()
+        import atexit
+        atexit.register(lambda: (print(times.table(), file=sys.stderr, flush=True),
+                                 timing.__exit__(None, None, None)))
 
     prompts: List[List[int]] = []
     if args.prompt_ids:

@@ -232,3 +232,16 @@ def test_long_prompt_then_decoding_at_head_size_128(tmp_path_factory, dtype):
     assert float(per.max()) < BUDGET[dtype], f"first bad decode position {1500 + int((per >= BUDGET[dtype]).nonzero()[0])}"
     eng.free_slot(s)
     eng.cache.check()
+
+
+def test_kernel_timing_reports_every_op(tmp_path_factory):
+    from inferllm_amd.kernels.profile import kernel_timing
+    eng, plain, config = setup(tmp_path_factory, "A", "bfloat16", use_graphs=False)
+    with kernel_timing() as t:
+        out = eng.generate([[1, 2, 3, 4]], max_new_tokens=3, stop_token_ids=[])
+    tot = t.totals()
+    assert len(out[0]) == 3
+    for op in ("embed", "add_rmsnorm", "linear", "attn_prefill", "attn_decode", "argmax"):
+        assert tot[op][0] > 0 and tot[op][1] > 0.0, op
+    assert tot["add_rmsnorm"][0] == 3 * (2 * config["num_hidden_layers"] + 1)
+    assert "share" in t.table()
