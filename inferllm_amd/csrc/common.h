@@ -43,6 +43,16 @@ __device__ __forceinline__ void st_f(void* p, int dt, size_t i, float v) {
     else ((float*)p)[i] = v;
 }
 
+typedef uint32_t illm_u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16 bytes of data that is read once (weights, cache rows): a non-temporal load, which keeps
+// the stream out of the way of lines that are used again.  Use it where an instruction reads
+// whole 128-byte lines; a line read in halves by two such loads is fetched twice.
+__device__ __forceinline__ uint4 ld16_stream(const void* p) {
+    const illm_u32x4_t v = __builtin_nontemporal_load((const illm_u32x4_t*)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = ILLM_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, ILLM_WAVE);
