@@ -85,11 +85,11 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
         uint4 kreg[NI], vreg[NI];
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-            kreg[j] = dim_ok ? *(const uint4*)(kcache + base + (size_t)j * KPI * hd)
+            kreg[j] = dim_ok ? ld16_stream(kcache + base + (size_t)j * KPI * hd)
                              : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-            vreg[j] = dim_ok ? *(const uint4*)(vcache + base + (size_t)j * KPI * hd)
+            vreg[j] = dim_ok ? ld16_stream(vcache + base + (size_t)j * KPI * hd)
                              : make_uint4(0, 0, 0, 0);
 
         // scores: lane (q, c) ends up owning key k0 + c * KPI + q (if c < NI)
