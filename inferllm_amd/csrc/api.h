@@ -78,11 +78,12 @@ int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int y_dt, int M
 int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M, int N,
                               int K, int ntb, int u, int waves, void* stream);
 
-// Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny product.
+// Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
+// product.  waves_wanted: waves per block (0: the default choice).
 int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* Y, int y_dt, int M, int F,
-                                 int K, void* stream);
+                                 int K, int waves_wanted, void* stream);
 
-// Few bfloat16 rows (M <= 16, hd % 32 == 0): the q|k|v product, the rotation of q and k (pairs
+// Few bfloat16 rows (M <= 16, hd % 16 == 0): the q|k|v product, the rotation of q and k (pairs
 // (i, i + hd/2), all dims) at row_pos[m], q into Y[M, (nh + 2 nkv) hd] (k and v parts untouched),
 // k and v into the paged cache of row_slot[m], all in one kernel.  waves_wanted: waves per block
 // (0: the default choice).

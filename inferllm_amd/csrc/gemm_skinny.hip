@@ -24,12 +24,12 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 // MAXW: most waves a block may have (register budget: 512 / (MAXW / 4) per lane).
 // What a block's tiles are and what happens to the sums:
 //   SK_PLAIN     NTB consecutive tiles of 16 rows of W; Y = sums.
-//   SK_GATE_UP   (NTB == 2) W is [gate rows (N) | up rows (N)]; the two tiles are the same 16 rows
-//                of each half and Y[M, N] = silu(gate) * up.
-//   SK_QKV_ROPE  (NTB == 2) W is [q heads | k heads | v heads]; a block of a q or k head takes 16
-//                rows and their rotation partners (hd/2 further), rotates the pairs by the row's
-//                position and writes q to Y and k to the paged cache; a block of a v head takes 32
-//                consecutive rows and writes them to the cache.
+//   SK_GATE_UP   (NTB == 1) W is [gate rows (N) | up rows (N)]; the tile is 8 gate rows and the
+//                same 8 up rows and Y[M, N] = silu(gate) * up.
+//   SK_QKV_ROPE  (NTB == 1) W is [q heads | k heads | v heads]; the tile of a block of a q or k head
+//                is 8 rows and their 8 rotation partners (hd/2 further); the block rotates the
+//                pairs by the row's position and writes q to Y and k to the paged cache; a block
+//                of a v head takes 16 consecutive rows and writes them to the cache.
 enum { SK_PLAIN = 0, SK_GATE_UP = 1, SK_QKV_ROPE = 2 };
 
 struct SkRope {
@@ -53,21 +53,27 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
     const int r = lane & 15, q = lane >> 4;
-    const int n_base = blockIdx.x * (DUAL ? 16 : 16 * NTB);
-    int tile_row[NTB];           // first W row of each of the block's tiles
+    const int n_base = blockIdx.x * (DUAL ? 8 : 16 * NTB);
+    int tile_row[NTB];           // SK_PLAIN: first W row of each of the block's tiles
 #pragma unroll
-    for (int nt = 0; nt < NTB; ++nt) tile_row[nt] = n_base + (DUAL ? nt * N : nt * 16);
-    int rot_head = -1, rot_j = 0;
+    for (int nt = 0; nt < NTB; ++nt) tile_row[nt] = n_base + nt * 16;
+    // the other modes (NTB == 1): the first 8 rows of the tile and the second 8 are apart (a load
+    // instruction reads 8 rows)
+    int rot_head = -1, rot_j = 0, row_lo = 0, row_hi = 0;
+    if (DUAL) {
+        row_lo = n_base;
+        row_hi = N + n_base;
+    }
     if (MODE == SK_QKV_ROPE) {
-        const int pph = rope.hd / 32, n_rot = (rope.nh + rope.nkv) * pph;
+        const int tph = rope.hd / 16, n_rot = (rope.nh + rope.nkv) * tph;
         if ((int)blockIdx.x < n_rot) {
-            rot_head = blockIdx.x / pph;
-            rot_j = blockIdx.x % pph;
-            tile_row[0] = rot_head * rope.hd + 16 * rot_j;
-            tile_row[NTB - 1] = tile_row[0] + rope.hd / 2;
+            rot_head = blockIdx.x / tph;
+            rot_j = blockIdx.x % tph;
+            row_lo = rot_head * rope.hd + 8 * rot_j;
+            row_hi = row_lo + rope.hd / 2;
         } else {
-            tile_row[0] = (rope.nh + rope.nkv) * rope.hd + 32 * ((int)blockIdx.x - n_rot);
-            tile_row[NTB - 1] = tile_row[0] + 16;
+            row_lo = (rope.nh + rope.nkv) * rope.hd + 16 * ((int)blockIdx.x - n_rot);
+            row_hi = row_lo + 8;
         }
     }
 
@@ -79,16 +85,19 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
         const int mrow = threadIdx.x & 15, ro = (threadIdx.x >> 4) * 4;
         const int pos = rope.row_pos[mrow], slot = rope.row_slot[mrow];
         if (rot_head >= 0) {
-            const float4* cs = (const float4*)(rope.cos_sin + (size_t)pos * rope.hd + 2 * (16 * rot_j + ro));
-            const float4 c0 = cs[0], c1 = cs[1];
-            pre_cs[0] = c0.x; pre_cs[1] = c0.y; pre_cs[2] = c0.z; pre_cs[3] = c0.w;
-            pre_cs[4] = c1.x; pre_cs[5] = c1.y; pre_cs[6] = c1.z; pre_cs[7] = c1.w;
-            if (rot_head >= rope.nh)
-                pre_off = cache_row_offset(rope.page_table, rope.table_stride, slot, pos,
-                                           rope.page_size, rope.ring, rope.nkv, rot_head - rope.nh,
-                                           rope.hd) + 16 * rot_j + ro;
+            if (ro < 8) {
+                const float4* cs =
+                    (const float4*)(rope.cos_sin + (size_t)pos * rope.hd + 2 * (8 * rot_j + ro));
+                const float4 c0 = cs[0], c1 = cs[1];
+                pre_cs[0] = c0.x; pre_cs[1] = c0.y; pre_cs[2] = c0.z; pre_cs[3] = c0.w;
+                pre_cs[4] = c1.x; pre_cs[5] = c1.y; pre_cs[6] = c1.z; pre_cs[7] = c1.w;
+                if (rot_head >= rope.nh)
+                    pre_off = cache_row_offset(rope.page_table, rope.table_stride, slot, pos,
+                                               rope.page_size, rope.ring, rope.nkv,
+                                               rot_head - rope.nh, rope.hd) + 8 * rot_j + ro;
+            }
         } else {
-            const int vrow = tile_row[0] - (rope.nh + rope.nkv) * rope.hd;
+            const int vrow = row_lo - (rope.nh + rope.nkv) * rope.hd;
             pre_off = cache_row_offset(rope.page_table, rope.table_stride, slot, pos, rope.page_size,
                                        rope.ring, rope.nkv, vrow / rope.hd, rope.hd) + vrow % rope.hd + ro;
         }
@@ -102,9 +111,9 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             int n = tile_row[nt] + (lane >> 3) + 8 * h;
-            const int last = DUAL ? 2 * N - 1 : N - 1;
-            if (DUAL) n = (n - nt * N < N) ? n : nt * N + N - 1;
-            else n = n < last ? n : last;
+            if (MODE != SK_PLAIN) n = (h ? row_hi : row_lo) + (lane >> 3);
+            const int last = DUAL ? (h + 1) * N - 1 : N - 1;
+            n = n < last ? n : last;
             wline[nt][h] = W + (size_t)n * K;
         }
     const bf16_t* xrow[MT];
@@ -183,7 +192,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     }
     // acc[nt][mt][i] = Y[m = mt*16 + r][n = n_base + nt*16 + q*4 + i]
     constexpr int PER_WAVE = SK_REGION_FLOATS;
-    if (waves > 1) {
+    if (waves > 1 || MODE != SK_PLAIN) {
 #pragma unroll
         for (int nt = 0; nt < NTB; ++nt)
 #pragma unroll
@@ -191,6 +200,62 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                 *(f32x4_t*)(red + (size_t)wave * PER_WAVE + ((nt * MT + mt) * 64 + lane) * 4) =
                     acc[nt][mt];
         __syncthreads();
+    }
+    if (MODE == SK_QKV_ROPE) {
+        // NTB == 1, MT == 1: lane (m, g) of the first wave's threads owns rows 4 g .. 4 g + 3 of
+        // the tile for X row m; rows 8 .. 15 of a rotated tile are the partners of rows 0 .. 7
+        const int mrow = threadIdx.x & 15, ro = (threadIdx.x >> 4) * 4;
+        if (threadIdx.x >= 64 || mrow >= M || (rot_head >= 0 && ro >= 8)) return;
+        auto total = [&](int l2) {
+            f32x4_t t = *(f32x4_t*)(red + l2 * 4);
+            for (int w = 1; w < waves; ++w) {
+                const f32x4_t o = *(f32x4_t*)(red + (size_t)w * PER_WAVE + l2 * 4);
+                t[0] += o[0]; t[1] += o[1]; t[2] += o[2]; t[3] += o[3];
+            }
+            return t;
+        };
+        const f32x4_t lo = total(threadIdx.x);
+        if (rot_head >= 0) {
+            const f32x4_t hi = total(threadIdx.x + 32);
+            float y0[4], y1[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float c = pre_cs[2 * i], sn = pre_cs[2 * i + 1];
+                y0[i] = lo[i] * c - hi[i] * sn;
+                y1[i] = lo[i] * sn + hi[i] * c;
+            }
+            bf16_t* dst = rot_head < rope.nh ? (bf16_t*)Y + (size_t)mrow * N + row_lo + ro
+                                             : rope.kcache + pre_off;
+            *(uint2*)dst = make_uint2(pack_bf16x2(y0[0], y0[1]), pack_bf16x2(y0[2], y0[3]));
+            *(uint2*)(dst + rope.hd / 2) =
+                make_uint2(pack_bf16x2(y1[0], y1[1]), pack_bf16x2(y1[2], y1[3]));
+        } else {
+            *(uint2*)(rope.vcache + pre_off) =
+                make_uint2(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]));
+        }
+        return;
+    }
+    if (DUAL) {
+        // NTB == 1: rows 0 .. 7 of the tile are gate rows, rows 8 .. 15 the up rows of the same
+        // outputs; a thread takes one X row's 4 outputs
+        for (int grp = threadIdx.x; grp < MT * 32; grp += blockDim.x) {
+            const int l2 = grp & 31, mt = grp >> 5;
+            const int mrow = mt * 16 + (l2 & 15), n0 = n_base + (l2 >> 4) * 4;
+            if (mrow >= M) continue;
+            const int e = (mt * 64 + l2) * 4;
+            f32x4_t g = *(f32x4_t*)(red + e), u = *(f32x4_t*)(red + e + 128);
+            for (int w = 1; w < waves; ++w) {
+                const f32x4_t og = *(f32x4_t*)(red + (size_t)w * PER_WAVE + e);
+                const f32x4_t ou = *(f32x4_t*)(red + (size_t)w * PER_WAVE + e + 128);
+                g[0] += og[0]; g[1] += og[1]; g[2] += og[2]; g[3] += og[3];
+                u[0] += ou[0]; u[1] += ou[1]; u[2] += ou[2]; u[3] += ou[3];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n0 + i < N)
+                    st_f(Y, y_dt, (size_t)mrow * N + n0 + i, (g[i] / (1.0f + expf(-g[i]))) * u[i]);
+        }
+        return;
     }
     // every thread of the block sums some of the (mt, lane) groups over the waves, tile by tile
     for (int grp = threadIdx.x; grp < MT * 64; grp += blockDim.x) {
@@ -215,44 +280,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
         }
         const int mrow = mt * 16 + (l2 & 15);
         if (mrow >= M) continue;
-        if (MODE == SK_QKV_ROPE) {
-            // MT == 1 and at least 64 threads: grp == threadIdx.x, the thread that prefetched
-            const int ro = (l2 >> 4) * 4;                 // this lane's 4 rows within a tile
-            if (rot_head >= 0) {
-                float y0[4], y1[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float c = pre_cs[2 * i], sn = pre_cs[2 * i + 1];
-                    y0[i] = v[0][i] * c - v[NTB - 1][i] * sn;
-                    y1[i] = v[0][i] * sn + v[NTB - 1][i] * c;
-                }
-                bf16_t* dst = rot_head < rope.nh ? (bf16_t*)Y + (size_t)mrow * N + tile_row[0] + ro
-                                                 : rope.kcache + pre_off;
-                *(uint2*)dst = make_uint2(pack_bf16x2(y0[0], y0[1]), pack_bf16x2(y0[2], y0[3]));
-                *(uint2*)(dst + rope.hd / 2) =
-                    make_uint2(pack_bf16x2(y1[0], y1[1]), pack_bf16x2(y1[2], y1[3]));
-            } else {
-                bf16_t* dst = rope.vcache + pre_off;
-                *(uint2*)dst = make_uint2(pack_bf16x2(v[0][0], v[0][1]), pack_bf16x2(v[0][2], v[0][3]));
-                *(uint2*)(dst + 16) = make_uint2(pack_bf16x2(v[NTB - 1][0], v[NTB - 1][1]),
-                                                 pack_bf16x2(v[NTB - 1][2], v[NTB - 1][3]));
-            }
-        } else if (DUAL) {
-            const int n0 = n_base + (l2 >> 4) * 4;
+        for (int nt = 0; nt < NTB; ++nt) {
+            const int n0 = tile_row[nt] + (l2 >> 4) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (n0 + i < N) {
-                    const float g = v[0][i];
-                    st_f(Y, y_dt, (size_t)mrow * N + n0 + i, (g / (1.0f + expf(-g))) * v[NTB - 1][i]);
-                }
-        } else {
-#pragma unroll
-            for (int nt = 0; nt < NTB; ++nt) {
-                const int n0 = tile_row[nt] + (l2 >> 4) * 4;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[nt][i]);
-            }
+                if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[nt][i]);
         }
     }
 }
@@ -265,13 +298,17 @@ static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M,
     constexpr int REGS = 2 * (NTB + MT) * U * 4 + NTB * 8 + NTB * MT * 4 + 40;
     constexpr int MAXW = REGS <= 128 ? 16 : (REGS <= 256 ? 8 : 4);
     waves = waves > MAXW ? MAXW : waves;
-    const int rows_per_block = DUAL ? 16 : 16 * NTB;
+    const int rows_per_block = DUAL ? 8 : 16 * NTB;
     const int blocks = (N + rows_per_block - 1) / rows_per_block;
     const size_t smem = (size_t)waves * NTB * (U > MT ? U : MT) * 1024;
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, MODE>), dim3(blocks), dim3(64 * waves),
                        smem, st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K, rope);
     return illm_launch_status();
 }
+
+// Measured on MI355X at the LLaMA-2-7B shapes: 16 W rows per block and about this many waves
+// on the chip are best for M <= 16; wider row tiles only pay when X has many rows.
+static const int SK_WAVES_ON_CHIP = 2400;
 
 static int clamp_waves(int w, int ntb, int mt, int u, int K) {
     const int ksteps = (K + 31) / 32;
@@ -308,11 +345,9 @@ extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int 
                                      int N, int K, void* stream) {
     if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
         return ILLM_ERR_ARG;
-    // measured on MI355X at the LLaMA-2-7B shapes: 16 W rows per block and about 1536 waves
-    // on the chip are best for M <= 16; wider row tiles only pay when X has many rows
     const int ntb = M <= 16 ? 1 : 2, u = 4;
     const int blocks = (N + 16 * ntb - 1) / (16 * ntb);
-    int waves = (1536 + blocks / 2) / blocks;
+    int waves = (SK_WAVES_ON_CHIP + blocks / 2) / blocks;
     waves = waves < 1 ? 1 : waves;
     return illm_gemm_skinny_bf16_cfg(X, W, Y, y_dt, M, N, K, ntb, u, waves, stream);
 }
@@ -320,43 +355,43 @@ extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int 
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T) with W = [Wg (F rows) | Wu (F rows)], [2F, K]:
 // the gate and up products and the SiLU-multiply in one kernel (src/core/graph.cpp:57-79).
 extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* Y, int y_dt, int M,
-                                            int F, int K, void* stream) {
+                                            int F, int K, int waves_wanted, void* stream) {
     if (M <= 0 || M > 64 || F <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
         return ILLM_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     const int mt = (M + 15) / 16;
-    const int blocks = (F + 15) / 16;
-    int waves = (1536 + blocks / 2) / blocks;
-    waves = clamp_waves(waves < 1 ? 1 : waves, 2, mt, 4, K);
+    const int blocks = (F + 7) / 8;
+    // measured at F = 11008, K = 4096: 4 to 8 waves a block are within 1 % of each other, 2 are 6 % slower
+    int waves = waves_wanted > 0 ? waves_wanted : (8192 + blocks / 2) / blocks;
+    waves = clamp_waves(waves < 1 ? 1 : waves, 1, mt, 4, K);
     switch (mt) {
-        case 1: return launch_skinny<1, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
-        case 2: return launch_skinny<2, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
-        case 3: return launch_skinny<3, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
-        default: return launch_skinny<4, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 1: return launch_skinny<1, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 2: return launch_skinny<2, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 3: return launch_skinny<3, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        default: return launch_skinny<4, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
     }
 }
 
 // Decode step of an attention layer's input side in one kernel: Y = X . Wqkv^T, the q and k heads
 // rotated (pairs (i, i + hd/2), all hd dims) by the angles at row_pos[m], q written to
 // Y[M, (nh + 2 nkv) hd] (its k and v parts are left untouched), k and v written to the paged cache
-// of row_slot[m].  M <= 16, hd % 32 == 0, K % 8 == 0, bfloat16.
+// of row_slot[m].  M <= 16, hd % 16 == 0, K % 8 == 0, bfloat16.
 extern "C" int illm_qkv_rope_store_skinny(const void* X, const void* W, void* Y, int M, int K,
                                           const float* cos_sin, int max_pos,
                                           const int32_t* row_pos, const int32_t* row_slot,
                                           void* kcache, void* vcache, const int32_t* page_table,
                                           int table_stride, int page_size, int ring, int nh, int nkv,
                                           int hd, int waves_wanted, void* stream) {
-    if (M <= 0 || M > 16 || K <= 0 || (K % 8) || nh <= 0 || nkv <= 0 || hd <= 0 || (hd % 32) ||
+    if (M <= 0 || M > 16 || K <= 0 || (K % 8) || nh <= 0 || nkv <= 0 || hd <= 0 || (hd % 16) ||
         !cos_sin || max_pos <= 0 || !row_pos || !row_slot || !kcache || !vcache || !page_table ||
         table_stride <= 0 || page_size <= 0)
         return ILLM_ERR_ARG;
     SkRope rope = {cos_sin, row_pos, row_slot, (bf16_t*)kcache, (bf16_t*)vcache, page_table,
                    table_stride, page_size, ring, nh, nkv, hd};
     const int N = (nh + 2 * nkv) * hd;
-    const int blocks = N / 32;
-    // measured at the 7B shape: about 1152 waves on the chip are best for 32-row blocks
-    int waves = waves_wanted > 0 ? waves_wanted : (1152 + blocks / 2) / blocks;
-    waves = clamp_waves(waves < 1 ? 1 : waves, 2, 1, 4, K);
-    return launch_skinny<1, 2, 4, SK_QKV_ROPE>(X, W, Y, ILLM_BF16, M, N, K, waves,
+    const int blocks = N / 16;
+    int waves = waves_wanted > 0 ? waves_wanted : (SK_WAVES_ON_CHIP + blocks / 2) / blocks;
+    waves = clamp_waves(waves < 1 ? 1 : waves, 1, 1, 4, K);
+    return launch_skinny<1, 1, 4, SK_QKV_ROPE>(X, W, Y, ILLM_BF16, M, N, K, waves,
                                                (hipStream_t)stream, rope);
 }

@@ -217,12 +217,13 @@ def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -
 
 
 QKV_ROPE_WAVES = 0       # waves per block of the fused kernel; 0: the kernel's own choice
+GATE_UP_WAVES = 0        # the same for the fused gate|up product
 
 
 def qkv_rope_store_fits(x: torch.Tensor, w_qkv: torch.Tensor, hd: int) -> bool:
     """Whether the one-kernel q|k|v product + rotation + cache store takes these operands."""
     return (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and
-            1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0 and hd % 32 == 0)
+            1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0 and hd % 16 == 0)
 
 
 def qkv_rope_store(x: torch.Tensor, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
@@ -262,7 +263,7 @@ def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
         _need(w_gate_up.dim() == 2 and w_gate_up.shape[1] == K, "gate_up_silu: shapes")
         y = torch.empty((M, F2 // 2), dtype=x.dtype, device=x.device)
         _check(_lib().illm_gemm_skinny_gateup_silu(_p(x), _p(w_gate_up), _p(y), _code(y), M,
-                                                   F2 // 2, K, _stream()), "gate_up_silu")
+                                                   F2 // 2, K, GATE_UP_WAVES, _stream()), "gate_up_silu")
         return y
     return silu_mul(linear(x, w_gate_up))
 

@@ -403,7 +403,8 @@ def test_window_edge_prefill_and_decode(dtype, hd):
         close(got.cpu().view(nh, hd), out[L - 1], dtype, scale=8)
 
 
-@pytest.mark.parametrize("M,nh,nkv,hd,K", [(1, 32, 32, 128, 4096), (8, 4, 2, 32, 64), (16, 6, 3, 64, 200), (3, 8, 1, 96, 72)])
+@pytest.mark.parametrize("M,nh,nkv,hd,K", [(1, 32, 32, 128, 4096), (8, 4, 2, 32, 64), (16, 6, 3, 64, 200), (3, 8, 1, 96, 72),
+                                          (5, 3, 3, 48, 136), (2, 2, 1, 16, 40)])
 def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K):
     """The fused decode kernel against product, then rotation and cache store."""
     from inferllm_amd.parts.position import rotary_table
