@@ -27,6 +27,14 @@ LLAMA2_7B = {"architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "interm
              "bos_token_id": 1, "eos_token_id": 2}
 
 
+LLAMA3_8B = dict(LLAMA2_7B, intermediate_size=14336, num_key_value_heads=8, vocab_size=128256,
+                 rope_theta=500000.0, max_position_embeddings=8192)
+LLAMA2_70B = dict(LLAMA2_7B, hidden_size=8192, intermediate_size=28672, num_hidden_layers=80,
+                  num_attention_heads=64, num_key_value_heads=8)
+SHAPES = {"llama2-7b": ("LLaMA-2-7B shape", LLAMA2_7B), "llama3-8b": ("LLaMA-3-8B shape", LLAMA3_8B),
+          "llama2-70b": ("LLaMA-2-70B shape", LLAMA2_70B)}
+
+
 def weight_bytes_per_step(cfg, layers, esz):
     E, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nh, nkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
@@ -58,6 +66,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
     ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--shape", default="llama2-7b", choices=sorted(SHAPES),
+                    help="layer sizes (default: the headline configuration)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
@@ -71,7 +81,8 @@ def main() -> int:
     from inferllm_amd import Engine, StepEntry
     from inferllm_amd.kernels import ops
 
-    cfg = dict(LLAMA2_7B)
+    shape_name, shape_cfg = SHAPES[args.shape]
+    cfg = dict(shape_cfg)
     full_layers = cfg["num_hidden_layers"]
     layers = args.layers or full_layers
     cfg["num_hidden_layers"] = layers
@@ -149,10 +160,11 @@ def main() -> int:
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dkey, "data": "synthetic: seeded random weights N(0, 0.02), uniform random token ids",
-        "config": {"model": "LLaMA-2-7B shape", "layers": layers, "layers_full": full_layers,
+        "config": {"model": shape_name, "layers": layers, "layers_full": full_layers,
                    "hidden_size": cfg["hidden_size"], "intermediate_size": cfg["intermediate_size"],
                    "num_attention_heads": cfg["num_attention_heads"],
-                   "num_key_value_heads": cfg["num_key_value_heads"], "head_dim": 128,
+                   "num_key_value_heads": cfg["num_key_value_heads"],
+                   "head_dim": cfg.get("head_dim", cfg["hidden_size"] // cfg["num_attention_heads"]),
                    "vocab_size": cfg["vocab_size"], "global_batch": args.batch,
                    "seq_len": ctx_len, "prompt_len": args.prompt, "rope_theta": cfg["rope_theta"],
                    "rms_norm_eps": cfg["rms_norm_eps"], "parallelism": "single GPU"},

@@ -92,23 +92,39 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
             vreg[j] = dim_ok ? ld16_stream(vcache + base + (size_t)j * KPI * hd)
                              : make_uint4(0, 0, 0, 0);
 
-        // scores: lane (q, c) ends up owning key k0 + c * KPI + q (if c < NI)
+        // scores: lane (q, c) ends up owning key k0 + c * KPI + q (if c < NI).  Every lane has a
+        // share of NI dot products; instead of NI full reductions over the LPR lanes of a row,
+        // each step halves what a lane keeps: at the step that pairs lanes c and c ^ b, the lane
+        // keeps the products whose index has c's bit b and hands the others over.
         float s_own[GC];
 #pragma unroll
-        for (int g = 0; g < GC; ++g) s_own[g] = NEG_INF;
+        for (int g = 0; g < GC; ++g) {
+            float part[NI];
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            float kf8[8];
-            unpack8(kreg[j], kf8);
+            for (int j = 0; j < NI; ++j) {
+                float kf8[8];
+                unpack8(kreg[j], kf8);
+                float p = 0.f;
 #pragma unroll
-            for (int g = 0; g < GC; ++g) {
-                float part = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) part = fmaf(qr[g][i], kf8[i], part);
-#pragma unroll
-                for (int o = 1; o < LPR; o <<= 1) part += __shfl_xor(part, o, ILLM_WAVE);
-                if (c == j) s_own[g] = part * scale;
+                for (int i = 0; i < 8; ++i) p = fmaf(qr[g][i], kf8[i], p);
+                part[j] = p;
             }
+            // lanes beyond the NI that own a product (LPR > NI): plain sums first
+#pragma unroll
+            for (int o = NI; o < LPR; o <<= 1)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) part[j] += __shfl_xor(part[j], o, ILLM_WAVE);
+#pragma unroll
+            for (int b = 1, n = NI / 2; b < NI; b <<= 1, n >>= 1) {
+                const bool up = (c & b) != 0;
+#pragma unroll
+                for (int k = 0; k < n; ++k) {
+                    const float keep = up ? part[2 * k + 1] : part[2 * k];
+                    const float send = up ? part[2 * k] : part[2 * k + 1];
+                    part[k] = keep + __shfl_xor(send, b, ILLM_WAVE);
+                }
+            }
+            s_own[g] = part[0] * scale;
         }
         const int key_own = k0 + c * KPI + q;
         const bool own_ok = (c < NI) && key_own < len && key_own >= kf;
