@@ -42,10 +42,28 @@ struct SkRope {
     int table_stride, page_size, ring, nh, nkv, hd;
 };
 
+// The residual add and the RMS norm between two products of few rows, without kernels of their
+// own (M <= 16).  The producing product (SK_PLAIN, float32 Y) adds its result to the residual
+// rows Y; if `nw` is given it also leaves xb = bfloat16(y * nw), the next product's operand up to
+// the row's scale, and the sum of y^2 over its 16 columns in ssq[m][its block].  The consuming
+// product gets xb as X and `ssq`: every result of row m is scaled by
+// 1 / sqrt(sum_p ssq[m][p] / K + eps), which is the row's norm since the scale is common to all k.
+struct SkResidual {
+    int accumulate;              // producer: Y += product
+    const void* nw;              // producer: norm weight [N] (bfloat16 or float32) or null
+    int nw_dt;
+    bf16_t* xb;                  // producer: [M, N]
+    float* ssq_out;              // producer: [M, gridDim.x]
+    const float* ssq;            // consumer: [M, parts] or null
+    int parts;
+    float eps;
+};
+
 template <int MT, int NTB, int SK_U, int MAXW, int MODE>
 __global__ void __launch_bounds__(64 * MAXW)
 gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
-                   void* __restrict__ Y, int y_dt, int M, int N, int K, SkRope rope) {
+                   void* __restrict__ Y, int y_dt, int M, int N, int K, SkRope rope,
+                   SkResidual res) {
     constexpr bool DUAL = MODE == SK_GATE_UP;
     // a wave's piece of LDS: first the staging of its W lines (NTB * SK_U KB), then its sums
     constexpr int SK_REGION_FLOATS = NTB * (SK_U > MT ? SK_U : MT) * 256;
@@ -53,6 +71,52 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int waves = blockDim.x >> 6;
     const int r = lane & 15, q = lane >> 4;
+    // consumer: the last wave, which has the fewest pieces of K if they do not divide evenly, adds
+    // up the rows' sums of squares (a row's parts as one load of the whole wave) while the others
+    // already stream W; the scales wait in LDS for the end
+    float* row_rs = red + (size_t)waves * SK_REGION_FLOATS;      // [16]
+    if (res.ssq && wave == waves - 1) {
+        // all rows' loads are asked for at once; then 16 sums over the wave in one halving
+        // exchange (a lane keeps the rows that share its bit), after which lane m has row m's
+        float t[16];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) t[m] = 0.f;
+        const bool by4 = (res.parts & 3) == 0;
+        for (int p = lane * 4; p < res.parts; p += 256) {
+            float4 v[16];
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                v[m] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (m < M) {
+                    const float* at = res.ssq + (size_t)m * res.parts + p;
+                    if (by4) {
+                        v[m] = *(const float4*)at;
+                    } else {
+                        v[m].x = at[0];
+                        if (p + 1 < res.parts) v[m].y = at[1];
+                        if (p + 2 < res.parts) v[m].z = at[2];
+                        if (p + 3 < res.parts) v[m].w = at[3];
+                    }
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < 16; ++m) t[m] += (v[m].x + v[m].y) + (v[m].z + v[m].w);
+        }
+#pragma unroll
+        for (int b = 1, n = 8; b < 16; b <<= 1, n >>= 1) {
+            const bool up = (lane & b) != 0;
+#pragma unroll
+            for (int k = 0; k < n; ++k) {
+                const float keep = up ? t[2 * k + 1] : t[2 * k];
+                const float send = up ? t[2 * k] : t[2 * k + 1];
+                t[k] = keep + __shfl_xor(send, b, ILLM_WAVE);
+            }
+        }
+        float tot = t[0];
+        tot += __shfl_xor(tot, 16, ILLM_WAVE);
+        tot += __shfl_xor(tot, 32, ILLM_WAVE);
+        if (lane < 16) row_rs[lane] = 1.0f / sqrtf(tot / (float)K + res.eps);
+    }
     const int n_base = blockIdx.x * (DUAL ? 8 : 16 * NTB);
     int tile_row[NTB];           // SK_PLAIN: first W row of each of the block's tiles
 #pragma unroll
@@ -75,6 +139,19 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
             row_lo = (rope.nh + rope.nkv) * rope.hd + 16 * ((int)blockIdx.x - n_rot);
             row_hi = row_lo + 8;
         }
+    }
+
+    // producer: the threads that will add to the residual rows fetch their 4 values and the norm
+    // weights now, so that they arrive while W is streamed
+    float pre_y[4] = {0.f, 0.f, 0.f, 0.f}, pre_nw[4] = {0.f, 0.f, 0.f, 0.f};
+    if (MODE == SK_PLAIN && res.accumulate && threadIdx.x < 64 && (int)(threadIdx.x & 15) < M) {
+        const int n0 = tile_row[0] + (threadIdx.x >> 4) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n0 + i < N) {
+                pre_y[i] = ((const float*)Y)[(size_t)(threadIdx.x & 15) * N + n0 + i];
+                if (res.nw) pre_nw[i] = ld_f(res.nw, res.nw_dt, n0 + i);
+            }
     }
 
     // SK_QKV_ROPE: the threads that will write the results fetch what that needs (position,
@@ -201,6 +278,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                     acc[nt][mt];
         __syncthreads();
     }
+    // consumer (MT == 1): the scale of X row m16
+    auto row_scale = [&](int m16) { return res.ssq ? row_rs[m16] : 1.0f; };
     if (MODE == SK_QKV_ROPE) {
         // NTB == 1, MT == 1: lane (m, g) of the first wave's threads owns rows 4 g .. 4 g + 3 of
         // the tile for X row m; rows 8 .. 15 of a rotated tile are the partners of rows 0 .. 7
@@ -214,9 +293,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
             }
             return t;
         };
-        const f32x4_t lo = total(threadIdx.x);
+        const float rs = row_scale(mrow);
+        f32x4_t lo = total(threadIdx.x);
+        lo[0] *= rs; lo[1] *= rs; lo[2] *= rs; lo[3] *= rs;
         if (rot_head >= 0) {
-            const f32x4_t hi = total(threadIdx.x + 32);
+            f32x4_t hi = total(threadIdx.x + 32);
+            hi[0] *= rs; hi[1] *= rs; hi[2] *= rs; hi[3] *= rs;
             float y0[4], y1[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -250,10 +332,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                 g[0] += og[0]; g[1] += og[1]; g[2] += og[2]; g[3] += og[3];
                 u[0] += ou[0]; u[1] += ou[1]; u[2] += ou[2]; u[3] += ou[3];
             }
+            const float rs = row_scale(l2 & 15);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (n0 + i < N)
-                    st_f(Y, y_dt, (size_t)mrow * N + n0 + i, (g[i] / (1.0f + expf(-g[i]))) * u[i]);
+                if (n0 + i < N) {
+                    const float gi = g[i] * rs;
+                    st_f(Y, y_dt, (size_t)mrow * N + n0 + i, (gi / (1.0f + expf(-gi))) * (u[i] * rs));
+                }
         }
         return;
     }
@@ -279,20 +364,59 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
             }
         }
         const int mrow = mt * 16 + (l2 & 15);
+        if (res.accumulate) {
+            // producer (MT == 1, NTB == 1: the threads are the first wave, all of it takes part
+            // in the exchange below): Y += sums; operand and sum of squares for the next norm
+            const int n0 = tile_row[0] + (l2 >> 4) * 4;
+            float sq = 0.f;
+            if (mrow < M) {
+                // grp == threadIdx.x here: the thread that fetched pre_y and pre_nw
+                float y[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    y[i] = pre_y[i] + v[0][i];
+                    if (res.nw && n0 + i < N) sq = fmaf(y[i], y[i], sq);
+                }
+                const size_t at = (size_t)mrow * N + n0;
+                if (n0 + 3 < N && (N & 3) == 0) {
+                    *(float4*)((float*)Y + at) = make_float4(y[0], y[1], y[2], y[3]);
+                    if (res.nw)
+                        *(uint2*)(res.xb + at) = make_uint2(pack_bf16x2(y[0] * pre_nw[0], y[1] * pre_nw[1]),
+                                                            pack_bf16x2(y[2] * pre_nw[2], y[3] * pre_nw[3]));
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n0 + i < N) {
+                            ((float*)Y)[at + i] = y[i];
+                            if (res.nw) res.xb[at + i] = f32_to_bf16(y[i] * pre_nw[i]);
+                        }
+                }
+            }
+            if (res.nw) {
+                sq += __shfl_xor(sq, 16, ILLM_WAVE);
+                sq += __shfl_xor(sq, 32, ILLM_WAVE);
+                if (l2 < 16 && mrow < M) res.ssq_out[(size_t)mrow * gridDim.x + blockIdx.x] = sq;
+            }
+            continue;
+        }
         if (mrow >= M) continue;
+        const float rs = MT == 1 ? row_scale(l2 & 15) : 1.0f;
 #pragma unroll
         for (int nt = 0; nt < NTB; ++nt) {
             const int n0 = tile_row[nt] + (l2 >> 4) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[nt][i]);
+                if (n0 + i < N) st_f(Y, y_dt, (size_t)mrow * N + n0 + i, v[nt][i] * rs);
         }
     }
 }
 
+static const SkResidual SK_NO_RESIDUAL = {0, nullptr, ILLM_BF16, nullptr, nullptr, nullptr, 0, 0.f};
+
 template <int MT, int NTB, int U, int MODE = SK_PLAIN>
 static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
-                         int waves, hipStream_t st, SkRope rope = SkRope()) {
+                         int waves, hipStream_t st, SkRope rope = SkRope(),
+                         SkResidual res = SK_NO_RESIDUAL) {
     constexpr bool DUAL = MODE == SK_GATE_UP;
     // registers a lane needs: operands of two pieces in flight and the accumulators
     constexpr int REGS = 2 * (NTB + MT) * U * 4 + NTB * 8 + NTB * MT * 4 + 40;
@@ -300,9 +424,9 @@ static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M,
     waves = waves > MAXW ? MAXW : waves;
     const int rows_per_block = DUAL ? 8 : 16 * NTB;
     const int blocks = (N + rows_per_block - 1) / rows_per_block;
-    const size_t smem = (size_t)waves * NTB * (U > MT ? U : MT) * 1024;
+    const size_t smem = (size_t)waves * NTB * (U > MT ? U : MT) * 1024 + 64;
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, MODE>), dim3(blocks), dim3(64 * waves),
-                       smem, st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K, rope);
+                       smem, st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K, rope, res);
     return illm_launch_status();
 }
 
@@ -313,7 +437,7 @@ static const int SK_WAVES_ON_CHIP = 2400;
 static int clamp_waves(int w, int ntb, int mt, int u, int K) {
     const int ksteps = (K + 31) / 32;
     const int max_by_k = (ksteps + u - 1) / u;           // more waves than k pieces would idle
-    const int lds_cap = 64 / (ntb * (u > mt ? u : mt));
+    const int lds_cap = 60 / (ntb * (u > mt ? u : mt));     // 64 KB of LDS a block, some left for the scales
     w = w > 16 ? 16 : w;
     w = w > lds_cap ? lds_cap : w;
     w = w > max_by_k ? max_by_k : w;
@@ -340,24 +464,58 @@ extern "C" int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, 
     return ILLM_ERR_ARG;
 }
 
+static bool scale_args_ok(const float* ssq, int parts, int M) {
+    return !ssq || (parts > 0 && M <= 16);
+}
+
 // Takes bfloat16 X and W, M in 1..64, K a multiple of 8.  Otherwise ILLM_ERR_ARG.
+// ssq != null (M <= 16): row m of the result is scaled by 1 / sqrt(sum_p ssq[m][p] / K + eps).
 extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int y_dt, int M,
-                                     int N, int K, void* stream) {
-    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
+                                     int N, int K, const float* ssq, int parts, float eps,
+                                     void* stream) {
+    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt) ||
+        !scale_args_ok(ssq, parts, M))
         return ILLM_ERR_ARG;
     const int ntb = M <= 16 ? 1 : 2, u = 4;
     const int blocks = (N + 16 * ntb - 1) / (16 * ntb);
     int waves = (SK_WAVES_ON_CHIP + blocks / 2) / blocks;
     waves = waves < 1 ? 1 : waves;
-    return illm_gemm_skinny_bf16_cfg(X, W, Y, y_dt, M, N, K, ntb, u, waves, stream);
+    if (!ssq) return illm_gemm_skinny_bf16_cfg(X, W, Y, y_dt, M, N, K, ntb, u, waves, stream);
+    SkResidual res = SK_NO_RESIDUAL;
+    res.ssq = ssq; res.parts = parts; res.eps = eps;
+    return launch_skinny<1, 1, 4>(X, W, Y, y_dt, M, N, K, clamp_waves(waves, 1, 1, 4, K),
+                                  (hipStream_t)stream, SkRope(), res);
+}
+
+// Y[M, N] (float32) += X . W^T for M <= 16 bfloat16 rows: a block's output projection with the
+// residual add.  nw != null: also xb[M, N] = bfloat16(Y * nw) and ssq_out[M][ceil(N / 16)], the
+// sums of Y^2 over each block's 16 columns, for a product that takes the norm (see SkResidual).
+extern "C" int illm_gemm_skinny_add(const void* X, const void* W, float* Y, int M, int N, int K,
+                                    const void* nw, int nw_dt, void* xb, float* ssq_out,
+                                    void* stream) {
+    if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K % 8) || !Y ||
+        (nw && (!illm_dtype_ok(nw_dt) || !xb || !ssq_out)))
+        return ILLM_ERR_ARG;
+    const int blocks = (N + 15) / 16;
+    int waves = (SK_WAVES_ON_CHIP + blocks / 2) / blocks;
+    waves = clamp_waves(waves < 1 ? 1 : waves, 1, 1, 4, K);
+    SkResidual res = SK_NO_RESIDUAL;
+    res.accumulate = 1; res.nw = nw; res.nw_dt = nw_dt; res.xb = (bf16_t*)xb; res.ssq_out = ssq_out;
+    return launch_skinny<1, 1, 4>(X, W, Y, ILLM_F32, M, N, K, waves, (hipStream_t)stream, SkRope(),
+                                  res);
 }
 
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T) with W = [Wg (F rows) | Wu (F rows)], [2F, K]:
 // the gate and up products and the SiLU-multiply in one kernel (src/core/graph.cpp:57-79).
+// ssq: as for illm_gemm_skinny_bf16.
 extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* Y, int y_dt, int M,
-                                            int F, int K, int waves_wanted, void* stream) {
-    if (M <= 0 || M > 64 || F <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
+                                            int F, int K, const float* ssq, int parts, float eps,
+                                            int waves_wanted, void* stream) {
+    if (M <= 0 || M > 64 || F <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt) ||
+        !scale_args_ok(ssq, parts, M))
         return ILLM_ERR_ARG;
+    SkResidual res = SK_NO_RESIDUAL;
+    res.ssq = ssq; res.parts = parts; res.eps = eps;
     hipStream_t st = (hipStream_t)stream;
     const int mt = (M + 15) / 16;
     const int blocks = (F + 7) / 8;
@@ -365,7 +523,7 @@ extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* 
     int waves = waves_wanted > 0 ? waves_wanted : (8192 + blocks / 2) / blocks;
     waves = clamp_waves(waves < 1 ? 1 : waves, 1, mt, 4, K);
     switch (mt) {
-        case 1: return launch_skinny<1, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
+        case 1: return launch_skinny<1, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st, SkRope(), res);
         case 2: return launch_skinny<2, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
         case 3: return launch_skinny<3, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
         default: return launch_skinny<4, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);
@@ -375,13 +533,17 @@ extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* 
 // Decode step of an attention layer's input side in one kernel: Y = X . Wqkv^T, the q and k heads
 // rotated (pairs (i, i + hd/2), all hd dims) by the angles at row_pos[m], q written to
 // Y[M, (nh + 2 nkv) hd] (its k and v parts are left untouched), k and v written to the paged cache
-// of row_slot[m].  M <= 16, hd % 16 == 0, K % 8 == 0, bfloat16.
+// of row_slot[m].  M <= 16, hd % 16 == 0, K % 8 == 0, bfloat16.  ssq: as for illm_gemm_skinny_bf16.
 extern "C" int illm_qkv_rope_store_skinny(const void* X, const void* W, void* Y, int M, int K,
                                           const float* cos_sin, int max_pos,
                                           const int32_t* row_pos, const int32_t* row_slot,
                                           void* kcache, void* vcache, const int32_t* page_table,
                                           int table_stride, int page_size, int ring, int nh, int nkv,
-                                          int hd, int waves_wanted, void* stream) {
+                                          int hd, const float* ssq, int parts, float eps,
+                                          int waves_wanted, void* stream) {
+    if (!scale_args_ok(ssq, parts, M)) return ILLM_ERR_ARG;
+    SkResidual res = SK_NO_RESIDUAL;
+    res.ssq = ssq; res.parts = parts; res.eps = eps;
     if (M <= 0 || M > 16 || K <= 0 || (K % 8) || nh <= 0 || nkv <= 0 || hd <= 0 || (hd % 16) ||
         !cos_sin || max_pos <= 0 || !row_pos || !row_slot || !kcache || !vcache || !page_table ||
         table_stride <= 0 || page_size <= 0)
@@ -393,5 +555,5 @@ extern "C" int illm_qkv_rope_store_skinny(const void* X, const void* W, void* Y,
     int waves = waves_wanted > 0 ? waves_wanted : (SK_WAVES_ON_CHIP + blocks / 2) / blocks;
     waves = clamp_waves(waves < 1 ? 1 : waves, 1, 1, 4, K);
     return launch_skinny<1, 1, 4, SK_QKV_ROPE>(X, W, Y, ILLM_BF16, M, N, K, waves,
-                                               (hipStream_t)stream, rope);
+                                               (hipStream_t)stream, rope, res);
 }

@@ -10,6 +10,8 @@ from typing import Dict, List, Optional
 
 import torch
 
+from ..kernels import ops
+
 from ..cache.manager import KVSpec, StateSpec
 from ..config.spec import ModelSpec
 from ..parts import build_part, part_class
@@ -96,10 +98,18 @@ class DecoderModel:
                 layer.position.on_embedding(x, ctx)
                 break
         pending = None
-        for e in self.schedule:
-            pending = self.layers[e.layer].forward(x, pending, ctx, e.cache_line, e.writes_cache)
+        for i, e in enumerate(self.schedule):
+            layer = self.layers[e.layer]
+            if getattr(layer, "takes_next_norm", False) and i + 1 < len(self.schedule):
+                # the norm that will meet this block's output, for kernels that prepare it
+                nxt = getattr(self.layers[self.schedule[i + 1].layer], "mixer_norm", None)
+                pending = layer.forward(x, pending, ctx, e.cache_line, e.writes_cache, next_norm=nxt)
+            else:
+                pending = layer.forward(x, pending, ctx, e.cache_line, e.writes_cache)
         if out_rows is None or out_rows.numel() == 0:
             return None
+        if isinstance(pending, ops.NormedRows):
+            pending = None                       # its sum is in x already
         h = self.final_norm.forward(x, pending, ctx, row_idx=out_rows)
         return self.head.forward(h, ctx)
 

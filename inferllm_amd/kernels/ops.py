@@ -172,8 +172,78 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> to
     return y
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """y = x . w^T, w stored [out, in] (src/kern/naive/naive.cpp:363-379)."""
+class NormedRows:
+    """Residual rows whose RMS norm the next product takes itself (few rows, bfloat16).
+
+    Left by `linear_add(..., norm=)`: `x` the float32 residual rows (the sum already in them),
+    `xb` = bfloat16(x * weight), `ssq[m][p]` partial sums of x^2.  A product of few rows reads
+    `xb` and scales row m of its result by 1 / sqrt(sum_p ssq[m][p] / K + eps), which is the
+    product of the normed rows since the scale is common to a row; anything else asks `rows()`
+    for the normed rows."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor, eps: float, act_dtype: torch.dtype,
+                 xb: torch.Tensor, ssq: torch.Tensor):
+        self.x, self.weight, self.eps, self.dtype = x, weight, float(eps), act_dtype
+        self.xb, self.ssq = xb, ssq
+        self.shape = x.shape
+        self._rows: Optional[torch.Tensor] = None
+
+    def rows(self) -> torch.Tensor:
+        if self._rows is None:
+            self._rows = add_rmsnorm(self.x, None, self.weight, self.eps, self.dtype)
+        return self._rows
+
+    def made_for(self, weight: torch.Tensor, eps: float) -> bool:
+        return weight is self.weight and float(eps) == self.eps
+
+
+def _operand(x):
+    """(tensor the kernel reads, ssq pointer, parts, eps) of a few-rows product's input."""
+    if isinstance(x, NormedRows):
+        return x.xb, _p(x.ssq), x.ssq.shape[1], ctypes.c_float(x.eps)
+    return x, None, 0, ctypes.c_float(0.0)
+
+
+def linear_add_fits(x, w: torch.Tensor, into: torch.Tensor) -> bool:
+    """Whether `linear_add` takes these operands (few bfloat16 rows into float32 rows)."""
+    return (isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and x.dim() == 2 and w.dim() == 2 and into.dtype == torch.float32 and
+            into.is_contiguous() and 1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0
+            and w.shape[1] == x.shape[1] and into.shape == (x.shape[0], w.shape[0]))
+
+
+def linear_add(x: torch.Tensor, w: torch.Tensor, into: torch.Tensor, norm=None,
+               act_dtype: torch.dtype = torch.bfloat16) -> Optional[NormedRows]:
+    """into += x . w^T in the product's kernel: the residual add of a block's output projection,
+    each element added by the one thread that owns it.  norm = (weight [N], eps) of the RMS norm
+    that follows: the kernel also leaves what the next few-rows product needs to take that norm
+    itself, returned as `NormedRows` (only if N % 8 == 0, else None as without `norm`)."""
+    _gpu(x, w, into)
+    _need(linear_add_fits(x, w, into), "linear_add: operands not taken")
+    M, K = x.shape
+    N = w.shape[0]
+    if norm is not None and (N % 8 or norm[0].dtype not in _CODES or act_dtype != torch.bfloat16
+                             or norm[0].shape != (N,)):
+        norm = None
+    if norm is None:
+        _check(_lib().illm_gemm_skinny_add(_p(x), _p(w), _p(into), M, N, K, None, BF16, None, None,
+                                           _stream()), "linear_add")
+        return None
+    weight, eps = norm
+    _gpu(weight)
+    xb = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    ssq = torch.empty((M, (N + 15) // 16), dtype=torch.float32, device=x.device)
+    _check(_lib().illm_gemm_skinny_add(_p(x), _p(w), _p(into), M, N, K, _p(weight), _code(weight),
+                                       _p(xb), _p(ssq), _stream()), "linear_add")
+    return NormedRows(into, weight, eps, act_dtype, xb, ssq)
+
+
+def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x . w^T, w stored [out, in] (src/kern/naive/naive.cpp:363-379).  x may be `NormedRows`."""
+    if isinstance(x, NormedRows):
+        if w.dtype == torch.bfloat16:
+            return gemm_skinny_bf16(x, w, out_dtype or x.dtype)
+        x = x.rows()
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32 or w.dtype == torch.float32:
         return gemm_generic(x, w, out_dtype)
@@ -201,18 +271,20 @@ def skinny_fits(M: int, N: int, K: int) -> bool:
     return 1 <= M <= SKINNY_MAX_ROWS and K % 8 == 0
 
 
-def gemm_skinny_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """x [M <= 64, K] . w [N, K]^T, both bfloat16, float32 accumulation on the matrix cores."""
-    _gpu(x, w)
-    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands")
-    _need(x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1],
-          f"linear: x {tuple(x.shape)} against w {tuple(w.shape)}")
-    M, K = x.shape
+def gemm_skinny_bf16(x, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M <= 64, K] . w [N, K]^T, both bfloat16, float32 accumulation on the matrix cores; or
+    x `NormedRows`: the product of the normed rows."""
+    xt, ssq, parts, eps = _operand(x)
+    _gpu(xt, w)
+    _need(xt.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands")
+    _need(xt.dim() == 2 and w.dim() == 2 and xt.shape[1] == w.shape[1],
+          f"linear: x {tuple(xt.shape)} against w {tuple(w.shape)}")
+    M, K = xt.shape
     N = w.shape[0]
     _need(skinny_fits(M, N, K), f"gemm_skinny: M={M} K={K} not taken")
-    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
-    _check(_lib().illm_gemm_skinny_bf16(_p(x), _p(w), _p(y), _code(y), M, N, K, _stream()),
-           "gemm_skinny")
+    y = torch.empty((M, N), dtype=out_dtype, device=xt.device)
+    _check(_lib().illm_gemm_skinny_bf16(_p(xt), _p(w), _p(y), _code(y), M, N, K, ssq, parts, eps,
+                                        _stream()), "gemm_skinny")
     return y
 
 
@@ -220,19 +292,21 @@ QKV_ROPE_WAVES = 0       # waves per block of the fused kernel; 0: the kernel's 
 GATE_UP_WAVES = 0        # the same for the fused gate|up product
 
 
-def qkv_rope_store_fits(x: torch.Tensor, w_qkv: torch.Tensor, hd: int) -> bool:
+def qkv_rope_store_fits(x, w_qkv: torch.Tensor, hd: int) -> bool:
     """Whether the one-kernel q|k|v product + rotation + cache store takes these operands."""
     return (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and
             1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0 and hd % 16 == 0)
 
 
-def qkv_rope_store(x: torch.Tensor, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
+def qkv_rope_store(x, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
                    row_pos: torch.Tensor, row_slot: torch.Tensor, kcache: torch.Tensor,
                    vcache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
                    nh: int, nkv: int, hd: int) -> torch.Tensor:
     """Decode only: x . Wqkv^T, q and k rotated (pairs (i, i + hd/2), all dims) at row_pos, q
-    returned in rows [q | k | v] whose k and v parts are NOT filled, k and v stored in the cache."""
-    _gpu(x, w_qkv, cos_sin, row_pos, row_slot, kcache, vcache, page_table)
+    returned in rows [q | k | v] whose k and v parts are NOT filled, k and v stored in the cache.
+    x may be `NormedRows`."""
+    xt, ssq, parts, eps = _operand(x)
+    _gpu(xt, w_qkv, cos_sin, row_pos, row_slot, kcache, vcache, page_table)
     _i32(row_pos, x.shape[0]); _i32(row_slot, x.shape[0]); _i32(page_table)
     M, K = x.shape
     N = (nh + 2 * nkv) * hd
@@ -243,28 +317,35 @@ def qkv_rope_store(x: torch.Tensor, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
     _need(kcache.dtype == torch.bfloat16 and kcache.shape[1:] == (nkv, page_size, hd) and
           vcache.shape == kcache.shape and vcache.dtype == torch.bfloat16 and page_table.dim() == 2,
           "qkv_rope_store: cache shape or dtype")
-    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=xt.device)
     _check(_lib().illm_qkv_rope_store_skinny(
-        _p(x), _p(w_qkv), _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
+        _p(xt), _p(w_qkv), _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
         _p(kcache), _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, nh, nkv, hd,
-        QKV_ROPE_WAVES, _stream()), "qkv_rope_store")
+        ssq, parts, eps, QKV_ROPE_WAVES, _stream()), "qkv_rope_store")
     return y
 
 
-def gate_up_silu(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+def gate_up_silu(x, w_gate_up: torch.Tensor) -> torch.Tensor:
     """silu(x . Wg^T) * (x . Wu^T) for w_gate_up = [Wg | Wu] stacked as [2F, K].
 
-    Few bfloat16 rows: one fused MFMA kernel.  Otherwise the product and `silu_mul`."""
+    Few bfloat16 rows: one fused MFMA kernel.  Otherwise the product and `silu_mul`.
+    x may be `NormedRows`."""
+    if isinstance(x, NormedRows) and (w_gate_up.dtype != torch.bfloat16 or w_gate_up.shape[0] % 2):
+        x = x.rows()
     M, K = x.shape
     F2 = w_gate_up.shape[0]
     if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and F2 % 2 == 0
             and 1 <= M <= SKINNY_BEST_ROWS and K % 8 == 0):
-        _gpu(x, w_gate_up)
+        xt, ssq, parts, eps = _operand(x)
+        _gpu(xt, w_gate_up)
         _need(w_gate_up.dim() == 2 and w_gate_up.shape[1] == K, "gate_up_silu: shapes")
-        y = torch.empty((M, F2 // 2), dtype=x.dtype, device=x.device)
-        _check(_lib().illm_gemm_skinny_gateup_silu(_p(x), _p(w_gate_up), _p(y), _code(y), M,
-                                                   F2 // 2, K, GATE_UP_WAVES, _stream()), "gate_up_silu")
+        y = torch.empty((M, F2 // 2), dtype=x.dtype, device=xt.device)
+        _check(_lib().illm_gemm_skinny_gateup_silu(_p(xt), _p(w_gate_up), _p(y), _code(y), M,
+                                                   F2 // 2, K, ssq, parts, eps, GATE_UP_WAVES,
+                                                   _stream()), "gate_up_silu")
         return y
+    if isinstance(x, NormedRows):
+        x = x.rows()
     return silu_mul(linear(x, w_gate_up))
 
 

@@ -31,6 +31,9 @@ class Attention(Mixer):
     Whole prompts attend over the step's own rows; single tokens over the cache.
     """
 
+    adds_residual = True
+    takes_normed_rows = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: Optional[int] = None, softmax_scale: Optional[float] = None, tensors=None):
         super().__init__(tensors)
@@ -57,7 +60,8 @@ class Attention(Mixer):
         self.w_qkv = _fuse([self._take(tensors, n) for n in ("q", "k", "v")])
         self.w_o = self._take(tensors, "o").contiguous()
 
-    def forward(self, h, ctx: StepContext, line, writes_cache, position):
+    def forward(self, h, ctx: StepContext, line, writes_cache, position, residual=None,
+                next_norm=None):
         nh, nkv, hd = self.nh, self.nkv, self.hd
         kc, vc, group = ctx.cache.kv_line(line)
         window = self.window or 0
@@ -91,4 +95,8 @@ class Attention(Mixer):
             o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
                                 ctx.seq_slot, ctx.seq_len, nh, nkv, hd, self.scale, window,
                                 nsplit, waves)
+        if residual is not None and ops.linear_add_fits(o, self.w_o, residual):
+            return ops.linear_add(o, self.w_o, residual,
+                                  next_norm.rms_params() if next_norm is not None else None,
+                                  ctx.act_dtype)
         return ops.linear(o, self.w_o)

@@ -56,6 +56,14 @@ class Part:
     be captured into a HIP graph.  A part that reads device data on the host sets it False.
     """
     graph_safe = True
+    # A short cut between a block's parts for steps of few rows (False: the plain protocol, which
+    # every part supports).  A mixer or feed-forward with `adds_residual` takes
+    # `forward(..., residual=x, next_norm=norm)` and may add its result to the float32 residual
+    # rows `x` in its last kernel; it then returns None, or, if that kernel could also prepare
+    # the norm that follows (`next_norm.rms_params()`), `ops.NormedRows` for the next part.
+    # A part with `takes_normed_rows` accepts `ops.NormedRows` as its `h`.
+    adds_residual = False
+    takes_normed_rows = False
 
     def __init__(self, tensors: Optional[Dict[str, str]] = None):
         self.tensors: Dict[str, str] = dict(tensors or {})
@@ -96,6 +104,11 @@ class FeedForward(Part):
 
 
 class Norm(Part):
+    def rms_params(self):
+        """(weight, eps) if the norm is a plain RMS norm that a product's kernel may take over
+        (see `Part.adds_residual`), else None."""
+        return None
+
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: StepContext,
                 row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Add `delta` to the float32 residual rows `x` (in place unless `row_idx`

@@ -20,6 +20,9 @@ class SwiGLU(FeedForward):
     elementwise kernels (src/kern/gpu/kernel_gpu.cu:183-258).
     """
 
+    adds_residual = True
+    takes_normed_rows = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, tensors=None):
         super().__init__(tensors)
         self.E, self.F = int(hidden_size), int(intermediate_size)
@@ -34,5 +37,10 @@ class SwiGLU(FeedForward):
         self.w_gate_up = _fuse([self._take(tensors, "gate"), self._take(tensors, "up")])
         self.w_down = self._take(tensors, "down").contiguous()
 
-    def forward(self, h, ctx: StepContext):
-        return ops.linear(ops.gate_up_silu(h, self.w_gate_up), self.w_down)
+    def forward(self, h, ctx: StepContext, residual=None, next_norm=None):
+        a = ops.gate_up_silu(h, self.w_gate_up)
+        if residual is not None and ops.linear_add_fits(a, self.w_down, residual):
+            return ops.linear_add(a, self.w_down, residual,
+                                  next_norm.rms_params() if next_norm is not None else None,
+                                  ctx.act_dtype)
+        return ops.linear(a, self.w_down)

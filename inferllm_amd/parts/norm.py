@@ -29,5 +29,8 @@ class RMSNorm(Norm):
     def load(self, tensors) -> None:
         self.weight = self._take(tensors, "weight").contiguous()
 
+    def rms_params(self):
+        return self.weight, self.eps
+
     def forward(self, x, delta, ctx: StepContext, row_idx=None):
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, ctx.act_dtype, row_idx)

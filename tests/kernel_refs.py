@@ -87,6 +87,10 @@ def qkv_rope_store_fits(x, w_qkv, hd):
     return False        # the CPU stand-in goes through linear + rope_store
 
 
+def linear_add_fits(x, w, into):
+    return False
+
+
 def gate_up_silu(x, w_gate_up):
     return silu_mul(linear(x, w_gate_up))
 
@@ -196,5 +200,6 @@ def patch(monkeypatch):
     """Put these functions in place of the GPU ops (CPU tests only)."""
     from inferllm_amd.kernels import ops
     for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic", "gate_up_silu", "qkv_rope_store_fits",
+                 "linear_add_fits",
                  "attn_prefill", "decode_splits", "attn_decode", "argmax", "sample"):
         monkeypatch.setattr(ops, name, globals()[name])

@@ -288,6 +288,66 @@ def test_gate_up_silu(M, F, K):
     assert not torch.allclose(got.double().cpu(), swapped, atol=0.1 * float(want.abs().max()))
 
 
+def _prepared_rows(M, K, nw_dtype, eps, seed=5):
+    """Residual rows with unequal scales and a norm weight far from 1, as `linear_add(norm=)`
+    leaves them (made here by adding a product of zeros), and their plain norm."""
+    x = rnd(M, K, seed=seed) * torch.linspace(0.02, 3.0, M)[:, None]
+    nw = (1 + rnd(K, seed=seed + 1) * 0.3).to(nw_dtype)
+    want = R.add_rmsnorm(x.clone(), None, nw, eps, torch.bfloat16)
+    zeros = torch.zeros(M, 8, dtype=torch.bfloat16, device=DEV)
+    rows = ops().linear_add(zeros, torch.zeros(K, 8, dtype=torch.bfloat16, device=DEV),
+                            x.clone().to(DEV), (nw.to(DEV), eps))
+    assert rows is not None and torch.equal(rows.x.cpu(), x)
+    return rows, want
+
+
+@pytest.mark.parametrize("nw_dtype", DTYPES)
+@pytest.mark.parametrize("ydt", DTYPES)
+@pytest.mark.parametrize("M,N,K,eps", [(1, 4096, 4096, 1e-5), (8, 100, 136, 1e-6), (16, 33, 1000, 1e-2), (5, 320, 96, 1e-5)])
+def test_gemm_skinny_takes_the_norm(nw_dtype, ydt, M, N, K, eps):
+    """The product of rows whose norm was prepared against norm, then product."""
+    rows, h = _prepared_rows(M, K, nw_dtype, eps)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=2)
+    got = ops().linear(rows, w.to(DEV), ydt)
+    # the kernel rounds x * weight to bfloat16 and scales the sums, the reference rounds the
+    # normed rows: the operands differ by bfloat16 roundings whatever the output's dtype
+    close(got, R.linear(h, w, ydt), torch.bfloat16, scale=math.sqrt(K))
+    close(rows.rows(), h, torch.bfloat16)                  # and can still be had normalised
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 11008, 4096), (8, 172, 64), (16, 203, 80), (3, 33, 1000)])
+def test_gate_up_silu_takes_the_norm(M, F, K):
+    rows, h = _prepared_rows(M, K, torch.bfloat16, 1e-5)
+    w = rnd(2 * F, K, dtype=torch.bfloat16, seed=2, std=0.2)
+    got = ops().gate_up_silu(rows, w.to(DEV))
+    g, u = R.linear(h, w[:F], torch.float64), R.linear(h, w[F:], torch.float64)
+    want = g / (1 + torch.exp(-g)) * u
+    close(got, want, torch.bfloat16, scale=max(1.0, float(want.abs().max())))
+
+
+@pytest.mark.parametrize("nw_dtype", [None] + DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 4096, 11008), (16, 104, 136), (7, 33, 1000)])
+def test_linear_add(M, N, K, nw_dtype):
+    """into += x . w^T in float32, nothing but the sum is rounded; with a norm's weight also
+    bfloat16(into * weight) and the rows' sums of squares in parts."""
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+    into = rnd(M, N, seed=3) * 10
+    dev = into.clone().to(DEV)
+    assert ops().linear_add_fits(x.to(DEV), w.to(DEV), dev)
+    nw = None if nw_dtype is None else (1 + rnd(N, seed=4) * 0.3).to(nw_dtype)
+    rows = ops().linear_add(x.to(DEV), w.to(DEV), dev, None if nw is None else (nw.to(DEV), 1e-5))
+    want = into.double() + R.linear(x, w, torch.float64)
+    torch.testing.assert_close(dev.double().cpu(), want, atol=2e-4 * math.sqrt(K), rtol=1e-5)
+    if nw is None or N % 8:
+        assert rows is None
+    else:
+        assert rows.x is dev and rows.ssq.shape == (M, (N + 15) // 16)
+        close(rows.xb, want * nw.double(), torch.bfloat16, scale=float(want.abs().max()))
+        torch.testing.assert_close(rows.ssq.double().sum(1).cpu(), (want ** 2).sum(1), rtol=1e-5, atol=1e-6)
+    assert not ops().linear_add_fits(x.to(DEV), w.to(DEV), dev.to(torch.bfloat16))
+    assert not ops().linear_add_fits(rnd(17, K, dtype=torch.bfloat16).to(DEV), w.to(DEV), torch.zeros(17, N, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attn_decode_finds_one_far_key(dtype):
     """One key among hundreds is made to stand out: the output must be its value."""
@@ -405,12 +465,16 @@ def test_window_edge_prefill_and_decode(dtype, hd):
 
 @pytest.mark.parametrize("M,nh,nkv,hd,K", [(1, 32, 32, 128, 4096), (8, 4, 2, 32, 64), (16, 6, 3, 64, 200), (3, 8, 1, 96, 72),
                                           (5, 3, 3, 48, 136), (2, 2, 1, 16, 40)])
-def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K):
-    """The fused decode kernel against product, then rotation and cache store."""
+@pytest.mark.parametrize("normed", [False, True])
+def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed):
+    """The fused decode kernel against (norm,) product, then rotation and cache store."""
     from inferllm_amd.parts.position import rotary_table
     dtype, page = torch.bfloat16, 64
     table = rotary_table(777.0, hd, 300, "cpu")
     x = rnd(M, K, dtype=dtype, seed=1)
+    x_dev = x.to(DEV)
+    if normed:
+        x_dev, x = _prepared_rows(M, K, torch.bfloat16, 1e-5)
     w = rnd((nh + 2 * nkv) * hd, K, dtype=dtype, seed=2, std=0.1)
     pos = torch.tensor([(37 * i + 5) % 290 for i in range(M)], dtype=torch.int32)
     slot = torch.randperm(M + 2, generator=torch.Generator().manual_seed(9))[:M].to(torch.int32)
@@ -422,7 +486,7 @@ def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K):
     qkv_ref = R.linear(x, w, torch.float64)
     kr, vr = kc.clone().double(), vc.clone().double()
     R.rope_store(qkv_ref, table, hd, 0, pos, slot, None, kr, vr, pt, page, 0, nh, nkv, hd)
-    got = ops().qkv_rope_store(x.to(DEV), w.to(DEV), table.to(DEV), pos.to(DEV), slot.to(DEV), kc_g := kc.to(DEV),
+    got = ops().qkv_rope_store(x_dev, w.to(DEV), table.to(DEV), pos.to(DEV), slot.to(DEV), kc_g := kc.to(DEV),
                                vc_g := vc.to(DEV), pt.to(DEV), page, 0, nh, nkv, hd).cpu()
     sc = math.sqrt(K) * 0.1
     close(got[:, :nh * hd], qkv_ref[:, :nh * hd], dtype, scale=sc)

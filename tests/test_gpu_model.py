@@ -243,5 +243,8 @@ def test_kernel_timing_reports_every_op(tmp_path_factory):
     assert len(out[0]) == 3
     for op in ("embed", "add_rmsnorm", "linear", "attn_prefill", "attn_decode", "argmax"):
         assert tot[op][0] > 0 and tot[op][1] > 0.0, op
-    assert tot["add_rmsnorm"][0] == 3 * (2 * config["num_hidden_layers"] + 1)
+    # every norm of the prompt's step is a launch; single-token steps take the norm inside the
+    # product that follows wherever the sizes allow, the last norm always remains
+    n_norms = 2 * config["num_hidden_layers"] + 1
+    assert n_norms + 2 <= tot["add_rmsnorm"][0] <= 3 * n_norms
     assert "share" in t.table()
