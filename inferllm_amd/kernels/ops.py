@@ -259,7 +259,65 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch
     if out_dtype == torch.float32:
         return gemm_generic(x, w, out_dtype)
     _gpu(x, w)
-    return torch.matmul(x, w.t())
+    return _planned_matmul(x, w)
+
+
+# The vendor GEMM's own choice of kernel is now and then a poor one for a shape (measured on
+# MI355X: 2048 x 22016 x 4096 takes 408 us whole and 253 us as 8192 + 13824 columns; most shapes
+# gain nothing).  So products of many rows are planned by measurement, once per shape: the whole
+# product against a few cuts of the output columns, each part written into its slice of one
+# result.  Every output element is still one kernel's sum; plans differ in rounding only.
+PLAN_PRODUCTS = True
+PLAN_MIN_ROWS = 1024          # below this no cut ever paid
+PLAN_MIN_COLS = 8192
+_PLANS: dict = {}             # (rows / 256 rounded up, N, K) -> cut points (empty: whole)
+
+
+def _split_candidates(N: int):
+    cuts = {(N // 8192) * 8192, (N // 4096) * 4096, (N // 2 // 256) * 256, 8192, 12288, 16384,
+            ((2 * N // 3) // 4096) * 4096, ((3 * N // 4) // 4096) * 4096}
+    return [()] + [(c,) for c in sorted(cuts) if 2048 <= c <= N - 1024]
+
+
+def _run_plan(x: torch.Tensor, w: torch.Tensor, plan, out: Optional[torch.Tensor] = None):
+    if not plan:
+        return torch.matmul(x, w.t(), out=out) if out is not None else torch.matmul(x, w.t())
+    if out is None:
+        out = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
+    edges = (0,) + tuple(plan) + (w.shape[0],)
+    for a, b in zip(edges[:-1], edges[1:]):
+        torch.matmul(x, w[a:b].t(), out=out[:, a:b])
+    return out
+
+
+def _measure_plan(x: torch.Tensor, w: torch.Tensor):
+    out = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
+    best, best_t = (), None
+    for plan in _split_candidates(w.shape[0]):
+        _run_plan(x, w, plan, out)                           # the first call of a shape sets up
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(3):
+            _run_plan(x, w, plan, out)
+        end.record()
+        end.synchronize()
+        t = start.elapsed_time(end)
+        if best_t is None or t < 0.97 * best_t:               # a cut has to pay clearly
+            best, best_t = plan, t
+    return best
+
+
+def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    M, K = x.shape
+    N = w.shape[0]
+    if (not PLAN_PRODUCTS or M < PLAN_MIN_ROWS or N < PLAN_MIN_COLS
+            or torch.cuda.is_current_stream_capturing()):
+        return torch.matmul(x, w.t())
+    key = (-(-M // 256), N, K)
+    plan = _PLANS.get(key)
+    if plan is None:
+        plan = _PLANS[key] = _measure_plan(x, w)
+    return _run_plan(x, w, plan)
 
 
 SKINNY_MAX_ROWS = 64     # rows the few-rows kernel takes

@@ -288,6 +288,26 @@ def test_gate_up_silu(M, F, K):
     assert not torch.allclose(got.double().cpu(), swapped, atol=0.1 * float(want.abs().max()))
 
 
+def test_products_of_many_rows_are_planned_once_and_stay_right():
+    """A product of many rows is measured whole and cut along its output columns, once per
+    shape; whatever plan wins, every element is the plain product."""
+    o = ops()
+    M, N, K = 1100, 9000, 64
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+    o._PLANS.clear()
+    got = o.linear(x.to(DEV), w.to(DEV))
+    key = (-(-M // 256), N, K)
+    assert key in o._PLANS and len(o._PLANS) == 1
+    close(got, R.linear(x, w), torch.bfloat16, scale=math.sqrt(K))
+    for plan in o._split_candidates(N):                    # every candidate gives the product
+        assert all(0 < c < N for c in plan)
+        close(o._run_plan(x.to(DEV), w.to(DEV), plan), R.linear(x, w), torch.bfloat16, scale=math.sqrt(K))
+    o.linear(x.to(DEV), w.to(DEV))
+    assert len(o._PLANS) == 1                              # measured once
+    o.linear(x[:1000].to(DEV), w.to(DEV))                  # fewer rows than planning is for
+    assert len(o._PLANS) == 1
+
+
 def _prepared_rows(M, K, nw_dtype, eps, seed=5):
     """Residual rows with unequal scales and a norm weight far from 1, as `linear_add(norm=)`
     leaves them (made here by adding a product of zeros), and their plain norm."""
