@@ -248,3 +248,43 @@ def test_kernel_timing_reports_every_op(tmp_path_factory):
     n_norms = 2 * config["num_hidden_layers"] + 1
     assert n_norms + 2 <= tot["add_rmsnorm"][0] <= 3 * n_norms
     assert "share" in t.table()
+
+
+@pytest.mark.parametrize("nkv,ffn", [(32, 11008), (8, 14336)])
+def test_real_layer_sizes_in_bfloat16(tmp_path_factory, nkv, ffn):
+    """Two layers of the LLaMA-2-7B sizes (width 4096, 32 heads of 128, feed-forward 11008,
+    vocabulary 32000) and of the LLaMA-3-8B ones (8 kv heads, feed-forward 14336): the sizes
+    the serving kernels are tuned for, which the tiny configurations never reach (products
+    over 4096 and 11008, 256 parts of a row's sum of squares, the vendor GEMM and the
+    matrix-core attention for the prompt, grouped decode attention on the matrix cores)."""
+    import inferllm_amd as I
+    from inferllm_amd import StepEntry
+    config = {"architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "intermediate_size": ffn,
+              "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": nkv,
+              "vocab_size": 32000, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+              "max_position_embeddings": 512, "tie_word_embeddings": False,
+              "bos_token_id": 1, "eos_token_id": 2}
+    d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=11, dtype=torch.bfloat16)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=4, poison_freed=True)
+    reqs = requests_for(config, [40, 23, 70], seed=3)
+    heads = [len(r) - 6 for r in reqs]
+    slots = [eng.alloc_slot() for _ in reqs]
+    got = [[] for _ in reqs]
+    out = eng.step([StepEntry(s, r[:h], list(range(h))) for s, r, h in zip(slots, reqs, heads)])
+    at = 0
+    for i, h in enumerate(heads):
+        got[i].append(out[at:at + h].clone())
+        at += h
+    for t in range(6):                                   # three rows: a padded bucket of four
+        out = eng.step([StepEntry(s, [r[h + t]], [0]) for s, r, h in zip(slots, reqs, heads)])
+        for i in range(len(reqs)):
+            got[i].append(out[i:i + 1].clone())
+    for i, r in enumerate(reqs):
+        want = plain_llama.forward_logits(config, w, r)
+        per_pos = (torch.cat(got[i]).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+        assert float(per_pos.max()) < BUDGET["bfloat16"], \
+            f"request {i}: first bad position {int((per_pos >= BUDGET['bfloat16']).nonzero()[0])} of {len(r)}"
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
