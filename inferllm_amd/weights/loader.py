@@ -19,7 +19,7 @@ from typing import Dict, Iterable, List, Optional, Tuple
 
 import torch
 
-from .safetensors_io import SafetensorsFile, open_model_files
+from .safetensors_io import PinnedStage, SafetensorsFile, open_model_files
 
 
 class WeightsError(ValueError):
@@ -99,13 +99,21 @@ def load_named_tensors(model_dir: str, expected: Dict[str, TensorWant], engine_d
                 stored[n] = e
         check_names(expected, stored, ignored_suffixes)
         out: Dict[str, torch.Tensor] = {}
+        on_gpu = torch.device(device).type == "cuda"
+        stage = PinnedStage() if on_gpu else None
         for n, w in expected.items():
             if n not in where:
                 continue
-            t = where[n].read(n)
-            if w.kind == "int" and t.numel() and (int(t.max()) > 2**31 - 1 or int(t.min()) < -2**31):
-                raise WeightsError([], [], [], [(n, "integers beyond int32")])
+            if on_gpu and w.kind != "int":
+                with torch.cuda.device(device):
+                    t = where[n].read_to_device(n, device, stage)
+            else:
+                t = where[n].read(n)
+                if w.kind == "int" and t.numel() and (int(t.max()) > 2**31 - 1 or int(t.min()) < -2**31):
+                    raise WeightsError([], [], [], [(n, "integers beyond int32")])
             out[n] = t.to(device=device, dtype=kept_dtype(t.dtype, w.kind, engine_dtype))
+        if stage is not None:
+            stage.finish()
         return out
     finally:
         for f in files:

@@ -31,6 +31,32 @@ class SafetensorsError(ValueError):
     pass
 
 
+class PinnedStage:
+    """Two pinned host buffers used in turn for copies to the device."""
+
+    def __init__(self, nbytes: int = 64 << 20):
+        self.nbytes = nbytes
+        self._bufs = [torch.empty(nbytes, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
+        self._events = [None, None]
+        self._i = 1
+
+    def next(self) -> torch.Tensor:
+        self._i ^= 1
+        if self._events[self._i] is not None:
+            self._events[self._i].synchronize()
+        return self._bufs[self._i]
+
+    def sent(self) -> None:
+        ev = torch.cuda.Event()
+        ev.record()
+        self._events[self._i] = ev
+
+    def finish(self) -> None:
+        for ev in self._events:
+            if ev is not None:
+                ev.synchronize()
+
+
 class SafetensorsFile:
     """One memory-mapped file: `.entries` maps names to (dtype string, shape)."""
 
@@ -80,6 +106,28 @@ class SafetensorsFile:
             return torch.empty(shape, dtype=dtype)
         raw = bytearray(self._map[self._data_start + b:self._data_start + t])   # one copy, owned
         return torch.frombuffer(raw, dtype=dtype).reshape(shape)
+
+    def read_to_device(self, name: str, device, stage: "PinnedStage") -> torch.Tensor:
+        """The tensor as stored, on a GPU: the file's bytes go through two pinned host buffers
+        in turn, one being filled from the file while the other is copied to the device."""
+        dt, shape = self.entries[name]
+        b, t = self._offsets[name]
+        out = torch.empty(shape, dtype=_DTYPES[dt], device=device)
+        if t == b:
+            return out
+        flat = out.view(-1).view(torch.uint8)
+        pos, end, done = self._data_start + b, self._data_start + t, 0
+        while pos < end:
+            n = min(stage.nbytes, end - pos)
+            buf = stage.next()                      # waits for the copy that last used it
+            got = os.preadv(self._f.fileno(), [memoryview(buf.numpy())[:n]], pos)
+            if got != n:
+                raise SafetensorsError(f"{self.path}: short read of tensor {name!r}")
+            flat[done:done + n].copy_(buf[:n], non_blocking=True)
+            stage.sent()
+            pos += n
+            done += n
+        return out
 
     def close(self) -> None:
         try:
