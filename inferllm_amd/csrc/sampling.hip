@@ -252,6 +252,145 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
     if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
 }
 
+// ---------------------------------------------------------------- sampler, small top_k
+// The same choice for 0 < top_k <= SB (the reference's default is 40) in a few passes over the
+// row instead of two bisections of 32 passes each: the top_k-th largest key by radix selection
+// (4 passes of 8 bits, histograms per wave in LDS), the kept ids gathered in id order into LDS,
+// top_p decided per kept id from the mass that lies before it in descending order, the draw by
+// inverse CDF over what is left.  Ties at the k-th value and at the top_p cut go to the lower ids.
+__global__ void __launch_bounds__(SB)
+sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
+                   int32_t* __restrict__ out, int V, float temp, int top_k, float top_p,
+                   float repeat_penalty, const int32_t* __restrict__ last_tokens, int n_last,
+                   const uint64_t* __restrict__ seeds, const int32_t* __restrict__ counters) {
+    constexpr int NW = SB / ILLM_WAVE;
+    __shared__ float red_f[NW];
+    __shared__ int red_i[NW];
+    __shared__ int last[256];
+    __shared__ int hist[NW][256];
+    __shared__ int sh_d, sh_above, sh_i;
+    __shared__ int cand_id[SB];
+    __shared__ float cand_s[SB];
+    const int b = blockIdx.x, tid = threadIdx.x, wave = tid / ILLM_WAVE;
+    const float* row = logits + (size_t)b * V;
+    float* s = scratch + (size_t)b * V;
+    const int nl = last_tokens ? min(n_last, 256) : 0;
+    if (tid < nl) last[tid] = last_tokens[(size_t)b * n_last + tid];
+
+    // 1. scaled scores; then the penalty, once for every id of the window
+    const float inv_temp = 1.0f / temp;
+    for (int i = tid; i < V; i += SB) s[i] = row[i] * inv_temp;
+    __syncthreads();
+    if (tid < nl) {
+        const int id = last[tid];
+        bool first = id >= 0 && id < V;
+        for (int j = 0; j < tid; ++j) first = first && last[j] != id;
+        if (first) {
+            const float l = row[id], v = l * inv_temp;
+            s[id] = l < 0.f ? v * repeat_penalty : v / repeat_penalty;
+        }
+    }
+    __syncthreads();
+
+    // 2. the key of the top_k-th largest score, 8 bits a pass; the largest score on the way
+    uint32_t prefix = 0;
+    int krem = top_k;
+    float mx = -INFINITY;
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        const uint32_t hi_mask = pass ? (0xffffffffu << (shift + 8)) : 0u;
+        for (int i = tid; i < NW * 256; i += SB) (&hist[0][0])[i] = 0;
+        __syncthreads();
+        for (int i = tid; i < V; i += SB) {
+            const float v = s[i];
+            if (pass == 0) mx = fmaxf(mx, v);
+            const uint32_t key = order_key(v);
+            if ((key & hi_mask) == prefix) atomicAdd(&hist[wave][(key >> shift) & 255u], 1);
+        }
+        __syncthreads();
+        if (tid < 256) {
+            int t = 0;
+            for (int w = 0; w < NW; ++w) t += hist[w][tid];
+            hist[0][tid] = t;
+        }
+        __syncthreads();
+        if (tid < 256) {
+            int above = 0;
+            for (int d = tid + 1; d < 256; ++d) above += hist[0][d];
+            if (above < krem && above + hist[0][tid] >= krem) { sh_d = tid; sh_above = above; }
+        }
+        __syncthreads();
+        prefix |= (uint32_t)sh_d << shift;
+        krem -= sh_above;
+        __syncthreads();
+    }
+    mx = block_max(mx, red_f);
+    // kept: key > prefix, and the first krem ids (ascending) with key == prefix
+
+    // 3. the kept ids and scores in id order into LDS
+    const int chunk = (V + SB - 1) / SB;
+    const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
+    int n_eq = 0, n_gt = 0;
+    for (int i = lo; i < hi; ++i) {
+        const uint32_t key = order_key(s[i]);
+        n_gt += key > prefix ? 1 : 0;
+        n_eq += key == prefix ? 1 : 0;
+    }
+    int total_i;
+    const int eq_before = block_exclusive_scan<int>(n_eq, red_i, &total_i);
+    const int eq_take = max(0, min(n_eq, krem - eq_before));
+    const int at0 = block_exclusive_scan<int>(n_gt + eq_take, red_i, &total_i);
+    const int n_kept = total_i;                        // == top_k
+    {
+        int at = at0, eq_left = eq_take;
+        for (int i = lo; i < hi; ++i) {
+            const float v = s[i];
+            const uint32_t key = order_key(v);
+            bool take = key > prefix;
+            if (key == prefix && eq_left > 0) { take = true; --eq_left; }
+            if (take && at < SB) { cand_id[at] = i; cand_s[at] = v; ++at; }
+        }
+    }
+    __syncthreads();
+
+    // 4. top_p: an id stays if the mass before it in descending order (ties: lower id first)
+    // does not yet reach top_p of the whole kept mass
+    const bool have = tid < n_kept;
+    const float my_s = have ? cand_s[tid] : -INFINITY;
+    const float my_p = have ? expf(my_s - mx) : 0.f;
+    bool stay = have;
+    if (top_p < 1.0f) {
+        const float z = block_sum_t<float>(my_p, red_f);
+        const float need = top_p * z;
+        if (have) {
+            float before = 0.f;
+            const uint32_t my_key = order_key(my_s);
+            for (int j = 0; j < n_kept; ++j) {
+                const uint32_t kj = order_key(cand_s[j]);
+                if (kj > my_key || (kj == my_key && j < tid)) before += expf(cand_s[j] - mx);
+            }
+            stay = before < need;
+        }
+    }
+
+    // 5. inverse CDF over what stays, in ascending id order (the order of the list)
+    const float mine = stay ? my_p : 0.f;
+    float total;
+    const float before = block_exclusive_scan<float>(mine, red_f, &total);
+    const float target = uniform_from(seeds[b], counters[b]) * total;
+    __syncthreads();
+    if (tid == 0) sh_i = -1;
+    __syncthreads();
+    if (mine > 0.f && target >= before && target < before + mine) atomicMax(&sh_i, cand_id[tid]);
+    __syncthreads();
+    if (sh_i < 0) {
+        // rounding put the target past the last id that stays: take that id
+        if (stay) atomicMax(&sh_i, cand_id[tid]);
+        __syncthreads();
+    }
+    if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
+}
+
 extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V,
                            float temp, int top_k, float top_p, float repeat_penalty,
                            const int32_t* last_tokens, int n_last, const uint64_t* seeds,
@@ -260,8 +399,13 @@ extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, in
         n_last < 0 || n_last > 256 || !seeds || !counters || !scratch)
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
-    hipLaunchKernelGGL(sample_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits, scratch,
-                       out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last, seeds,
-                       counters);
+    if (top_k > 0 && top_k <= SB && top_k < V)
+        hipLaunchKernelGGL(sample_topk_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
+                           scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
+                           seeds, counters);
+    else
+        hipLaunchKernelGGL(sample_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
+                           scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
+                           seeds, counters);
     return illm_launch_status();
 }

@@ -410,14 +410,15 @@ def interval_ok(logits_row, token, u, temperature, top_k, top_p, penalty, last):
 
 @pytest.mark.parametrize("V,temperature,top_k,top_p,penalty", [
     (256, 0.8, 0, 1.0, 1.0), (320, 0.8, 40, 0.95, 1.1), (411, 0.1, 40, 0.95, 1.3), (1000, 1.5, 5, 1.0, 1.0),
-    (32000, 1.0, 0, 0.9, 1.0), (300, 0.7, 1, 1.0, 1.0), (128256, 0.9, 50, 0.8, 1.2)])
+    (32000, 1.0, 0, 0.9, 1.0), (300, 0.7, 1, 1.0, 1.0), (128256, 0.9, 50, 0.8, 1.2),
+    (2000, 0.9, 1024, 0.7, 1.1), (2000, 0.9, 1025, 0.7, 1.0), (50, 1.0, 49, 0.5, 1.0), (32000, 0.1, 40, 0.95, 1.1)])
 def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top_p, penalty):
     from inferllm_amd.sampling.params import uniform
     B = 6
     logits = rnd(B, V, seed=8, std=2.0)
     logits[2] = 0.0                                            # all equal: ties everywhere
     last = torch.full((B, 8), -1, dtype=torch.int32)
-    last[:, :3] = torch.tensor([1, 5, V - 1], dtype=torch.int32)
+    last[:, :4] = torch.tensor([1, 5, V - 1, 5], dtype=torch.int32)     # an id twice: penalised once
     seeds = torch.tensor([3, 99, 12345, -7, 2**62, 0], dtype=torch.int64)
     counters = torch.tensor([0, 1, 2, 3, 4, 5], dtype=torch.int32)
     got = ops().sample(logits.to(DEV), temperature, top_k, top_p, penalty,
