@@ -22,6 +22,24 @@ class Sampler:
         params.validate()
         self.params = params
         self.device = device
+        self._stage: Optional[torch.Tensor] = None     # pinned [seeds (2 words each) | counters | windows]
+
+    def _upload(self, seeds, counters, windows):
+        """One pinned buffer, one copy: (seeds int64 [B], counters int32 [B], windows int32 [B, n] or None)."""
+        B = len(seeds)
+        n = len(windows[0]) if windows else 0
+        words = B * (3 + n)
+        if self._stage is None or self._stage.numel() < words:
+            self._stage = torch.empty(max(words, 1024), dtype=torch.int32,
+                                      pin_memory=torch.device(self.device).type == "cuda")
+        host = self._stage[:words]
+        host[:2 * B].view(torch.int64).copy_(torch.tensor([_as_i64(int(s)) for s in seeds], dtype=torch.int64))
+        host[2 * B:3 * B] = torch.tensor([int(c) for c in counters], dtype=torch.int32)
+        if n:
+            host[3 * B:] = torch.tensor(windows, dtype=torch.int32).view(-1)
+        dev = host.to(self.device, non_blocking=True)
+        return (dev[:2 * B].view(torch.int64), dev[2 * B:3 * B],
+                dev[3 * B:].view(B, n) if n else None)
 
     def __call__(self, logits: torch.Tensor, seeds: Sequence[int], counters: Sequence[int],
                  histories: Optional[Sequence[Sequence[int]]] = None) -> List[int]:
@@ -29,13 +47,10 @@ class Sampler:
         p = self.params
         if p.greedy:
             return ops.argmax(logits.contiguous()).tolist()
-        B = logits.shape[0]
-        last = None
+        rows = None
         if p.repeat_penalty != 1.0 and p.repeat_last_n > 0 and histories is not None:
             n = p.repeat_last_n
             rows = [([-1] * n + [int(t) for t in h])[-n:] for h in histories]
-            last = torch.tensor(rows, dtype=torch.int32, device=self.device)
-        seeds_t = torch.tensor([_as_i64(int(s)) for s in seeds], dtype=torch.int64, device=self.device)
-        counters_t = torch.tensor([int(c) for c in counters], dtype=torch.int32, device=self.device)
+        seeds_t, counters_t, last = self._upload(seeds, counters, rows)
         return ops.sample(logits.contiguous(), p.temperature, p.top_k, p.top_p, p.repeat_penalty,
                           last, seeds_t, counters_t).tolist()
