@@ -40,6 +40,11 @@ int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_pos, int ro
 int illm_gemm_generic(const void* X, int x_dt, const void* W, int w_dt, void* Y, int y_dt,
                       int M, int N, int K, void* stream);
 
+// The same product for M <= 16 rows when X and W are float32 and K % 4 == 0: W is read once
+// (decoding on the 32-bit path); plain float32 multiply-adds.
+int illm_gemv_rows_f32(const float* X, const float* W, void* Y, int y_dt, int M, int N, int K,
+                       void* stream);
+
 // Causal attention over packed rows of whole prompts (keys and values of the step
 // itself).  cu_seqlens[n_seqs + 1]; window <= 0: all earlier keys.
 int illm_attn_prefill_generic(const void* qkv, void* out, int dt, const int32_t* cu_seqlens,

@@ -76,3 +76,86 @@ extern "C" int illm_gemm_generic(const void* X, int x_dt, const void* W, int w_d
                        (hipStream_t)stream, X, x_dt, W, w_dt, Y, y_dt, M, N, K);
     return illm_launch_status();
 }
+
+
+// ---------------------------------------------------------------- few rows, float32
+// The same product for M <= 16 rows of float32 X and float32 W (decoding on the 32-bit path),
+// bound by reading W once: a block of 4 waves takes R = 64 / MR rows of W (MR = M rounded up to
+// 4, 8 or 16), the waves split K in interleaved pieces of 256, a lane multiplies 4 consecutive k
+// of every W row with every X row (plain multiply-adds, float32), and the R * MR sums of a wave
+// are added over its lanes by a halving exchange that leaves sum number l in lane l.  The waves'
+// sums are added in wave order.  The order of a sum depends on K only, not on the row's place.
+template <int MR>
+__global__ void __launch_bounds__(256)
+gemv_rows_f32_kernel(const float* __restrict__ X, const float* __restrict__ W, void* __restrict__ Y,
+                     int y_dt, int M, int N, int K) {
+    constexpr int R = 64 / MR;
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * R;
+    const float* wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wrow[r] = W + (size_t)min(n0 + r, N - 1) * K;
+    float acc[R][MR];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
+
+    for (int k = (wave * 64 + lane) * 4; k < K; k += 4 * 256) {      // K is a multiple of 4
+        float4 w[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[r] = *(const float4*)(wrow[r] + k);
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            const float4 x = *(const float4*)(X + (size_t)min(m, M - 1) * K + k);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                float a = acc[r][m];
+                a = fmaf(w[r].x, x.x, a);
+                a = fmaf(w[r].y, x.y, a);
+                a = fmaf(w[r].z, x.z, a);
+                a = fmaf(w[r].w, x.w, a);
+                acc[r][m] = a;
+            }
+        }
+    }
+    // 64 sums over 64 lanes: at the step that pairs lanes l and l ^ b a lane keeps the sums
+    // whose number has l's bit b; sum number e = r * MR + m ends in lane e
+    float v[64];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) v[r * MR + m] = acc[r][m];
+#pragma unroll
+    for (int b = 1, n = 32; b < 64; b <<= 1, n >>= 1) {
+        const bool up = (lane & b) != 0;
+#pragma unroll
+        for (int i = 0; i < n; ++i) {
+            const float keep = up ? v[2 * i + 1] : v[2 * i];
+            const float send = up ? v[2 * i] : v[2 * i + 1];
+            v[i] = keep + __shfl_xor(send, b, ILLM_WAVE);
+        }
+    }
+    part[wave][lane] = v[0];
+    __syncthreads();
+    if (wave == 0) {
+        const float t = ((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane];
+        const int r = lane / MR, m = lane % MR;
+        if (m < M && n0 + r < N) st_f(Y, y_dt, (size_t)m * N + n0 + r, t);
+    }
+}
+
+// float32 X [M <= 16, K] and W [N, K], K % 4 == 0; Y float32 or bfloat16.  Else ILLM_ERR_ARG.
+extern "C" int illm_gemv_rows_f32(const float* X, const float* W, void* Y, int y_dt, int M, int N,
+                                  int K, void* stream) {
+    if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K % 4) || !illm_dtype_ok(y_dt)) return ILLM_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (M <= 4)
+        hipLaunchKernelGGL(gemv_rows_f32_kernel<4>, dim3((N + 15) / 16), dim3(256), 0, st, X, W, Y, y_dt, M, N, K);
+    else if (M <= 8)
+        hipLaunchKernelGGL(gemv_rows_f32_kernel<8>, dim3((N + 7) / 8), dim3(256), 0, st, X, W, Y, y_dt, M, N, K);
+    else
+        hipLaunchKernelGGL(gemv_rows_f32_kernel<16>, dim3((N + 3) / 4), dim3(256), 0, st, X, W, Y, y_dt, M, N, K);
+    return illm_launch_status();
+}

@@ -204,6 +204,23 @@ def _operand(x):
     return x, None, 0, ctypes.c_float(0.0)
 
 
+def gemv_rows_f32_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.float32 and w.dtype == torch.float32 and x.dim() == 2 and w.dim() == 2
+            and 1 <= x.shape[0] <= 16 and x.shape[1] % 4 == 0 and x.shape[1] == w.shape[1]
+            and x.is_contiguous() and w.is_contiguous())
+
+
+def gemv_rows_f32(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M <= 16, K] . w [N, K]^T, both float32, plain float32 multiply-adds, W read once."""
+    _gpu(x, w)
+    _need(gemv_rows_f32_fits(x, w), "gemv_rows_f32: operands not taken")
+    M, K = x.shape
+    y = torch.empty((M, w.shape[0]), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_gemv_rows_f32(_p(x), _p(w), _p(y), _code(y), M, w.shape[0], K, _stream()),
+           "gemv_rows_f32")
+    return y
+
+
 def linear_add_fits(x, w: torch.Tensor, into: torch.Tensor) -> bool:
     """Whether `linear_add` takes these operands (few bfloat16 rows into float32 rows)."""
     return (isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
@@ -246,6 +263,8 @@ def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch
         x = x.rows()
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.float32 or w.dtype == torch.float32:
+        if gemv_rows_f32_fits(x, w):
+            return gemv_rows_f32(x, w, out_dtype)
         return gemm_generic(x, w, out_dtype)
     M, K = x.shape
     if M == 0:

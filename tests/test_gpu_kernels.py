@@ -288,6 +288,22 @@ def test_gate_up_silu(M, F, K):
     assert not torch.allclose(got.double().cpu(), swapped, atol=0.1 * float(want.abs().max()))
 
 
+@pytest.mark.parametrize("ydt", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 100, 136), (16, 33, 1000), (5, 320, 96), (3, 7, 4), (9, 11008, 4096)])
+def test_gemv_rows_f32(ydt, M, N, K):
+    """The 32-bit path's product of few rows: float32 sums, W read once."""
+    x, w = rnd(M, K, seed=1), rnd(N, K, seed=2)
+    assert ops().gemv_rows_f32_fits(x.to(DEV), w.to(DEV))
+    got = ops().linear(x.to(DEV), w.to(DEV), ydt)
+    want = R.linear(x, w, torch.float64)
+    if ydt == torch.float32:
+        torch.testing.assert_close(got.double().cpu(), want, atol=2e-6 * math.sqrt(K) * 4, rtol=1e-5)
+    else:
+        close(got, want, ydt, scale=math.sqrt(K))
+    assert not ops().gemv_rows_f32_fits(rnd(17, K).to(DEV), w.to(DEV))
+    assert not ops().gemv_rows_f32_fits(x.to(DEV).to(torch.bfloat16), w.to(DEV))
+
+
 def test_products_of_many_rows_are_planned_once_and_stay_right():
     """A product of many rows is measured whole and cut along its output columns, once per
     shape; whatever plan wins, every element is the plain product."""
