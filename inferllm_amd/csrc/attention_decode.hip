@@ -41,7 +41,7 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     constexpr int NI = LPR < 16 ? LPR : 16;    // load instructions per tile
     constexpr int TK = NI * KPI;               // keys per tile
     extern __shared__ float wave_res[];        // [waves][GC][hd + 2], used when waves > 1
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index(), waves = blockDim.x >> 6;
     const int q = lane / LPR, c = lane % LPR;
     const int G = nh / nkv;
     const int kvh = blockIdx.x % nkv, g0 = (blockIdx.x / nkv) * GC;
@@ -261,7 +261,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
     constexpr int PLD = 20;                    // floats per key row of P in LDS (16 heads + pad)
     // per wave 64 * PLD floats of P; after the tiles the same memory holds the waves' results
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index(), waves = blockDim.x >> 6;
     float* ps = lds + (size_t)wave * 64 * PLD;
     const int r = lane & 15, q4 = lane >> 4;   // MFMA roles: key / head, and k group
     const int q = lane / LPR, c = lane % LPR;  // V row roles

@@ -61,7 +61,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     if (q0 >= len) return;
     const int kvh = h / (nh / nkv);
     const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, wave = wave_index(), lane = tid & 63;
     const int lq = lane & 31, half = lane >> 5;
     const int q_row0 = q0 + wave * 32;
     const int q = q_row0 + lq;

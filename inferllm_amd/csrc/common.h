@@ -53,6 +53,12 @@ __device__ __forceinline__ uint4 ld16_stream(const void* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// The wave's number within its block, as a value the compiler knows to be the same in all
+// lanes: loops and branches on it run on the scalar unit instead of under lane masks.
+__device__ __forceinline__ int wave_index() {
+    return __builtin_amdgcn_readfirstlane((int)(threadIdx.x / ILLM_WAVE));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = ILLM_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, ILLM_WAVE);

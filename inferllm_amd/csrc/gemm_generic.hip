@@ -91,7 +91,7 @@ gemv_rows_f32_kernel(const float* __restrict__ X, const float* __restrict__ W, v
                      int y_dt, int M, int N, int K) {
     constexpr int R = 64 / MR;
     __shared__ float part[4][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     const int n0 = blockIdx.x * R;
     const float* wrow[R];
 #pragma unroll

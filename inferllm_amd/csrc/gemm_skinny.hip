@@ -68,7 +68,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     // a wave's piece of LDS: first the staging of its W lines (NTB * SK_U KB), then its sums
     constexpr int SK_REGION_FLOATS = NTB * (SK_U > MT ? SK_U : MT) * 256;
     extern __shared__ float red[];   // [waves][SK_REGION_FLOATS]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     const int waves = blockDim.x >> 6;
     const int r = lane & 15, q = lane >> 4;
     // consumer: the last wave, which has the fewest pieces of K if they do not divide evenly, adds
