@@ -138,19 +138,27 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
         }
         const bool need_mask = (k0 + PF_BN > q_row0 + 1) || (k0 + PF_BN > len) || (window > 0);
         float mx = NEG_INF;
+        if (need_mask) {                 // the same for the whole wave: one branch, two bodies
 #pragma unroll
-        for (int sub = 0; sub < 2; ++sub)
+            for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float v = s[sub][i] * scale_log2;
-                if (need_mask) {
+                for (int i = 0; i < 16; ++i) {
                     const int key = k0 + sub * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
                     const bool ok = key <= q && key < len && (window <= 0 || key > q - window);
-                    v = ok ? v : NEG_INF;
+                    const float v = ok ? s[sub][i] * scale_log2 : NEG_INF;
+                    s[sub][i] = v;
+                    mx = fmaxf(mx, v);
                 }
-                s[sub][i] = v;
-                mx = fmaxf(mx, v);
-            }
+        } else {
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float v = s[sub][i] * scale_log2;
+                    s[sub][i] = v;
+                    mx = fmaxf(mx, v);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
