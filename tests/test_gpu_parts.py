@@ -116,6 +116,47 @@ def test_norm_feed_forward_and_block_parts(dtype):
     assert rel(out, P.swiglu_ffn(h.cpu(), w["g"], w["u"], w["d"])) < TOL[dtype]
 
 
+def test_feed_forward_adds_to_the_stream_and_prepares_the_next_norm():
+    """The short cut of few bfloat16 rows: the feed-forward adds its output to the residual rows
+    itself and hands on rows prepared for the norm that follows; a block takes them only for
+    the norm they were made for, and a part that does not take them gets plain normed rows."""
+    from inferllm_amd.parts import build_part
+    from inferllm_amd.parts.block import PreNormBlock
+    from inferllm_amd.config import PartSpec
+    from inferllm_amd.kernels import ops
+    dtype, E, F, eps = torch.bfloat16, 64, 96, 1e-5
+    mk_norm = lambda name: build_part("norm", PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": name}))
+    n_next, n_other = mk_norm("n1"), mk_norm("n2")
+    ffn = build_part("feed_forward", PartSpec("swiglu", {"hidden_size": E, "intermediate_size": F},
+                                              {"gate": "g", "up": "u", "down": "d"}))
+    w = {"n1": (1 + rnd(E, seed=1, std=0.2)).to(dtype), "n2": (1 + rnd(E, seed=7, std=0.2)).to(dtype),
+         "g": rnd(F, E, seed=2, std=0.2).to(dtype), "u": rnd(F, E, seed=3, std=0.2).to(dtype),
+         "d": rnd(E, F, seed=4, std=0.2).to(dtype)}
+    for p in (n_next, n_other, ffn):
+        p.load({k: v.to(DEV) for k, v in w.items()})
+    cache, slots = make_ctx([0], None, {}, dtype)
+    ctx = step_ctx(cache, slots, [0], [5], dtype, False)
+    x = rnd(5, E, seed=5, std=0.5)
+    h = rnd(5, E, seed=6, std=0.5).to(dtype)
+    want_x = x.double() + P.swiglu_ffn(h, w["g"], w["u"], w["d"])
+    xg = x.to(DEV)
+    rows = ffn.forward(h.to(DEV), ctx, residual=xg, next_norm=n_next)
+    assert isinstance(rows, ops.NormedRows) and rows.x is xg
+    assert rel(xg, want_x) < TOL[dtype]                                   # the sum is in the stream
+    takes = type("Takes", (), {"takes_normed_rows": True})()
+    plain = type("Plain", (), {"takes_normed_rows": False})()
+    assert PreNormBlock._enter(n_next, takes, xg, rows, ctx) is rows       # made for this norm
+    got = PreNormBlock._enter(n_next, plain, xg, rows, ctx)                # a part that wants rows
+    assert rel(got, P.rms_norm(want_x, w["n1"], eps)) < TOL[dtype]
+    got = PreNormBlock._enter(n_other, takes, xg, rows, ctx)               # made for another norm
+    assert isinstance(got, torch.Tensor) and rel(got, P.rms_norm(want_x, w["n2"], eps)) < TOL[dtype]
+    assert rel(xg, want_x) < TOL[dtype]                                   # and nothing was added twice
+    # the product of the prepared rows is the product of the normed rows
+    wq = rnd(40, E, seed=9, std=0.2).to(dtype)
+    want = P.linear(P.rms_norm(want_x, w["n1"], eps), wq)
+    assert rel(ops.linear(rows, wq.to(DEV)), want) < TOL[dtype]
+
+
 @pytest.mark.parametrize("n_reqs", [3, 20])
 def test_decode_graph_replays_equal_eager_steps(tmp_path, n_reqs):
     """The same decode steps through the captured HIP graph (replayed many times, with other
