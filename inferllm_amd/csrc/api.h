@@ -78,14 +78,21 @@ int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache, const 
 // ssq != null (M <= 16 only): X is bfloat16(x * norm weight) of residual rows x whose sums of
 // squares lie in ssq[M][parts] (left by illm_gemm_skinny_add), and row m of the result is scaled
 // by 1 / sqrt(sum_p ssq[m][p] / K + eps): the product of the RMS norm of x.
-int illm_gemm_skinny_bf16(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
-                          const float* ssq, int parts, float eps, void* stream);
+// Wt (here and below, may be null): a copy of W laid out for these kernels,
+// [tile][K / 32][16 rows][32 k] with tile t holding the 16 rows that block t works on (plain
+// product: rows 16 t ..; gate|up: 8 gate rows 8 t .. and the same 8 up rows; q|k|v: 8 rows of a
+// head and their 8 rotation partners, then 16 rows per tile for v), rows beyond the matrix zero.
+// Used when M <= 16 and K % 32 == 0; W itself is then not read.
+int illm_gemm_skinny_bf16(const void* X, const void* W, const void* Wt, void* Y, int y_dt, int M,
+                          int N, int K, const float* ssq, int parts, float eps, int waves_wanted,
+                          void* stream);
 
 // Y[M, N] (float32 residual rows) += X . W^T for M <= 16 bfloat16 rows.  nw != null (the weight of
 // the RMS norm that follows, bfloat16 or float32 [N]): also xb[M, N] = bfloat16(Y * nw) and
 // ssq_out[M][ceil(N / 16)], partial sums of Y^2, for a product that takes `ssq`.
-int illm_gemm_skinny_add(const void* X, const void* W, float* Y, int M, int N, int K,
-                         const void* nw, int nw_dt, void* xb, float* ssq_out, void* stream);
+int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y, int M, int N,
+                         int K, const void* nw, int nw_dt, void* xb, float* ssq_out,
+                         int waves_wanted, void* stream);
 
 // Tuning entry of the same product: rows of W per block 16 * ntb (ntb 1, 2, 4), u * 64 bytes
 // of a W row per wave iteration (u 4, 8), waves per block.
@@ -94,15 +101,15 @@ int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, i
 
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
 // product, `ssq` included.  waves_wanted: waves per block (0: the default choice).
-int illm_gemm_skinny_gateup_silu(const void* X, const void* W, void* Y, int y_dt, int M, int F,
-                                 int K, const float* ssq, int parts, float eps, int waves_wanted,
-                                 void* stream);
+int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const void* Wt, void* Y, int y_dt,
+                                 int M, int F, int K, const float* ssq, int parts, float eps,
+                                 int waves_wanted, void* stream);
 
 // Few bfloat16 rows (M <= 16, hd % 16 == 0): the q|k|v product, the rotation of q and k (pairs
 // (i, i + hd/2), all dims) at row_pos[m], q into Y[M, (nh + 2 nkv) hd] (k and v parts untouched),
 // k and v into the paged cache of row_slot[m], all in one kernel.  ssq: as for
 // illm_gemm_skinny_bf16.  waves_wanted: waves per block (0: the default choice).
-int illm_qkv_rope_store_skinny(const void* X, const void* W, void* Y, int M, int K,
+int illm_qkv_rope_store_skinny(const void* X, const void* W, const void* Wt, void* Y, int M, int K,
                                const float* cos_sin, int max_pos, const int32_t* row_pos,
                                const int32_t* row_slot, void* kcache, void* vcache,
                                const int32_t* page_table, int table_stride, int page_size, int ring,

@@ -11,6 +11,7 @@ from typing import Dict, List, Optional, Sequence, Union
 
 import torch
 
+from ..kernels import ops
 from ..cache.manager import PAGE_SIZE, CacheManager, round_up
 from ..config.registry import config_from_dict, load_config
 from ..sampling.params import SamplingParams
@@ -40,6 +41,9 @@ class Engine:
     residual stream, statistics and logits.  dtype "float32": everything in true
     float32 (own multiply-add kernels; no matrix-core or reduced-precision mode).
 
+    `decode_copies`: keep a second copy of every matrix in the layout of the few-rows kernels
+    (decoding reads that one, prompts the row-major one); default: if it fits comfortably.
+
     Cache size: `max_tokens` is the most tokens live sequences hold together (each
     rounded up to 64), `max_batch` the most live sequences, `max_seq_len` the longest
     sequence (default: the model's max positions).
@@ -48,7 +52,7 @@ class Engine:
     def __init__(self, config, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  max_batch: int = 8, max_seq_len: Optional[int] = None,
                  max_tokens: Optional[int] = None, use_graphs: bool = True,
-                 poison_freed: bool = False):
+                 poison_freed: bool = False, decode_copies: Optional[bool] = None):
         self.config = config
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
@@ -59,7 +63,18 @@ class Engine:
         torch.cuda.set_device(self.device)
         self.spec = config.to_spec()
         self.model = DecoderModel(self.spec)
-        self.model.load(tensors)
+        if decode_copies is None:
+            # a second copy of the matrices, laid out for the few-rows kernels of decoding, if it
+            # takes no more than a quarter of the memory that is free now
+            nbytes = sum(t.numel() * t.element_size() for t in tensors.values() if t.dim() == 2)
+            free, _total = torch.cuda.mem_get_info(self.device)
+            decode_copies = self.dtype == torch.bfloat16 and nbytes <= free // 4
+        self.decode_copies = bool(decode_copies) and self.dtype == torch.bfloat16
+        ops.DECODE_COPIES = self.decode_copies
+        try:
+            self.model.load(tensors)
+        finally:
+            ops.DECODE_COPIES = False
         limit = self.spec.max_positions
         self.max_seq_len = min(int(max_seq_len), limit) if max_seq_len else limit
         self.max_batch = int(max_batch)

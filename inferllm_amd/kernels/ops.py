@@ -172,6 +172,81 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> to
     return y
 
 
+class Weight:
+    """A matrix [N, K] of a product with, optionally, a second copy laid out for the few-rows
+    kernels (`tile_weight`).  Wherever the ops take a weight they take this or a plain tensor."""
+    __slots__ = ("plain", "tiled")
+
+    def __init__(self, plain: torch.Tensor, tiled: Optional[torch.Tensor] = None):
+        self.plain, self.tiled = plain, tiled
+
+    @property
+    def shape(self):
+        return self.plain.shape
+
+    @property
+    def dtype(self):
+        return self.plain.dtype
+
+
+DECODE_COPIES = False         # whether `decode_weight` makes the second copy (set by the engine)
+
+
+def _w(w):
+    """(plain tensor, pointer of the tiled copy or None) of a weight argument."""
+    if isinstance(w, Weight):
+        return w.plain, (_p(w.tiled) if w.tiled is not None else None)
+    return w, None
+
+
+def plain_weight(w) -> torch.Tensor:
+    return w.plain if isinstance(w, Weight) else w
+
+
+def tile_rows(N: int, mode: str = "plain", nh: int = 0, nkv: int = 0, hd: int = 0) -> torch.Tensor:
+    """Row numbers (int64 [tiles, 16], -1 = a zero row) of the tiles the few-rows kernels work on.
+    "plain": 16 consecutive rows.  "gate_up" (N = 2F rows [gate | up]): 8 gate rows and the same
+    8 up rows.  "qkv" (rows [q heads | k heads | v heads]): 8 rows of a q or k head and their
+    rotation partners hd/2 further, then 16 consecutive rows of v."""
+    if mode == "plain":
+        t = torch.arange(((N + 15) // 16) * 16).view(-1, 16)
+        return torch.where(t < N, t, torch.full_like(t, -1))
+    if mode == "gate_up":
+        F = N // 2
+        lo = torch.arange(((F + 7) // 8) * 8).view(-1, 8)
+        ok = lo < F
+        return torch.cat([torch.where(ok, lo, torch.full_like(lo, -1)),
+                          torch.where(ok, lo + F, torch.full_like(lo, -1))], dim=1)
+    if mode == "qkv":
+        heads = torch.arange(nh + nkv).view(-1, 1, 1) * hd
+        j = torch.arange(hd // 16).view(1, -1, 1) * 8
+        i = torch.arange(8).view(1, 1, -1)
+        lo = (heads + j + i).view(-1, 8)
+        rot = torch.cat([lo, lo + hd // 2], dim=1)
+        v = ((nh + nkv) * hd + torch.arange(nkv * hd)).view(-1, 16)
+        return torch.cat([rot, v], dim=0)
+    raise ValueError(f"unknown tile mode {mode!r}")
+
+
+def tile_weight(w: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    """The copy [tiles][K / 32][16][32] of w [N, K] for the given tiles of rows (K % 32 == 0)."""
+    N, K = w.shape
+    _need(K % 32 == 0 and w.dtype == torch.bfloat16, "tile_weight: bfloat16 with K a multiple of 32")
+    rows = rows.to(w.device)
+    picked = w[rows.clamp(min=0).view(-1)]
+    picked[(rows < 0).view(-1)] = 0
+    return picked.view(rows.shape[0], 16, K // 32, 32).permute(0, 2, 1, 3).contiguous()
+
+
+def decode_weight(w: torch.Tensor, mode: str = "plain", **geometry):
+    """The weight as the parts keep it: with a tiled copy for the few-rows kernels if the engine
+    asked for decode copies and the matrix allows it, else the tensor itself."""
+    if (DECODE_COPIES and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0
+            and w.is_cuda and (mode != "qkv" or geometry.get("hd", 0) % 16 == 0)):
+        return Weight(w, tile_weight(w, tile_rows(w.shape[0], mode, **geometry)))
+    return w
+
+
 class NormedRows:
     """Residual rows whose RMS norm the next product takes itself (few rows, bfloat16).
 
@@ -221,47 +296,53 @@ def gemv_rows_f32(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> t
     return y
 
 
-def linear_add_fits(x, w: torch.Tensor, into: torch.Tensor) -> bool:
+def linear_add_fits(x, w, into: torch.Tensor) -> bool:
     """Whether `linear_add` takes these operands (few bfloat16 rows into float32 rows)."""
+    w = plain_weight(w)
     return (isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
             and x.dim() == 2 and w.dim() == 2 and into.dtype == torch.float32 and
             into.is_contiguous() and 1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0
             and w.shape[1] == x.shape[1] and into.shape == (x.shape[0], w.shape[0]))
 
 
-def linear_add(x: torch.Tensor, w: torch.Tensor, into: torch.Tensor, norm=None,
+def linear_add(x: torch.Tensor, w, into: torch.Tensor, norm=None,
                act_dtype: torch.dtype = torch.bfloat16) -> Optional[NormedRows]:
     """into += x . w^T in the product's kernel: the residual add of a block's output projection,
     each element added by the one thread that owns it.  norm = (weight [N], eps) of the RMS norm
     that follows: the kernel also leaves what the next few-rows product needs to take that norm
     itself, returned as `NormedRows` (only if N % 8 == 0, else None as without `norm`)."""
-    _gpu(x, w, into)
     _need(linear_add_fits(x, w, into), "linear_add: operands not taken")
+    w, wt = _w(w)
+    _gpu(x, w, into)
     M, K = x.shape
     N = w.shape[0]
     if norm is not None and (N % 8 or norm[0].dtype not in _CODES or act_dtype != torch.bfloat16
                              or norm[0].shape != (N,)):
         norm = None
     if norm is None:
-        _check(_lib().illm_gemm_skinny_add(_p(x), _p(w), _p(into), M, N, K, None, BF16, None, None,
-                                           _stream()), "linear_add")
+        _check(_lib().illm_gemm_skinny_add(_p(x), _p(w), wt, _p(into), M, N, K, None, BF16, None,
+                                           None, PLAIN_WAVES, _stream()), "linear_add")
         return None
     weight, eps = norm
     _gpu(weight)
     xb = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     ssq = torch.empty((M, (N + 15) // 16), dtype=torch.float32, device=x.device)
-    _check(_lib().illm_gemm_skinny_add(_p(x), _p(w), _p(into), M, N, K, _p(weight), _code(weight),
-                                       _p(xb), _p(ssq), _stream()), "linear_add")
+    _check(_lib().illm_gemm_skinny_add(_p(x), _p(w), wt, _p(into), M, N, K, _p(weight),
+                                       _code(weight), _p(xb), _p(ssq), PLAIN_WAVES, _stream()),
+           "linear_add")
     return NormedRows(into, weight, eps, act_dtype, xb, ssq)
 
 
-def linear(x, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """y = x . w^T, w stored [out, in] (src/kern/naive/naive.cpp:363-379).  x may be `NormedRows`."""
+def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """y = x . w^T, w stored [out, in] (src/kern/naive/naive.cpp:363-379).  x may be
+    `NormedRows`, w a `Weight`."""
     if isinstance(x, NormedRows):
         if w.dtype == torch.bfloat16:
             return gemm_skinny_bf16(x, w, out_dtype or x.dtype)
         x = x.rows()
     out_dtype = out_dtype or x.dtype
+    if isinstance(w, Weight) and not (x.dtype == torch.bfloat16 and 1 <= x.shape[0] <= SKINNY_BEST_ROWS):
+        w = w.plain                                      # only the few-rows kernel reads the copy
     if x.dtype == torch.float32 or w.dtype == torch.float32:
         if gemv_rows_f32_fits(x, w):
             return gemv_rows_f32(x, w, out_dtype)
@@ -348,10 +429,11 @@ def skinny_fits(M: int, N: int, K: int) -> bool:
     return 1 <= M <= SKINNY_MAX_ROWS and K % 8 == 0
 
 
-def gemm_skinny_bf16(x, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+def gemm_skinny_bf16(x, w, out_dtype: torch.dtype) -> torch.Tensor:
     """x [M <= 64, K] . w [N, K]^T, both bfloat16, float32 accumulation on the matrix cores; or
     x `NormedRows`: the product of the normed rows."""
     xt, ssq, parts, eps = _operand(x)
+    w, wt = _w(w)
     _gpu(xt, w)
     _need(xt.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny: bfloat16 operands")
     _need(xt.dim() == 2 and w.dim() == 2 and xt.shape[1] == w.shape[1],
@@ -360,22 +442,23 @@ def gemm_skinny_bf16(x, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor
     N = w.shape[0]
     _need(skinny_fits(M, N, K), f"gemm_skinny: M={M} K={K} not taken")
     y = torch.empty((M, N), dtype=out_dtype, device=xt.device)
-    _check(_lib().illm_gemm_skinny_bf16(_p(xt), _p(w), _p(y), _code(y), M, N, K, ssq, parts, eps,
-                                        _stream()), "gemm_skinny")
+    _check(_lib().illm_gemm_skinny_bf16(_p(xt), _p(w), wt, _p(y), _code(y), M, N, K, ssq, parts,
+                                        eps, PLAIN_WAVES, _stream()), "gemm_skinny")
     return y
 
 
 QKV_ROPE_WAVES = 0       # waves per block of the fused kernel; 0: the kernel's own choice
 GATE_UP_WAVES = 0        # the same for the fused gate|up product
+PLAIN_WAVES = 0          # and for the plain few-rows product
 
 
-def qkv_rope_store_fits(x, w_qkv: torch.Tensor, hd: int) -> bool:
+def qkv_rope_store_fits(x, w_qkv, hd: int) -> bool:
     """Whether the one-kernel q|k|v product + rotation + cache store takes these operands."""
     return (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and
             1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0 and hd % 16 == 0)
 
 
-def qkv_rope_store(x, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
+def qkv_rope_store(x, w_qkv, cos_sin: torch.Tensor,
                    row_pos: torch.Tensor, row_slot: torch.Tensor, kcache: torch.Tensor,
                    vcache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
                    nh: int, nkv: int, hd: int) -> torch.Tensor:
@@ -383,11 +466,12 @@ def qkv_rope_store(x, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
     returned in rows [q | k | v] whose k and v parts are NOT filled, k and v stored in the cache.
     x may be `NormedRows`."""
     xt, ssq, parts, eps = _operand(x)
+    _need(qkv_rope_store_fits(x, w_qkv, hd), "qkv_rope_store: operands not taken")
+    w_qkv, wt = _w(w_qkv)
     _gpu(xt, w_qkv, cos_sin, row_pos, row_slot, kcache, vcache, page_table)
     _i32(row_pos, x.shape[0]); _i32(row_slot, x.shape[0]); _i32(page_table)
     M, K = x.shape
     N = (nh + 2 * nkv) * hd
-    _need(qkv_rope_store_fits(x, w_qkv, hd), "qkv_rope_store: operands not taken")
     _need(w_qkv.shape == (N, K), f"qkv_rope_store: weight {tuple(w_qkv.shape)} vs ({N}, {K})")
     _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[1] * 2 == hd and
           cos_sin.shape[2] == 2, "qkv_rope_store: angle table must be float32 [max_pos, hd/2, 2]")
@@ -396,13 +480,13 @@ def qkv_rope_store(x, w_qkv: torch.Tensor, cos_sin: torch.Tensor,
           "qkv_rope_store: cache shape or dtype")
     y = torch.empty((M, N), dtype=torch.bfloat16, device=xt.device)
     _check(_lib().illm_qkv_rope_store_skinny(
-        _p(xt), _p(w_qkv), _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
+        _p(xt), _p(w_qkv), wt, _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
         _p(kcache), _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, nh, nkv, hd,
         ssq, parts, eps, QKV_ROPE_WAVES, _stream()), "qkv_rope_store")
     return y
 
 
-def gate_up_silu(x, w_gate_up: torch.Tensor) -> torch.Tensor:
+def gate_up_silu(x, w_gate_up) -> torch.Tensor:
     """silu(x . Wg^T) * (x . Wu^T) for w_gate_up = [Wg | Wu] stacked as [2F, K].
 
     Few bfloat16 rows: one fused MFMA kernel.  Otherwise the product and `silu_mul`.
@@ -414,16 +498,17 @@ def gate_up_silu(x, w_gate_up: torch.Tensor) -> torch.Tensor:
     if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and F2 % 2 == 0
             and 1 <= M <= SKINNY_BEST_ROWS and K % 8 == 0):
         xt, ssq, parts, eps = _operand(x)
-        _gpu(xt, w_gate_up)
-        _need(w_gate_up.dim() == 2 and w_gate_up.shape[1] == K, "gate_up_silu: shapes")
+        wp, wt = _w(w_gate_up)
+        _gpu(xt, wp)
+        _need(wp.dim() == 2 and wp.shape[1] == K, "gate_up_silu: shapes")
         y = torch.empty((M, F2 // 2), dtype=x.dtype, device=xt.device)
-        _check(_lib().illm_gemm_skinny_gateup_silu(_p(xt), _p(w_gate_up), _p(y), _code(y), M,
+        _check(_lib().illm_gemm_skinny_gateup_silu(_p(xt), _p(wp), wt, _p(y), _code(y), M,
                                                    F2 // 2, K, ssq, parts, eps, GATE_UP_WAVES,
                                                    _stream()), "gate_up_silu")
         return y
     if isinstance(x, NormedRows):
         x = x.rows()
-    return silu_mul(linear(x, w_gate_up))
+    return silu_mul(linear(x, plain_weight(w_gate_up)))
 
 
 # ------------------------------------------------------------------ attention

@@ -57,8 +57,9 @@ class Attention(Mixer):
         return KVSpec("window" if self.window else "full", self.nkv, self.hd, self.window)
 
     def load(self, tensors) -> None:
-        self.w_qkv = _fuse([self._take(tensors, n) for n in ("q", "k", "v")])
-        self.w_o = self._take(tensors, "o").contiguous()
+        self.w_qkv = ops.decode_weight(_fuse([self._take(tensors, n) for n in ("q", "k", "v")]),
+                                       "qkv", nh=self.nh, nkv=self.nkv, hd=self.hd)
+        self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous())
 
     def forward(self, h, ctx: StepContext, line, writes_cache, position, residual=None,
                 next_norm=None):
@@ -78,7 +79,7 @@ class Attention(Mixer):
         else:
             # keys and values are those an earlier run of this step stored on the line: only q
             # is projected and encoded (as packed rows with no kv heads)
-            q = ops.linear(h, self.w_qkv[: nh * hd])
+            q = ops.linear(h, ops.plain_weight(self.w_qkv)[: nh * hd])
             if position is not None:
                 position.on_qkv(q, ctx, nh, 0, hd, None, None, None)
             if ctx.prefill:

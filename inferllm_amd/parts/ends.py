@@ -54,7 +54,8 @@ class LMHead(Head):
 
     def load(self, tensors) -> None:
         own = self.tensors["weight"]
-        self.weight = (tensors[own] if own in tensors else tensors[self.tied_fallback]).contiguous()
+        self.weight = ops.decode_weight(
+            (tensors[own] if own in tensors else tensors[self.tied_fallback]).contiguous())
 
     def forward(self, h, ctx: StepContext):
         return ops.linear(h, self.weight, out_dtype=torch.float32)

@@ -34,8 +34,9 @@ class SwiGLU(FeedForward):
                 "down": TensorWant((self.E, self.F))}
 
     def load(self, tensors) -> None:
-        self.w_gate_up = _fuse([self._take(tensors, "gate"), self._take(tensors, "up")])
-        self.w_down = self._take(tensors, "down").contiguous()
+        self.w_gate_up = ops.decode_weight(_fuse([self._take(tensors, "gate"), self._take(tensors, "up")]),
+                                           "gate_up")
+        self.w_down = ops.decode_weight(self._take(tensors, "down").contiguous())
 
     def forward(self, h, ctx: StepContext, residual=None, next_norm=None):
         a = ops.gate_up_silu(h, self.w_gate_up)

@@ -304,6 +304,54 @@ def test_gemv_rows_f32(ydt, M, N, K):
     assert not ops().gemv_rows_f32_fits(x.to(DEV).to(torch.bfloat16), w.to(DEV))
 
 
+def _decode_copy(w, mode="plain", **geometry):
+    o = ops()
+    return o.Weight(w, o.tile_weight(w, o.tile_rows(w.shape[0], mode, **geometry)))
+
+
+def test_tile_rows_cover_every_row_once():
+    o = ops()
+    for rows, N in ((o.tile_rows(100), 100), (o.tile_rows(2 * 44, "gate_up"), 88),
+                    (o.tile_rows((6 + 2 * 3) * 48, "qkv", nh=6, nkv=3, hd=48), 12 * 48)):
+        assert rows.shape[1] == 16
+        kept = rows[rows >= 0]
+        assert sorted(kept.tolist()) == list(range(N))
+    g = o.tile_rows(2 * 44, "gate_up")
+    assert g[5, :8].tolist() == [40, 41, 42, 43, -1, -1, -1, -1] and g[5, 8:12].tolist() == [84, 85, 86, 87]
+    q = o.tile_rows((2 + 2) * 32, "qkv", nh=2, nkv=1, hd=32)
+    assert q[1].tolist() == list(range(8, 16)) + list(range(24, 32))          # a row and its partner hd/2 on
+    assert q[-1].tolist() == list(range(3 * 32 + 16, 4 * 32))                  # v: 16 rows in a run
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 100, 160), (16, 33, 992), (5, 320, 96), (9, 4096, 11008)])
+def test_products_from_the_decode_copy_equal_those_from_the_matrix(M, N, K, monkeypatch):
+    """The copy laid out for the few-rows kernels holds the same numbers in another order: with
+    K cut over the same number of waves the products are the same sums in the same order, bit
+    for bit."""
+    o = ops()
+    for knob in ("PLAIN_WAVES", "GATE_UP_WAVES", "QKV_ROPE_WAVES"):
+        monkeypatch.setattr(o, knob, 3)
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1).to(DEV), rnd(N, K, dtype=torch.bfloat16, seed=2).to(DEV)
+    wc = _decode_copy(w)
+    assert wc.tiled.shape == ((N + 15) // 16, K // 32, 16, 32)
+    for ydt in DTYPES:
+        assert torch.equal(o.linear(x, wc, ydt), o.linear(x, w, ydt))
+    into_a, into_b = rnd(M, N, seed=3).to(DEV), rnd(M, N, seed=3).to(DEV)
+    nw = (1 + rnd(N, seed=4) * 0.3).to(torch.bfloat16).to(DEV)
+    ra, rb = o.linear_add(x, wc, into_a, (nw, 1e-5)), o.linear_add(x, w, into_b, (nw, 1e-5))
+    assert torch.equal(into_a, into_b)
+    if ra is not None:
+        assert torch.equal(ra.xb, rb.xb) and torch.equal(ra.ssq, rb.ssq)
+        w2 = rnd(48, N, dtype=torch.bfloat16, seed=5).to(DEV)
+        if N % 32 == 0:
+            assert torch.equal(o.linear(ra, _decode_copy(w2)), o.linear(rb, w2))
+    if K % 64 == 0:                                        # gate|up: N rows as two halves
+        wg = rnd(2 * 56, K, dtype=torch.bfloat16, seed=6, std=0.2).to(DEV)
+        assert torch.equal(o.gate_up_silu(x, _decode_copy(wg, "gate_up")), o.gate_up_silu(x, wg))
+    xl = rnd(17, K, dtype=torch.bfloat16, seed=7).to(DEV)     # more rows: the matrix itself is read
+    assert torch.equal(o.linear(xl, wc), o.linear(xl, w))
+
+
 def test_products_of_many_rows_are_planned_once_and_stay_right():
     """A product of many rows is measured whole and cut along its output columns, once per
     shape; whatever plan wins, every element is the plain product."""
@@ -501,9 +549,10 @@ def test_window_edge_prefill_and_decode(dtype, hd):
 
 
 @pytest.mark.parametrize("M,nh,nkv,hd,K", [(1, 32, 32, 128, 4096), (8, 4, 2, 32, 64), (16, 6, 3, 64, 200), (3, 8, 1, 96, 72),
-                                          (5, 3, 3, 48, 136), (2, 2, 1, 16, 40)])
+                                          (5, 3, 3, 48, 136), (2, 2, 1, 16, 40), (5, 3, 3, 48, 160), (7, 2, 2, 16, 96)])
+@pytest.mark.parametrize("copy", [False, True])
 @pytest.mark.parametrize("normed", [False, True])
-def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed):
+def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed, copy):
     """The fused decode kernel against (norm,) product, then rotation and cache store."""
     from inferllm_amd.parts.position import rotary_table
     dtype, page = torch.bfloat16, 64
@@ -523,7 +572,10 @@ def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed):
     qkv_ref = R.linear(x, w, torch.float64)
     kr, vr = kc.clone().double(), vc.clone().double()
     R.rope_store(qkv_ref, table, hd, 0, pos, slot, None, kr, vr, pt, page, 0, nh, nkv, hd)
-    got = ops().qkv_rope_store(x_dev, w.to(DEV), table.to(DEV), pos.to(DEV), slot.to(DEV), kc_g := kc.to(DEV),
+    if copy and K % 32:
+        pytest.skip("a decode copy needs K % 32 == 0")
+    w_dev = _decode_copy(w.to(DEV), "qkv", nh=nh, nkv=nkv, hd=hd) if copy else w.to(DEV)
+    got = ops().qkv_rope_store(x_dev, w_dev, table.to(DEV), pos.to(DEV), slot.to(DEV), kc_g := kc.to(DEV),
                                vc_g := vc.to(DEV), pt.to(DEV), page, 0, nh, nkv, hd).cpu()
     sc = math.sqrt(K) * 0.1
     close(got[:, :nh * hd], qkv_ref[:, :nh * hd], dtype, scale=sc)

@@ -57,11 +57,14 @@ def test_whole_requests(tmp_path_factory, name, dtype):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("copies", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_last_32_tokens_one_by_one(tmp_path_factory, name, dtype):
+def test_last_32_tokens_one_by_one(tmp_path_factory, name, dtype, copies):
+    """`copies`: with and without the second copy of the matrices that decoding reads."""
     from inferllm_amd import StepEntry
-    eng, plain, config = setup(tmp_path_factory, name, dtype)
+    eng, plain, config = setup(tmp_path_factory, name, dtype, decode_copies=copies)
+    assert eng.decode_copies == (copies and dtype == "bfloat16")
     for ids in requests_for(config, [33, 100, 128], seed=5):
         want = plain(ids)
         s = eng.alloc_slot()
