@@ -182,10 +182,11 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> to
 class Weight:
     """A matrix [N, K] of a product with, optionally, a second copy laid out for the few-rows
     kernels (`tile_weight`).  Wherever the ops take a weight they take this or a plain tensor."""
-    __slots__ = ("plain", "tiled")
+    __slots__ = ("plain", "tiled", "mode")
 
-    def __init__(self, plain: torch.Tensor, tiled: Optional[torch.Tensor] = None):
-        self.plain, self.tiled = plain, tiled
+    def __init__(self, plain: torch.Tensor, tiled: Optional[torch.Tensor] = None, mode: str = "plain"):
+        # mode: which kernel's tiles the copy follows (`tile_rows`); only that kernel may read it
+        self.plain, self.tiled, self.mode = plain, tiled, mode
 
     @property
     def shape(self):
@@ -199,10 +200,11 @@ class Weight:
 DECODE_COPIES = False         # whether `decode_weight` makes the second copy (set by the engine)
 
 
-def _w(w):
-    """(plain tensor, pointer of the tiled copy or None) of a weight argument."""
+def _w(w, mode: str = "plain"):
+    """(plain tensor, pointer of the tiled copy or None) of a weight argument, for the kernel
+    whose tiles are `mode`; a copy made for another kernel's tiles is not used."""
     if isinstance(w, Weight):
-        return w.plain, (_p(w.tiled) if w.tiled is not None else None)
+        return w.plain, (_p(w.tiled) if w.tiled is not None and w.mode == mode else None)
     return w, None
 
 
@@ -250,7 +252,7 @@ def decode_weight(w: torch.Tensor, mode: str = "plain", **geometry):
     asked for decode copies and the matrix allows it, else the tensor itself."""
     if (DECODE_COPIES and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0
             and w.is_cuda and (mode != "qkv" or geometry.get("hd", 0) % 16 == 0)):
-        return Weight(w, tile_weight(w, tile_rows(w.shape[0], mode, **geometry)))
+        return Weight(w, tile_weight(w, tile_rows(w.shape[0], mode, **geometry)), mode)
     return w
 
 
@@ -474,7 +476,7 @@ def qkv_rope_store(x, w_qkv, cos_sin: torch.Tensor,
     x may be `NormedRows`."""
     xt, ssq, parts, eps = _operand(x)
     _need(qkv_rope_store_fits(x, w_qkv, hd), "qkv_rope_store: operands not taken")
-    w_qkv, wt = _w(w_qkv)
+    w_qkv, wt = _w(w_qkv, "qkv")
     _gpu(xt, w_qkv, cos_sin, row_pos, row_slot, kcache, vcache, page_table)
     _i32(row_pos, x.shape[0]); _i32(row_slot, x.shape[0]); _i32(page_table)
     M, K = x.shape
@@ -505,7 +507,7 @@ def gate_up_silu(x, w_gate_up) -> torch.Tensor:
     if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and F2 % 2 == 0
             and 1 <= M <= SKINNY_BEST_ROWS and K % 8 == 0):
         xt, ssq, parts, eps = _operand(x)
-        wp, wt = _w(w_gate_up)
+        wp, wt = _w(w_gate_up, "gate_up")
         _gpu(xt, wp)
         _need(wp.dim() == 2 and wp.shape[1] == K, "gate_up_silu: shapes")
         y = torch.empty((M, F2 // 2), dtype=x.dtype, device=xt.device)

@@ -306,7 +306,7 @@ def test_gemv_rows_f32(ydt, M, N, K):
 
 def _decode_copy(w, mode="plain", **geometry):
     o = ops()
-    return o.Weight(w, o.tile_weight(w, o.tile_rows(w.shape[0], mode, **geometry)))
+    return o.Weight(w, o.tile_weight(w, o.tile_rows(w.shape[0], mode, **geometry)), mode)
 
 
 def test_tile_rows_cover_every_row_once():
@@ -350,6 +350,11 @@ def test_products_from_the_decode_copy_equal_those_from_the_matrix(M, N, K, monk
         assert torch.equal(o.gate_up_silu(x, _decode_copy(wg, "gate_up")), o.gate_up_silu(x, wg))
     xl = rnd(17, K, dtype=torch.bfloat16, seed=7).to(DEV)     # more rows: the matrix itself is read
     assert torch.equal(o.linear(xl, wc), o.linear(xl, w))
+    # a copy that follows another kernel's tiles is never read by the plain product
+    if N % 2 == 0 and K % 64 == 0:
+        other = _decode_copy(w, "gate_up")
+        assert not torch.equal(other.tiled.view(-1)[: 16 * K], wc.tiled.view(-1)[: 16 * K]) or N <= 16
+        assert torch.equal(o.linear(x, other), o.linear(x, w))
 
 
 def test_products_of_many_rows_are_planned_once_and_stay_right():

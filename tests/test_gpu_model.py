@@ -28,7 +28,7 @@ def setup(tmp_path_factory, name, dtype, **kw):
     config = CONFIGS[name]
     key = (name, dtype)
     if key not in _cache:
-        d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=7, dtype=STORE[dtype])
+        d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=7, dtype=STORE[dtype], gain=4.0)
         _cache[key] = (d, read_weights(d))
     d, w = _cache[key]
     kw.setdefault("max_batch", 4)
@@ -55,6 +55,23 @@ def test_whole_requests(tmp_path_factory, name, dtype):
         assert err(got, plain(ids)) < BUDGET[dtype]
         eng.free_slot(s)
     eng.cache.check()
+
+
+@pytest.mark.parametrize("copies", [True, False])
+def test_short_prompts_at_head_size_128(tmp_path_factory, copies):
+    """Prompts of at most 16 tokens take the few-rows kernels in their first step too, where the
+    q|k|v product is the plain one: with head size 128 the decode copy of that matrix follows
+    other tiles (rows and their rotation partners) and must not be read by it."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "D", "bfloat16", decode_copies=copies)
+    for ids in requests_for(config, [1, 5, 16, 17], seed=9):
+        s = eng.alloc_slot()
+        got = [eng.step([StepEntry(s, ids, list(range(len(ids))))]).clone()]
+        more = random_ids(3, config["vocab_size"], 77)
+        for t in more:
+            got.append(eng.step([StepEntry(s, [t], [0])]).clone())
+        assert err(torch.cat(got), plain(ids + more)) < BUDGET["bfloat16"], len(ids)
+        eng.free_slot(s)
 
 
 @pytest.mark.parametrize("copies", [True, False])
@@ -197,7 +214,7 @@ def test_command_line_generates_like_the_plain_model(tmp_path):
     import subprocess
     import sys
     config = CONFIGS["A"]
-    d = make_model_dir(tmp_path, config, seed=7, dtype=torch.float32)
+    d = make_model_dir(tmp_path, config, seed=7, dtype=torch.float32, gain=4.0)
     w = read_weights(d)
     prompts = requests_for(config, [7, 3], seed=3)
     ids_file = tmp_path / "prompts.txt"
@@ -267,7 +284,7 @@ def test_real_layer_sizes_in_bfloat16(tmp_path_factory, nkv, ffn):
               "vocab_size": 32000, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
               "max_position_embeddings": 512, "tie_word_embeddings": False,
               "bos_token_id": 1, "eos_token_id": 2}
-    d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=11, dtype=torch.bfloat16)
+    d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=11, dtype=torch.bfloat16, gain=2.0)
     w = read_weights(d)
     eng = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=4, poison_freed=True)
     reqs = requests_for(config, [40, 23, 70], seed=3)

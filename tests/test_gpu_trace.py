@@ -54,7 +54,7 @@ def worst(got, want):
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_three_schedules_agree_with_the_plain_model(tmp_path, name, dtype):
     config = CONFIGS[name]
-    d = make_model_dir(tmp_path, config, seed=13, dtype=STORE[dtype])
+    d = make_model_dir(tmp_path, config, seed=13, dtype=STORE[dtype], gain=4.0)
     w = read_weights(d)
     lens = [40, 70, 33, 100, 36]
     reqs = [random_ids(n, config["vocab_size"], 100 + i) for i, n in enumerate(lens)]

@@ -35,7 +35,7 @@ def emulated(monkeypatch):
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_whole_prompt_equals_plain(name, tmp_path, emulated):
     config = CONFIGS[name]
-    d = make_model_dir(tmp_path, config, seed=3)
+    d = make_model_dir(tmp_path, config, seed=3, gain=4.0)
     w = read_weights(d)
     ids = random_ids(70, config["vocab_size"], 1)
     want = plain_llama.forward_logits(config, w, ids)
@@ -50,7 +50,7 @@ def test_whole_prompt_equals_plain(name, tmp_path, emulated):
 
 def test_tail_decoding_and_ragged_batches_equal_plain(tmp_path, emulated):
     config = CONFIGS["B"]
-    d = make_model_dir(tmp_path, config, seed=5)
+    d = make_model_dir(tmp_path, config, seed=5, gain=4.0)
     w = read_weights(d)
     V = config["vocab_size"]
     reqs = [random_ids(n, V, 10 + n) for n in (70, 9, 131, 66, 3)]
@@ -97,7 +97,7 @@ def test_tail_decoding_and_ragged_batches_equal_plain(tmp_path, emulated):
 
 def test_step_refuses_mixed_phases_and_bad_ids(tmp_path, emulated):
     config = CONFIGS["A"]
-    w = read_weights(make_model_dir(tmp_path, config, seed=1))
+    w = read_weights(make_model_dir(tmp_path, config, seed=1, gain=4.0))
     r = build_runner(config, w)
     a, b = r.cache.alloc_slot(), r.cache.alloc_slot()
     r.step([StepEntry(a, [1, 2, 3], [])])

@@ -35,12 +35,28 @@ TINY_D = {"architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermedia
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
-def make_model_dir(tmp_path, config: dict, seed: int, dtype=torch.float32) -> str:
-    """Write a random model folder for `config` under tmp_path; returns the folder."""
+def make_model_dir(tmp_path, config: dict, seed: int, dtype=torch.float32, gain: float = 1.0) -> str:
+    """Write a random model folder for `config` under tmp_path; returns the folder.
+
+    gain: every matrix is multiplied by it.  The library's random weights are N(0, 0.02): with
+    them queries and keys are tiny, every softmax is nearly uniform and a fault in the attention
+    path (a wrong row of a projection, a wrong key) moves the logits by a per cent or two, within
+    what bfloat16 is allowed.  With gain 4 the scores spread over several units and such a fault
+    moves the logits by their own size."""
     import inferllm_amd as I
-    d = os.path.join(str(tmp_path), f"model_{abs(hash(json.dumps(config, sort_keys=True))) % 10**8}_{seed}_{str(dtype)[6:]}")
+    from inferllm_amd.weights import open_model_files
+    from inferllm_amd.weights.safetensors_io import write_safetensors
+    d = os.path.join(str(tmp_path), f"model_{abs(hash(json.dumps(config, sort_keys=True))) % 10**8}_{seed}_{str(dtype)[6:]}_{gain}")
     if not os.path.isdir(d):
         I.write_random_model(d, I.config_from_dict(config), seed=seed, dtype=dtype)
+        if gain != 1.0:
+            tensors = []
+            for f in open_model_files(d):
+                for n in f.names():
+                    t = f.read(n)
+                    tensors.append((n, (t.float() * gain).to(t.dtype) if t.dim() == 2 else t))
+                f.close()
+            write_safetensors(os.path.join(d, "model.safetensors"), tensors, metadata={"format": "pt"})
     return d
 
 
