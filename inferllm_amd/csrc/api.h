@@ -99,6 +99,10 @@ int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y,
 int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M, int N,
                               int K, int ntb, int u, int waves, void* stream);
 
+// Tuning: tiles a block of the tiled plain and gate|up products takes (1 or 2; 0: the default,
+// two when there are at least 1024 tiles).
+void illm_set_skinny_tiles_per_block(int n);
+
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
 // product, `ssq` included.  waves_wanted: waves per block (0: the default choice).
 int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const void* Wt, void* Y, int y_dt,

@@ -122,7 +122,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
         tot += __shfl_xor(tot, 32, ILLM_WAVE);
         if (lane < 16) row_rs[lane] = 1.0f / sqrtf(tot / (float)K + res.eps);
     }
-    const int n_base = blockIdx.x * (DUAL ? 8 : 16 * NTB);
+    const int n_base = blockIdx.x * (DUAL ? 8 * NTB : 16 * NTB);
     int tile_row[NTB];           // SK_PLAIN: first W row of each of the block's tiles
 #pragma unroll
     for (int nt = 0; nt < NTB; ++nt) tile_row[nt] = n_base + nt * 16;
@@ -193,7 +193,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             int n = tile_row[nt] + (lane >> 3) + 8 * h;
-            if (MODE != SK_PLAIN) n = (h ? row_hi : row_lo) + (lane >> 3);
+            if (MODE != SK_PLAIN) n = (h ? row_hi : row_lo) + (DUAL ? 8 * nt : 0) + (lane >> 3);
             const int last = DUAL ? (h + 1) * N - 1 : N - 1;
             n = n < last ? n : last;
             wline[nt][h] = W + (size_t)n * K;
@@ -218,8 +218,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     // handles a wave's accesses in order, no barrier is needed.
     uint4* stage = (uint4*)red + (size_t)wave * (SK_REGION_FLOATS / 4);
     const int w_row = lane >> 3, w_chunk = lane & 7;
-    // TILED: this lane's 8 values of k-step 0 of the block's tile
-    const bf16_t* wtile = W + (size_t)blockIdx.x * ((K + 31) / 32) * 512 + (r * 4 + q) * 8;
+    // TILED: this lane's 8 values of k-step 0 of the block's first tile; a last block may have
+    // fewer than NTB tiles (SK_GATE_UP with NTB > 1)
+    const bf16_t* wtile = W + (size_t)blockIdx.x * NTB * ((K + 31) / 32) * 512 + (r * 4 + q) * 8;
+    bool tile_ok[NTB];
+#pragma unroll
+    for (int nt = 0; nt < NTB; ++nt) tile_ok[nt] = DUAL ? n_base + 8 * nt < N : tile_row[nt] < N || MODE != SK_PLAIN;
 
     const int ksteps = (K + 31) / 32;
     const int stride = waves * SK_U;
@@ -231,7 +235,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
             const int kw = (s0 + (u & ~1)) * 32 + w_chunk * 8;
 #pragma unroll
             for (int nt = 0; nt < NTB; ++nt) {
-                if (TILED) aa[nt][u] = s0 + u < ksteps ? ld16_stream(wtile + (size_t)(s0 + u) * 512) : make_uint4(0, 0, 0, 0);
+                if (TILED)
+                    aa[nt][u] = (s0 + u < ksteps && tile_ok[nt])
+                                    ? ld16_stream(wtile + ((size_t)nt * ksteps + s0 + u) * 512)
+                                    : make_uint4(0, 0, 0, 0);
                 else aa[nt][u] = kw < K ? ld16_stream(wline[nt][u & 1] + kw) : make_uint4(0, 0, 0, 0);
             }
             const int k = (s0 + u) * 32 + q * 8;
@@ -330,13 +337,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
         return;
     }
     if (DUAL) {
-        // NTB == 1: rows 0 .. 7 of the tile are gate rows, rows 8 .. 15 the up rows of the same
-        // outputs; a thread takes one X row's 4 outputs
-        for (int grp = threadIdx.x; grp < MT * 32; grp += blockDim.x) {
-            const int l2 = grp & 31, mt = grp >> 5;
-            const int mrow = mt * 16 + (l2 & 15), n0 = n_base + (l2 >> 4) * 4;
+        // rows 0 .. 7 of a tile are gate rows, rows 8 .. 15 the up rows of the same outputs; a
+        // thread takes one X row's 4 outputs of one tile
+        for (int grp = threadIdx.x; grp < NTB * MT * 32; grp += blockDim.x) {
+            const int l2 = grp & 31, mt = (grp >> 5) % MT, nt = (grp >> 5) / MT;
+            const int mrow = mt * 16 + (l2 & 15), n0 = n_base + 8 * nt + (l2 >> 4) * 4;
             if (mrow >= M) continue;
-            const int e = (mt * 64 + l2) * 4;
+            const int e = ((nt * MT + mt) * 64 + l2) * 4;
             f32x4_t g = *(f32x4_t*)(red + e), u = *(f32x4_t*)(red + e + 128);
             for (int w = 1; w < waves; ++w) {
                 const f32x4_t og = *(f32x4_t*)(red + (size_t)w * PER_WAVE + e);
@@ -434,7 +441,7 @@ static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M,
     constexpr int REGS = 2 * (NTB + MT) * U * 4 + NTB * 8 + NTB * MT * 4 + 40;
     constexpr int MAXW = REGS <= 128 ? 16 : (REGS <= 256 ? 8 : 4);
     waves = waves > MAXW ? MAXW : waves;
-    const int rows_per_block = DUAL ? 8 : 16 * NTB;
+    const int rows_per_block = DUAL ? 8 * NTB : 16 * NTB;
     const int blocks = (N + rows_per_block - 1) / rows_per_block;
     const size_t smem = (size_t)waves * NTB * ((!TILED && U > MT) ? U : MT) * 1024 + 64;
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, MODE, TILED>), dim3(blocks), dim3(64 * waves),
@@ -445,6 +452,10 @@ static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M,
 // Measured on MI355X at the LLaMA-2-7B shapes: 16 W rows per block and about this many waves
 // on the chip are best for M <= 16; wider row tiles only pay when X has many rows.
 static const int SK_WAVES_ON_CHIP = 2400;
+// Tiles a block of the tiled gate|up and plain products takes: 0 = by the number of tiles (two
+// from 1024 tiles on), 1 or 2 = forced (tuning).
+static int SK_TILES_PER_BLOCK = 0;
+extern "C" void illm_set_skinny_tiles_per_block(int n) { SK_TILES_PER_BLOCK = (n == 1 || n == 2) ? n : 0; }
 static const int SK_WAVES_ON_CHIP_TILED = 3072;      // from the tiled copy (no staging in LDS)
 
 static int clamp_waves(int w, int ntb, int mt, int u, int K) {
@@ -502,9 +513,18 @@ extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, const void* W
     SkResidual res = SK_NO_RESIDUAL;
     res.ssq = ssq; res.parts = parts; res.eps = eps;
     waves = clamp_waves(waves, 1, 1, 4, K);
-    if (use_tiled(Wt, M, K))
+    if (use_tiled(Wt, M, K)) {
+        // with many tiles (the head) a block takes two: X is read half as often
+        if (SK_TILES_PER_BLOCK == 2 || (SK_TILES_PER_BLOCK == 0 && blocks >= 1024)) {
+            const int blocks2 = (blocks + 1) / 2;
+            int w2 = waves_wanted > 0 ? waves_wanted : (on_chip + blocks2 / 2) / blocks2;
+            return launch_skinny<1, 2, 4, SK_PLAIN, true>(X, Wt, Y, y_dt, M, N, K,
+                                                          clamp_waves(w2 < 1 ? 1 : w2, 2, 1, 4, K),
+                                                          (hipStream_t)stream, SkRope(), res);
+        }
         return launch_skinny<1, 1, 4, SK_PLAIN, true>(X, Wt, Y, y_dt, M, N, K, waves,
                                                       (hipStream_t)stream, SkRope(), res);
+    }
     return launch_skinny<1, 1, 4>(X, W, Y, y_dt, M, N, K, waves, (hipStream_t)stream, SkRope(), res);
 }
 
@@ -549,8 +569,23 @@ extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const 
     const int on_chip = use_tiled(Wt, M, K) ? 4096 : 8192;
     int waves = waves_wanted > 0 ? waves_wanted : (on_chip + blocks / 2) / blocks;
     waves = clamp_waves(waves < 1 ? 1 : waves, 1, mt, 4, K);
-    if (use_tiled(Wt, M, K))
+    if (use_tiled(Wt, M, K)) {
+        // with many tiles a block takes two: X is read half as often (measured at F = 11008, 8 and
+        // 16 rows: 36 -> 31 us and 46 -> 33 us; one row: no change)
+        if (SK_TILES_PER_BLOCK == 2 || (SK_TILES_PER_BLOCK == 0 && blocks >= 1024)) {
+            const int blocks2 = (F + 15) / 16;
+            int w2 = waves_wanted > 0 ? waves_wanted : (1400 + blocks2 / 2) / blocks2;
+            w2 = clamp_waves(w2 < 1 ? 1 : w2, 2, mt, 4, K);
+            return launch_skinny<1, 2, 4, SK_GATE_UP, true>(X, Wt, Y, y_dt, M, F, K, w2, st, SkRope(), res);
+        }
         return launch_skinny<1, 1, 4, SK_GATE_UP, true>(X, Wt, Y, y_dt, M, F, K, waves, st, SkRope(), res);
+    }
+    if (mt == 1 && (SK_TILES_PER_BLOCK == 2 || (SK_TILES_PER_BLOCK == 0 && blocks >= 1024))) {
+        const int blocks2 = (F + 15) / 16;
+        int w2 = waves_wanted > 0 ? waves_wanted : (1400 + blocks2 / 2) / blocks2;
+        w2 = clamp_waves(w2 < 1 ? 1 : w2, 2, mt, 4, K);
+        return launch_skinny<1, 2, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, w2, st, SkRope(), res);
+    }
     switch (mt) {
         case 1: return launch_skinny<1, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st, SkRope(), res);
         case 2: return launch_skinny<2, 1, 4, SK_GATE_UP>(X, W, Y, y_dt, M, F, K, waves, st);

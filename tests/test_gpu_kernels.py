@@ -323,7 +323,8 @@ def test_tile_rows_cover_every_row_once():
     assert q[-1].tolist() == list(range(3 * 32 + 16, 4 * 32))                  # v: 16 rows in a run
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 100, 160), (16, 33, 992), (5, 320, 96), (9, 4096, 11008)])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 100, 160), (16, 33, 992), (5, 320, 96), (9, 4096, 11008),
+                                   (8, 16400, 64)])      # 1025 tiles: two a block, the last block has one
 def test_products_from_the_decode_copy_equal_those_from_the_matrix(M, N, K, monkeypatch):
     """The copy laid out for the few-rows kernels holds the same numbers in another order: with
     K cut over the same number of waves the products are the same sums in the same order, bit
@@ -346,8 +347,9 @@ def test_products_from_the_decode_copy_equal_those_from_the_matrix(M, N, K, monk
         if N % 32 == 0:
             assert torch.equal(o.linear(ra, _decode_copy(w2)), o.linear(rb, w2))
     if K % 64 == 0:                                        # gate|up: N rows as two halves
-        wg = rnd(2 * 56, K, dtype=torch.bfloat16, seed=6, std=0.2).to(DEV)
-        assert torch.equal(o.gate_up_silu(x, _decode_copy(wg, "gate_up")), o.gate_up_silu(x, wg))
+        for F in (56, 8200):                               # 8200: 1025 tiles, two a block
+            wg = rnd(2 * F, K, dtype=torch.bfloat16, seed=6, std=0.2).to(DEV)
+            assert torch.equal(o.gate_up_silu(x, _decode_copy(wg, "gate_up")), o.gate_up_silu(x, wg))
     xl = rnd(17, K, dtype=torch.bfloat16, seed=7).to(DEV)     # more rows: the matrix itself is read
     assert torch.equal(o.linear(xl, wc), o.linear(xl, w))
     # a copy that follows another kernel's tiles is never read by the plain product
