@@ -11,6 +11,12 @@ Matrix products: float32 operands always go to the library's own float32 kernel
 MFMA kernels of this library when the shape fits them (few rows: decoding), and
 to the vendor GEMM through `torch.matmul` otherwise, which is where the reference
 uses a vendor GEMM too (cublasSgemm, src/kern/gpu/kernel_gpu.cu:420-435).
+
+Three things ride on the products of few rows.  `Weight`: a matrix with a second
+copy in the kernels' own tile order (`decode_weight`).  `linear_add` / `NormedRows`:
+the residual add in the product's epilogue and the RMS norm that follows it taken
+by the next product.  `_planned_matmul`: products of many rows measured once per
+shape, whole against cut along the output columns.
 """
 from __future__ import annotations
 
