@@ -45,7 +45,7 @@ def requests_for(config, lens, seed=0):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_whole_requests(tmp_path_factory, name, dtype):
     from inferllm_amd import StepEntry
     eng, plain, config = setup(tmp_path_factory, name, dtype)
@@ -76,7 +76,7 @@ def test_short_prompts_at_head_size_128(tmp_path_factory, copies):
 
 @pytest.mark.parametrize("copies", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_last_32_tokens_one_by_one(tmp_path_factory, name, dtype, copies):
     """`copies`: with and without the second copy of the matrices that decoding reads."""
     from inferllm_amd import StepEntry
@@ -97,7 +97,7 @@ def test_last_32_tokens_one_by_one(tmp_path_factory, name, dtype, copies):
 
 @pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_unequal_batches_with_slot_reuse(tmp_path_factory, name, dtype, graphs):
     """Batches of three requests of unequal lengths, one batch after another in two
     slots' worth of spare room; shorter requests end earlier; every position's
