@@ -51,7 +51,7 @@ def worst(got, want):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_three_schedules_agree_with_the_plain_model(tmp_path, name, dtype):
     config = CONFIGS[name]
     d = make_model_dir(tmp_path, config, seed=13, dtype=STORE[dtype], gain=4.0)
