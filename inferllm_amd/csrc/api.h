@@ -17,10 +17,12 @@ int illm_embed(const int32_t* tokens, const void* table, int table_dt, float* ou
 
 // Residual add and RMS norm.  in_row = row_idx ? row_idx[r] : r;
 // v = x[in_row] (+ delta[in_row]); when delta is given and row_idx is not, v is
-// written back to x.  out[r] = v * rsqrt(mean(v^2) + eps) * w.
-int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const void* w, int w_dt,
-                     void* out, int out_dt, const int32_t* row_idx, int rows, int E, float eps,
-                     void* stream);
+// written back to x.  out[r] = v * rsqrt(mean(v^2) + eps) * w.  delta may be `planes` >= 1
+// arrays, plane_stride elements apart (the sums of a product whose K was split,
+// illm_gemm_mid_bf16), which are added in order.
+int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int planes, size_t plane_stride,
+                     const void* w, int w_dt, void* out, int out_dt, const int32_t* row_idx,
+                     int rows, int E, float eps, void* stream);
 
 // out[t, f] = silu(gate_up[t, f]) * gate_up[t, F + f].
 int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* stream);
@@ -98,6 +100,20 @@ int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y,
 // of a W row per wave iteration (u 4, 8), waves per block.
 int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M, int N,
                               int K, int ntb, int u, int waves, void* stream);
+
+// The same from the tiled copy with more row tiles (tuning; mt = ceil(M / 16) up to 4, ntb 1 or
+// 2, u 2 or 4).
+int illm_gemm_skinny_tiled_cfg(const void* X, const void* Wt, void* Y, int y_dt, int M, int N,
+                               int K, int ntb, int u, int waves, void* stream);
+
+// Y = X[M, K] . W[N, K]^T for M up to 64 (meant for 17..64) from the tiled copy Wt of W, K a
+// multiple of 32, X shared by a block's waves through LDS.  splits == 1: Y is [M, N] of y_dt;
+// splits > 1: K is cut into that many ranges and Y is float32 [splits][M][N], the planes to be
+// added by the caller (illm_add_rmsnorm takes them).  illm_gemm_mid_splits: the splits to use.
+int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M, int N, int K,
+                       int splits, void* stream);
+int illm_gemm_mid_splits(int N, int K);
+void illm_set_mid_tiles_per_wave(int n);      // tuning: 1 or 2 (0: by the number of tiles)
 
 // Tuning: tiles a block of the tiled plain and gate|up products takes (1 or 2; 0: the default,
 // two when there are at least 1024 tiles).

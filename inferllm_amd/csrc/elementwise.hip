@@ -34,8 +34,18 @@ extern "C" int illm_embed(const int32_t* tokens, const void* table, int table_dt
 // ---------------------------------------------------------------- add + rmsnorm
 // One block per row.  The sum of squares is taken in float32 in an order that
 // depends on E and the block size only, never on the row's place in the batch.
+// `delta` may be `planes` arrays of the same shape, `plane_stride` elements apart (the sums of
+// a product whose K was split): they are added in order.
+__device__ __forceinline__ float ld_planes(const void* delta, int dt, size_t i, int planes,
+                                           size_t plane_stride) {
+    float d = ld_f(delta, dt, i);
+    for (int s = 1; s < planes; ++s) d += ld_f(delta, dt, i + s * plane_stride);
+    return d;
+}
+
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ delta,
-                                   int delta_dt, const void* __restrict__ w, int w_dt,
+                                   int delta_dt, int planes, size_t plane_stride,
+                                   const void* __restrict__ w, int w_dt,
                                    void* __restrict__ out, int out_dt,
                                    const int32_t* __restrict__ row_idx, int E, float eps) {
     __shared__ float red[16];
@@ -46,7 +56,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict
     for (int i = threadIdx.x; i < E; i += blockDim.x) {
         float v = x[ib + i];
         if (delta) {
-            v += ld_f(delta, delta_dt, ib + i);
+            v += ld_planes(delta, delta_dt, ib + i, planes, plane_stride);
             if (!row_idx) x[ib + i] = v;
         }
         ss += v * v;
@@ -55,7 +65,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const void* __restrict
     const float scale = 1.0f / sqrtf(ss / (float)E + eps);
     for (int i = threadIdx.x; i < E; i += blockDim.x) {
         float v = x[ib + i];
-        if (delta && row_idx) v += ld_f(delta, delta_dt, ib + i);
+        if (delta && row_idx) v += ld_planes(delta, delta_dt, ib + i, planes, plane_stride);
         st_f(out, out_dt, ob + i, (v * scale) * ld_f(w, w_dt, i));
     }
 }
@@ -86,6 +96,7 @@ __device__ __forceinline__ void st4_f(void* p, int dt, size_t i4, float4 v) {
 template <int NV, int TH>
 __global__ void __launch_bounds__(TH)
 add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, int delta_dt,
+                       int planes, size_t plane_stride4,
                        const void* __restrict__ w, int w_dt, void* __restrict__ out, int out_dt,
                        const int32_t* __restrict__ row_idx, int E, float eps) {
     __shared__ float red[16];
@@ -109,7 +120,20 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
         for (int j = 0; j < NV; ++j) {
             const int i = threadIdx.x + TH * j;
             if (i < E4) {
-                const float4 d = ld4_f(delta, delta_dt, ib + i);
+                float4 d = ld4_f(delta, delta_dt, ib + i);
+                // the planes of a split product, four loads at a time, added in order
+                for (int s0 = 1; s0 < planes; s0 += 4) {
+                    float4 e[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        e[t] = s0 + t < planes
+                                   ? ld4_f(delta, delta_dt, ib + i + (size_t)(s0 + t) * plane_stride4)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        d.x += e[t].x; d.y += e[t].y; d.z += e[t].z; d.w += e[t].w;
+                    }
+                }
                 v[j].x += d.x; v[j].y += d.y; v[j].z += d.z; v[j].w += d.w;
                 if (!row_idx) ((float4*)x)[ib + i] = v[j];
             }
@@ -131,17 +155,20 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const void* __restrict__ delta, in
     }
 }
 
-extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const void* w,
-                                int w_dt, void* out, int out_dt, const int32_t* row_idx,
-                                int rows, int E, float eps, void* stream) {
+extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, int planes,
+                                size_t plane_stride, const void* w, int w_dt, void* out,
+                                int out_dt, const int32_t* row_idx, int rows, int E, float eps,
+                                void* stream) {
     if (rows < 0 || E <= 0 || !illm_dtype_ok(w_dt) || !illm_dtype_ok(out_dt) ||
-        (delta && !illm_dtype_ok(delta_dt)))
+        (delta && (!illm_dtype_ok(delta_dt) || planes < 1 ||
+                   (planes > 1 && E % 4 == 0 && plane_stride % 4))))
         return ILLM_ERR_ARG;
     if (rows == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
 #define VEC(NV_, TH_)                                                                         \
     hipLaunchKernelGGL((add_rmsnorm_vec_kernel<NV_, TH_>), dim3(rows), dim3(TH_), 0, st, x,   \
-                       delta, delta_dt, w, w_dt, out, out_dt, row_idx, E, eps)
+                       delta, delta_dt, planes, plane_stride / 4, w, w_dt, out, out_dt, row_idx, \
+                       E, eps)
     // few rows (decoding): wide blocks, one group of 4 floats per thread, to shorten the row's
     // critical path; many rows: narrow blocks so that more rows are in flight per CU
     if (E % 4 == 0 && rows <= 128 && E > 1024 && E <= 4096) VEC(1, 1024);
@@ -151,8 +178,8 @@ extern "C" int illm_add_rmsnorm(float* x, const void* delta, int delta_dt, const
     else if (E % 4 == 0 && E <= 4096) VEC(4, 256);
     else if (E % 4 == 0 && E <= 8192) VEC(8, 256);
     else
-        hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, delta, delta_dt, w,
-                           w_dt, out, out_dt, row_idx, E, eps);
+        hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(rows), dim3(256), 0, st, x, delta, delta_dt,
+                           planes, plane_stride, w, w_dt, out, out_dt, row_idx, E, eps);
 #undef VEC
     return illm_launch_status();
 }

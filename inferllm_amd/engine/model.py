@@ -100,9 +100,10 @@ class DecoderModel:
         pending = None
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
-            if getattr(layer, "takes_next_norm", False) and i + 1 < len(self.schedule):
+            if getattr(layer, "takes_next_norm", False):
                 # the norm that will meet this block's output, for kernels that prepare it
-                nxt = getattr(self.layers[self.schedule[i + 1].layer], "mixer_norm", None)
+                nxt = (getattr(self.layers[self.schedule[i + 1].layer], "mixer_norm", None)
+                       if i + 1 < len(self.schedule) else self.final_norm)
                 pending = layer.forward(x, pending, ctx, e.cache_line, e.writes_cache, next_norm=nxt)
             else:
                 pending = layer.forward(x, pending, ctx, e.cache_line, e.writes_cache)

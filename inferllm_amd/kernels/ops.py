@@ -105,19 +105,25 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     """RMS norm of the float32 residual rows `x` [T, E] after adding `delta` to them.
 
     Without `row_idx` the sum is written back to `x`.  With `row_idx` only those
-    rows are normed (and `x` is left as it is).
+    rows are normed (and `x` is left as it is).  `delta` may be [S, T, E]: the planes of a
+    product whose K was split (`linear_planes`), added in order.
     """
     _gpu(x, delta, weight, row_idx)
     _i32(row_idx)
     _need(x.dtype == torch.float32 and x.dim() == 2, "add_rmsnorm: x must be float32 [T, E]")
     T, E = x.shape
     _need(weight.shape == (E,), f"add_rmsnorm: weight {tuple(weight.shape)} for width {E}")
+    planes = 1
     if delta is not None:
-        _need(delta.shape == x.shape, "add_rmsnorm: delta must have x's shape")
+        if delta.dim() == 3:
+            planes = delta.shape[0]
+            _need(planes >= 1 and E % 4 == 0, "add_rmsnorm: planes need a width that is a multiple of 4")
+        _need(delta.shape[-2:] == x.shape, "add_rmsnorm: delta must have x's shape")
     rows = T if row_idx is None else row_idx.numel()
     out = torch.empty((rows, E), dtype=out_dtype, device=x.device)
     _check(_lib().illm_add_rmsnorm(
-        _p(x), _p(delta), _code(delta) if delta is not None else 0, _p(weight), _code(weight),
+        _p(x), _p(delta), _code(delta) if delta is not None else 0, planes,
+        ctypes.c_size_t(T * E), _p(weight), _code(weight),
         _p(out), _code(out), _p(row_idx), rows, E, ctypes.c_float(eps), _stream()), "add_rmsnorm")
     return out
 
@@ -346,6 +352,39 @@ def linear_add(x: torch.Tensor, w, into: torch.Tensor, norm=None,
                                        _code(weight), _p(xb), _p(ssq), PLAIN_WAVES, _stream()),
            "linear_add")
     return NormedRows(into, weight, eps, act_dtype, xb, ssq)
+
+
+MID_MIN_ROWS = 17        # rows from which `linear_planes` stands in for the vendor GEMM
+MID_MAX_ROWS = 64
+MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the norm that adds the
+                         # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
+                         # K >= 2 N (the down projection) and the same time when K = N
+
+
+def linear_planes_fits(x, w) -> bool:
+    """Whether `linear_planes` takes these operands: 17 to 64 bfloat16 rows and a matrix with a
+    decode copy in plain tile order that has few rows for its length (K >= 2 N)."""
+    return (isinstance(w, Weight) and w.tiled is not None and w.mode == "plain"
+            and isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and x.dim() == 2
+            and MID_MIN_ROWS <= x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.plain.shape[1]
+            and w.plain.shape[0] % 4 == 0 and w.plain.shape[0] <= MID_MAX_COLS
+            and w.plain.shape[1] >= 2 * w.plain.shape[0])
+
+
+def linear_planes(x: torch.Tensor, w: "Weight", splits: int = 0) -> torch.Tensor:
+    """x . w^T as float32 planes [S, M, N] whose sum over S is the product: K is cut into S
+    ranges so that a matrix with few rows fills the chip (csrc/gemm_mid.hip).  The planes go to
+    `add_rmsnorm` as `delta`, which adds them in order."""
+    _need(linear_planes_fits(x, w), "linear_planes: operands not taken")
+    x = x.contiguous()
+    _gpu(x, w.plain)
+    M, K = x.shape
+    N = w.plain.shape[0]
+    S = splits or _lib().illm_gemm_mid_splits(N, K)
+    y = torch.empty((S, M, N), dtype=torch.float32, device=x.device)
+    _check(_lib().illm_gemm_mid_bf16(_p(x), _p(w.tiled), _p(y), F32, M, N, K, S, _stream()),
+           "linear_planes")
+    return y
 
 
 def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:

@@ -18,7 +18,7 @@ import torch
 from . import ops
 
 _TIMED = ("embed", "add_rmsnorm", "silu_mul", "rope_store", "qkv_rope_store", "gate_up_silu",
-          "linear", "linear_add", "attn_prefill", "attn_decode", "argmax", "sample")
+          "linear", "linear_add", "linear_planes", "attn_prefill", "attn_decode", "argmax", "sample")
 
 
 class KernelTimes:

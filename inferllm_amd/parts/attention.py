@@ -100,4 +100,6 @@ class Attention(Mixer):
             return ops.linear_add(o, self.w_o, residual,
                                   next_norm.rms_params() if next_norm is not None else None,
                                   ctx.act_dtype)
+        if next_norm is not None and getattr(next_norm, "adds_planes", False) and ops.linear_planes_fits(o, self.w_o):
+            return ops.linear_planes(o, self.w_o)
         return ops.linear(o, self.w_o)

@@ -104,6 +104,11 @@ class FeedForward(Part):
 
 
 class Norm(Part):
+    # True: `forward` also takes `delta` as float32 planes [S, rows, width] that it adds in order
+    # (a product whose K was split, `ops.linear_planes`).  Parts hand planes only to a norm that
+    # says so.
+    adds_planes = False
+
     def rms_params(self):
         """(weight, eps) if the norm is a plain RMS norm that a product's kernel may take over
         (see `Part.adds_residual`), else None."""

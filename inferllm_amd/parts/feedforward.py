@@ -44,4 +44,6 @@ class SwiGLU(FeedForward):
             return ops.linear_add(a, self.w_down, residual,
                                   next_norm.rms_params() if next_norm is not None else None,
                                   ctx.act_dtype)
+        if next_norm is not None and getattr(next_norm, "adds_planes", False) and ops.linear_planes_fits(a, self.w_down):
+            return ops.linear_planes(a, self.w_down)
         return ops.linear(a, self.w_down)

@@ -18,6 +18,8 @@ class RMSNorm(Norm):
     (the reference fixes 1e-6 / 1e-5 at src/graph/llama_like.cpp:78 and src/core/graph.h:163).
     """
 
+    adds_planes = True
+
     def __init__(self, size: int, eps: float, tensors=None):
         super().__init__(tensors)
         self.size, self.eps = int(size), float(eps)

@@ -21,6 +21,8 @@ def embed(tokens, table):
 
 def add_rmsnorm(x, delta, weight, eps, out_dtype, row_idx=None):
     if delta is not None:
+        if delta.dim() == 3:                           # planes of a split product
+            delta = delta.to(F64).sum(0)
         s = (x.to(F64) + delta.to(F64)).to(torch.float32)
         if row_idx is None:
             x.copy_(s)

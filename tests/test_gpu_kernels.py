@@ -66,6 +66,25 @@ def test_add_rmsnorm(out_dtype, w_dtype, T, E, eps):
             assert torch.equal(xg2.cpu(), x)   # gathered rows leave x alone
 
 
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("S,T,E", [(1, 3, 80), (3, 20, 96), (8, 64, 4096), (5, 17, 6000), (2, 3, 8196), (13, 4, 1536)])
+def test_add_rmsnorm_adds_planes(out_dtype, S, T, E):
+    """delta as the planes of a product whose K was split: their sum is added, in float32."""
+    x = rnd(T, E, seed=1)
+    w = (1 + rnd(E, seed=2) * 0.1).to(torch.bfloat16)
+    planes = rnd(S, T, E, seed=3) * torch.linspace(0.5, 2.0, S)[:, None, None]
+    xr, xg = x.clone(), x.clone().to(DEV)
+    want = R.add_rmsnorm(xr, planes, w, 1e-5, out_dtype)
+    got = ops().add_rmsnorm(xg, planes.to(DEV), w.to(DEV), 1e-5, out_dtype)
+    close(got, want, out_dtype)
+    close(xg, xr, torch.float32, scale=4.0)
+    idx = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32)
+    xg2 = x.clone().to(DEV)
+    got = ops().add_rmsnorm(xg2, planes.to(DEV), w.to(DEV), 1e-5, out_dtype, idx.to(DEV))
+    close(got, R.add_rmsnorm(x.clone(), planes, w, 1e-5, out_dtype, idx), out_dtype)
+    assert torch.equal(xg2.cpu(), x)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,F", [(4, 10), (5, 130), (3, 11008), (1, 173), (70, 64), (2, 2056)])
 def test_silu_mul(dtype, T, F):
@@ -437,6 +456,65 @@ def test_linear_add(M, N, K, nw_dtype):
         torch.testing.assert_close(rows.ssq.double().sum(1).cpu(), (want ** 2).sum(1), rtol=1e-5, atol=1e-6)
     assert not ops().linear_add_fits(x.to(DEV), w.to(DEV), dev.to(torch.bfloat16))
     assert not ops().linear_add_fits(rnd(17, K, dtype=torch.bfloat16).to(DEV), w.to(DEV), torch.zeros(17, N, device=DEV))
+
+
+def _plain_copy(w):
+    o = ops()
+    return o.Weight(w, o.tile_weight(w, o.tile_rows(w.shape[0], "plain")), "plain")
+
+
+# rows 17..64 in every count of 16-row tiles; N with a last tile of 4 rows, with fewer tiles than
+# a block's waves, with tiles beyond a multiple of 4; K of one piece, of a partial last piece
+@pytest.mark.parametrize("tiles_per_wave", [0, 1, 2])
+@pytest.mark.parametrize("M,N,K,splits", [(17, 40, 96, 0), (33, 100, 224, 0), (64, 4096, 11008, 0),
+                                          (50, 84, 1184, 5), (48, 20, 64, 1), (31, 72, 352, 3),
+                                          (64, 36, 2048, 16), (20, 8192, 16384, 0)])
+def test_linear_planes(M, N, K, splits, tiles_per_wave):
+    """The product for 17 to 64 rows, K cut into ranges: the planes add up to x . w^T, and what
+    `add_rmsnorm` makes of them is the residual add and norm of the product."""
+    o = ops()
+    if N >= 8192 and tiles_per_wave:
+        return                   # the large case is there for the library's own choice of tiles
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+    wc = _plain_copy(w.to(DEV))
+    assert o.linear_planes_fits(x.to(DEV), wc)
+    o._lib().illm_set_mid_tiles_per_wave(tiles_per_wave)
+    try:
+        planes = o.linear_planes(x.to(DEV), wc, splits)
+    finally:
+        o._lib().illm_set_mid_tiles_per_wave(0)
+    assert planes.dtype == torch.float32 and planes.shape[1:] == (M, N)
+    assert splits == 0 or planes.shape[0] == splits
+    want = R.linear(x, w, torch.float64)
+    torch.testing.assert_close(planes.double().sum(0).cpu(), want, atol=2e-4 * math.sqrt(K), rtol=1e-5)
+    into = rnd(M, N, seed=3) * 10
+    nw = (1 + rnd(N, seed=4) * 0.3).to(torch.bfloat16)
+    dev = into.clone().to(DEV)
+    got = o.add_rmsnorm(dev, planes, nw.to(DEV), 1e-5, torch.bfloat16)
+    ref_x = into.clone()
+    close(got, R.add_rmsnorm(ref_x, want.float(), nw, 1e-5, torch.bfloat16), torch.bfloat16, scale=4.0)
+    torch.testing.assert_close(dev.cpu(), ref_x, atol=2e-4 * math.sqrt(K), rtol=1e-5)
+
+
+def test_linear_planes_refuses_what_it_does_not_take():
+    o = ops()
+    w = rnd(64, 256, dtype=torch.bfloat16).to(DEV)
+    x = rnd(20, 256, dtype=torch.bfloat16).to(DEV)
+    assert o.linear_planes_fits(x, _plain_copy(w))
+    assert not o.linear_planes_fits(x, w)                                  # no decode copy
+    assert not o.linear_planes_fits(x[:16], _plain_copy(w))                # the few-rows kernels' rows
+    assert not o.linear_planes_fits(rnd(65, 256, dtype=torch.bfloat16).to(DEV), _plain_copy(w))
+    assert not o.linear_planes_fits(x.float(), _plain_copy(w))
+    wide = rnd(256, 256, dtype=torch.bfloat16).to(DEV)                      # K < 2 N: the vendor GEMM's
+    assert not o.linear_planes_fits(x, _plain_copy(wide))
+    gate_up = o.Weight(w, o.tile_weight(w, o.tile_rows(64, "gate_up")), "gate_up")
+    assert not o.linear_planes_fits(x, gate_up)                            # another kernel's tile order
+    with pytest.raises(Exception):
+        o.linear_planes(x, w)
+    y = torch.empty(2, 20, 64, device=DEV)
+    assert o._lib().illm_gemm_mid_bf16(o._p(x), o._p(_plain_copy(w).tiled), o._p(y), 0, 20, 64, 250, 2, None) != 0
+    assert o._lib().illm_gemm_mid_bf16(o._p(x), o._p(_plain_copy(w).tiled), o._p(y), 0, 65, 64, 256, 2, None) != 0
+    assert o._lib().illm_gemm_mid_bf16(o._p(x), o._p(_plain_copy(w).tiled), o._p(y), 0, 20, 64, 256, 3, None) != 0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

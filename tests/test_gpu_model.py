@@ -74,6 +74,45 @@ def test_short_prompts_at_head_size_128(tmp_path_factory, copies):
         eng.free_slot(s)
 
 
+def test_steps_of_17_to_64_rows(tmp_path_factory, monkeypatch):
+    """Steps of 17 to 64 rows (a prompt of that length, or that many sequences decoding) read the
+    decode copy of the down projection with K cut into ranges, whose planes the next norm adds
+    (configuration B: 96 x 256).  24 sequences decode together after prompts of unequal lengths;
+    one prompt of 40 tokens runs alone."""
+    from inferllm_amd import StepEntry
+    from inferllm_amd.kernels import ops
+    calls = []
+    real = ops.linear_planes
+    monkeypatch.setattr(ops, "linear_planes", lambda x, w, *a: calls.append(x.shape[0]) or real(x, w, *a))
+    eng, plain, config = setup(tmp_path_factory, "B", "bfloat16", max_batch=24, decode_copies=True)
+    ids = requests_for(config, [40], seed=2)[0]
+    s = eng.alloc_slot()
+    assert err(eng.step([StepEntry(s, ids, list(range(40)))]), plain(ids)) < BUDGET["bfloat16"]
+    eng.free_slot(s)
+    assert calls and set(calls) == {40}
+    del calls[:]
+    reqs = requests_for(config, [3 + (5 * i) % 11 for i in range(24)], seed=4)
+    heads = [len(r) - 2 for r in reqs]
+    slots = [eng.alloc_slot() for _ in reqs]
+    got = [[] for _ in reqs]
+    out = eng.step([StepEntry(s, r[:h], list(range(h))) for s, r, h in zip(slots, reqs, heads)])
+    at = 0
+    for i, h in enumerate(heads):
+        got[i].append(out[at:at + h].clone())
+        at += h
+    assert not calls                                     # more than 64 rows: the vendor GEMM
+    for t in range(2):
+        out = eng.step([StepEntry(s, [r[h + t]], [0]) for s, r, h in zip(slots, reqs, heads)])
+        for i in range(len(reqs)):
+            got[i].append(out[i:i + 1].clone())
+    assert calls and set(calls) <= set(range(24, 65))    # 24 rows, or the bucket they are padded to
+    for i, r in enumerate(reqs):
+        assert err(torch.cat(got[i]), plain(r)) < BUDGET["bfloat16"], i
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("copies", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C", "D"])
