@@ -79,7 +79,7 @@ class KVGroup:
             self.ring = 0
         self.pages_per_seq = self.ring if self.ring else seq_pages
         self.n_pages = min(pages_full, n_slots * self.pages_per_seq)
-        self.pool = FreeList(self.n_pages, "page")
+        self.pool = FreeList(self.n_pages, "page", scatter=True)
         self.spare_page = self.n_pages
         shape = (len(self.lines), self.n_pages + 1, spec.num_kv_heads, page_size, spec.head_dim)
         self.k = torch.zeros(shape, dtype=dtype, device=device)

@@ -7,6 +7,7 @@ cursor's role is played here by a length per slot.
 """
 from __future__ import annotations
 
+import random
 from typing import List
 
 
@@ -19,14 +20,23 @@ class CacheFull(CacheError):
 
 
 class FreeList:
-    """Integers 0..n-1, handed out lowest-last-freed first and taken back exactly once."""
+    """Integers 0..n-1, handed out last-freed first and taken back exactly once.
 
-    def __init__(self, n: int, what: str):
+    At the start they come in rising order, or with `scatter` in a fixed shuffled order.  Pages
+    are scattered: sequences that start together get equally many pages one after the other, and
+    when that number is a power of two their keys lie at power-of-two distances in memory, which
+    the memory channels serve unevenly (measured on MI355X, decode attention of 8 sequences over
+    pages in rising order against shuffled ones: 19.5 against 16.9 us at 512 keys, 107 against
+    91 us at 4096)."""
+
+    def __init__(self, n: int, what: str, scatter: bool = False):
         if n < 0:
             raise CacheError(f"negative number of {what}s")
         self.n = n
         self.what = what
         self._free: List[int] = list(range(n - 1, -1, -1))  # pop() gives 0 first
+        if scatter:
+            random.Random(n).shuffle(self._free)
         self._held = set()
 
     def alloc(self) -> int:
