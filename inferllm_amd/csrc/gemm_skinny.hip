@@ -488,25 +488,6 @@ extern "C" int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, 
     return ILLM_ERR_ARG;
 }
 
-// Tuning entry for the tiled copy: mt = ceil(M / 16) in 1..4, ntb in {1, 2}, u in {2, 4}.
-extern "C" int illm_gemm_skinny_tiled_cfg(const void* X, const void* Wt, void* Y, int y_dt, int M,
-                                           int N, int K, int ntb, int u, int waves, void* stream) {
-    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 32) || !illm_dtype_ok(y_dt))
-        return ILLM_ERR_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    const int mt = (M + 15) / 16;
-    waves = clamp_waves(waves, ntb, mt, mt, K);
-#define GO(MT_, NTB_, U_)                                                                     \
-    if (mt == MT_ && ntb == NTB_ && u == U_)                                                  \
-        return launch_skinny<MT_, NTB_, U_, SK_PLAIN, true>(X, Wt, Y, y_dt, M, N, K, waves, st)
-    GO(1, 1, 4); GO(1, 2, 4);
-    GO(2, 1, 4); GO(2, 2, 4); GO(2, 1, 2); GO(2, 2, 2);
-    GO(3, 1, 4); GO(3, 2, 4); GO(3, 1, 2); GO(3, 2, 2);
-    GO(4, 1, 4); GO(4, 2, 4); GO(4, 1, 2); GO(4, 2, 2);
-#undef GO
-    return ILLM_ERR_ARG;
-}
-
 static bool scale_args_ok(const float* ssq, int parts, int M) {
     return !ssq || (parts > 0 && M <= 16);
 }
