@@ -252,6 +252,37 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
     if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
 }
 
+// Walks of a row by one block wait for each load in turn unless several are asked for at once:
+// these bring eight values at a time, all loads issued before the first is used.
+template <typename F>
+__device__ __forceinline__ void each_strided8(const float* a, int n, int tid, F f) {
+    for (int base = tid; base < n; base += SB * 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + u * SB;
+            v[u] = i < n ? a[i] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + u * SB;
+            if (i < n) f(i, v[u]);
+        }
+    }
+}
+
+template <typename F>
+__device__ __forceinline__ void each_in_order8(const float* a, int lo, int hi, F f) {
+    for (int base = lo; base < hi; base += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = base + u < hi ? a[base + u] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (base + u < hi) f(base + u, v[u]);
+    }
+}
+
 // ---------------------------------------------------------------- sampler, small top_k
 // The same choice for 0 < top_k <= SB (the reference's default is 40) in a few passes over the
 // row instead of two bisections of 32 passes each: the top_k-th largest key by radix selection
@@ -279,7 +310,7 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
 
     // 1. scaled scores; then the penalty, once for every id of the window
     const float inv_temp = 1.0f / temp;
-    for (int i = tid; i < V; i += SB) s[i] = row[i] * inv_temp;
+    each_strided8(row, V, tid, [&](int i, float v) { s[i] = v * inv_temp; });
     __syncthreads();
     if (tid < nl) {
         const int id = last[tid];
@@ -301,12 +332,11 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
         const uint32_t hi_mask = pass ? (0xffffffffu << (shift + 8)) : 0u;
         for (int i = tid; i < NW * 256; i += SB) (&hist[0][0])[i] = 0;
         __syncthreads();
-        for (int i = tid; i < V; i += SB) {
-            const float v = s[i];
+        each_strided8(s, V, tid, [&](int, float v) {
             if (pass == 0) mx = fmaxf(mx, v);
             const uint32_t key = order_key(v);
             if ((key & hi_mask) == prefix) atomicAdd(&hist[wave][(key >> shift) & 255u], 1);
-        }
+        });
         __syncthreads();
         if (tid < 256) {
             int t = 0;
@@ -314,10 +344,25 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
             hist[0][tid] = t;
         }
         __syncthreads();
+        // how many keys have a larger digit: a suffix sum over the 256 digits, within each of
+        // the first four waves by shuffles, across them through LDS
+        int cnt = 0, suffix = 0;
         if (tid < 256) {
-            int above = 0;
-            for (int d = tid + 1; d < 256; ++d) above += hist[0][d];
-            if (above < krem && above + hist[0][tid] >= krem) { sh_d = tid; sh_above = above; }
+            cnt = hist[0][tid];
+            suffix = cnt;
+            const int ln = tid & (ILLM_WAVE - 1);
+#pragma unroll
+            for (int o = 1; o < ILLM_WAVE; o <<= 1) {
+                const int t = __shfl_down(suffix, o, ILLM_WAVE);
+                if (ln + o < ILLM_WAVE) suffix += t;
+            }
+            if (ln == 0) red_i[wave] = suffix;
+        }
+        __syncthreads();
+        if (tid < 256) {
+            int above = suffix - cnt;
+            for (int w = wave + 1; w < 4; ++w) above += red_i[w];
+            if (above < krem && above + cnt >= krem) { sh_d = tid; sh_above = above; }
         }
         __syncthreads();
         prefix |= (uint32_t)sh_d << shift;
@@ -331,11 +376,11 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
     const int chunk = (V + SB - 1) / SB;
     const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
     int n_eq = 0, n_gt = 0;
-    for (int i = lo; i < hi; ++i) {
-        const uint32_t key = order_key(s[i]);
+    each_in_order8(s, lo, hi, [&](int, float v) {
+        const uint32_t key = order_key(v);
         n_gt += key > prefix ? 1 : 0;
         n_eq += key == prefix ? 1 : 0;
-    }
+    });
     int total_i;
     const int eq_before = block_exclusive_scan<int>(n_eq, red_i, &total_i);
     const int eq_take = max(0, min(n_eq, krem - eq_before));
@@ -343,13 +388,12 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
     const int n_kept = total_i;                        // == top_k
     {
         int at = at0, eq_left = eq_take;
-        for (int i = lo; i < hi; ++i) {
-            const float v = s[i];
+        each_in_order8(s, lo, hi, [&](int i, float v) {
             const uint32_t key = order_key(v);
             bool take = key > prefix;
             if (key == prefix && eq_left > 0) { take = true; --eq_left; }
             if (take && at < SB) { cand_id[at] = i; cand_s[at] = v; ++at; }
-        }
+        });
     }
     __syncthreads();
 

@@ -3,6 +3,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -33,10 +34,11 @@ class Sampler:
             self._stage = torch.empty(max(words, 1024), dtype=torch.int32,
                                       pin_memory=torch.device(self.device).type == "cuda")
         host = self._stage[:words]
-        host[:2 * B].view(torch.int64).copy_(torch.tensor([_as_i64(int(s)) for s in seeds], dtype=torch.int64))
-        host[2 * B:3 * B] = torch.tensor([int(c) for c in counters], dtype=torch.int32)
+        flat = host.numpy()                              # shares the pinned memory
+        flat[:2 * B].view(np.int64)[:] = [_as_i64(int(s)) for s in seeds]
+        flat[2 * B:3 * B] = counters
         if n:
-            host[3 * B:] = torch.tensor(windows, dtype=torch.int32).view(-1)
+            flat[3 * B:].reshape(B, n)[:] = windows
         dev = host.to(self.device, non_blocking=True)
         return (dev[:2 * B].view(torch.int64), dev[2 * B:3 * B],
                 dev[3 * B:].view(B, n) if n else None)
@@ -50,7 +52,7 @@ class Sampler:
         rows = None
         if p.repeat_penalty != 1.0 and p.repeat_last_n > 0 and histories is not None:
             n = p.repeat_last_n
-            rows = [([-1] * n + [int(t) for t in h])[-n:] for h in histories]
+            rows = [[-1] * (n - min(n, len(h))) + list(h[-n:]) for h in histories]
         seeds_t, counters_t, last = self._upload(seeds, counters, rows)
         return ops.sample(logits.contiguous(), p.temperature, p.top_k, p.top_p, p.repeat_penalty,
                           last, seeds_t, counters_t).tolist()
