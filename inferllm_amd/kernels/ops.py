@@ -12,11 +12,13 @@ MFMA kernels of this library when the shape fits them (few rows: decoding), and
 to the vendor GEMM through `torch.matmul` otherwise, which is where the reference
 uses a vendor GEMM too (cublasSgemm, src/kern/gpu/kernel_gpu.cu:420-435).
 
-Three things ride on the products of few rows.  `Weight`: a matrix with a second
-copy in the kernels' own tile order (`decode_weight`).  `linear_add` / `NormedRows`:
-the residual add in the product's epilogue and the RMS norm that follows it taken
-by the next product.  `_planned_matmul`: products of many rows measured once per
-shape, whole against cut along the output columns.
+Four things ride on the products.  `Weight`: a matrix with a second copy in the
+kernels' own tile order (`decode_weight`).  `linear_add` / `NormedRows`: the
+residual add in the product's epilogue and the RMS norm that follows it taken by
+the next product (up to 16 rows).  `linear_planes`: the product of 17 to 64 rows
+with a long thin matrix, K cut into ranges whose float32 planes `add_rmsnorm` adds.
+`_planned_matmul`: products of many rows measured once per shape, whole against
+cut along the output columns.
 """
 from __future__ import annotations
 
