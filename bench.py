@@ -5,8 +5,8 @@
 
 Default: the LLaMA-2-7B layer sizes (32 layers, hidden 4096, 32/32 heads of 128,
 feed-forward 11008, vocabulary 32000) with seeded random bfloat16 weights, a batch
-of 8 sequences with 512-token prompts, cache context 4096.  A step is one decode
-step of the whole batch: step function, greedy choice on the device, the tokens
+of 8 sequences with 512-token prompts that decode 256 tokens (8 more to warm up),
+cache context 4096.  A step is one decode step of the whole batch: step function, greedy choice on the device, the tokens
 back on the host.  One JSON line is printed: decoded tokens per second, the
 prefill of 2,048 tokens, the decode step against the HBM roofline, and decoding
 at batch 1 and 64.  Peaks are the published ones of MI355X (HBM 8 TB/s, dense
@@ -61,7 +61,7 @@ def prefill_flops(cfg, layers, T, out_rows=1):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
@@ -173,8 +173,8 @@ def main() -> int:
     }
     if not args.no_points:
         out["prefill"] = prefill_run()
-        b1, _, _ = decode_run(1, min(args.steps, 64), 4)
-        b64, _, _ = decode_run(64, min(args.steps, 32), 4)
+        b1, _, _ = decode_run(1, min(args.steps, 256), 4)
+        b64, _, _ = decode_run(64, min(args.steps, 256), 4)
         out["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
     print(json.dumps(out), flush=True)
     return 0
