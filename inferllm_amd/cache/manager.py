@@ -162,14 +162,15 @@ class CacheManager:
             line: torch.zeros((max_slots + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
             for line, s in state_lines.items()}
         self.len_host = torch.zeros(max_slots + 1, dtype=torch.int32)
-        self.len_host[self.spare_slot] = 1      # padding rows attend to one (spare) key, not to none
+        self._len = self.len_host.numpy()       # the same memory; element access costs far less
+        self._len[self.spare_slot] = 1          # padding rows attend to one (spare) key, not to none
         self.slot_len = self.len_host.to(device)
         self._len_dirty = False
 
     # ------------------------------------------------------------ slots
     def alloc_slot(self) -> int:
         slot = self.slots.alloc()
-        self.len_host[slot] = 0
+        self._len[slot] = 0
         self._len_dirty = True
         for t in self.states.values():
             t[slot].zero_()
@@ -179,18 +180,18 @@ class CacheManager:
         self.slots.free(slot)           # raises if not held
         for g in self.groups:
             g.release(slot, self.poison_freed)
-        self.len_host[slot] = 0
+        self._len[slot] = 0
         self._len_dirty = True
 
     def length(self, slot: int) -> int:
-        return int(self.len_host[slot])
+        return int(self._len[slot])
 
     # ------------------------------------------------------------ steps
     def extend(self, slot: int, start_pos: int, n_tokens: int) -> None:
         """Make room for `n_tokens` more tokens of `slot`, which must now hold `start_pos`."""
         if slot not in self.slots._held:
             raise CacheError(f"slot {slot} is not held")
-        have = int(self.len_host[slot])
+        have = int(self._len[slot])
         if start_pos != have:
             raise CacheError(f"slot {slot} holds {have} tokens; a step starting at {start_pos} "
                              "does not follow")
@@ -199,7 +200,7 @@ class CacheManager:
             raise CacheFull(f"sequence would reach {new_len} tokens; the limit is {self.max_seq_len}")
         for g in self.groups:
             g.reserve(slot, new_len)
-        self.len_host[slot] = new_len
+        self._len[slot] = new_len
         self._len_dirty = True
 
     def upload(self, lengths: bool = True) -> None:
@@ -224,7 +225,7 @@ class CacheManager:
 
     def tokens_held(self) -> int:
         """Tokens held now, each sequence rounded up to whole pages."""
-        return sum(round_up(int(self.len_host[s]), self.page_size) for s in self.slots.held())
+        return sum(round_up(int(self._len[s]), self.page_size) for s in self.slots.held())
 
     def check(self) -> None:
         self.slots.check()
