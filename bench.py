@@ -80,6 +80,7 @@ def main() -> int:
     import torch
     from inferllm_amd import Engine, StepEntry
     from inferllm_amd.kernels import ops
+    from inferllm_amd.sampling import Sampler, SamplingParams
 
     shape_name, shape_cfg = SHAPES[args.shape]
     cfg = dict(shape_cfg)
@@ -112,10 +113,18 @@ def main() -> int:
             for j, t in zip(part, ops.argmax(logits.contiguous()).tolist()):
                 toks[j] = t
 
+        # as the generation loop runs greedy requests: a step starts from the tokens the last
+        # one chose on the device, and the host reads every step's tokens while the next runs
+        sampler = Sampler(SamplingParams(), eng.device)             # greedy
+        draw = sampler.draw(eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)]),
+                            [0] * batch, [0] * batch)
+
         def one():
-            nonlocal toks
-            logits = eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)])
-            toks = ops.argmax(logits).tolist()
+            nonlocal draw
+            logits = eng.step([StepEntry(s, [0], [0]) for s in slots], device_tokens=draw.device)
+            following = sampler.draw(logits, [0] * batch, [0] * batch)
+            draw.tokens()
+            draw = following
 
         for _ in range(warmup):
             one()
@@ -125,7 +134,7 @@ def main() -> int:
             one()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        mean_ctx = args.prompt + warmup + (steps + 1) / 2.0
+        mean_ctx = args.prompt + 1 + warmup + (steps + 1) / 2.0
         for s in slots:
             eng.free_slot(s)
         return batch * steps / dt, dt / steps * 1e3, mean_ctx

@@ -115,9 +115,10 @@ class Engine:
     def free_slot(self, slot: int) -> None:
         self.cache.free_slot(slot)
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry],
+             device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """See `StepRunner.step`.  The returned tensor is valid until the next step."""
-        return self.runner.step(entries)
+        return self.runner.step(entries, device_tokens)
 
     # ------------------------------------------------------------ generation
     def generate(self, prompts: Sequence[Sequence[int]], temperature: float = 0.0,
@@ -144,7 +145,8 @@ class Engine:
         loop = GenerationLoop(self.step, sampler, self.alloc_slot, self.free_slot,
                               max_batch=self.max_batch, max_tokens=self.cache.max_tokens,
                               max_seq_len=self.max_seq_len, page_size=self.cache.page_size,
-                              sync=lambda: torch.cuda.synchronize(self.device), on_token=on_token)
+                              sync=lambda: torch.cuda.synchronize(self.device), on_token=on_token,
+                              draw=sampler.draw)
         out = loop.run(prompts, params, max_new_tokens, stops, include_stop)
         self.last_stats = loop.stats
         return out

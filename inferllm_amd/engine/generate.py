@@ -7,7 +7,14 @@ sequence ends at a stop token, at its `max_new_tokens`, or when it reaches the
 longest length the cache allows; it then leaves the batch (its slot is given
 back) while the others go on.  No request joins a batch that has started.
 
-The loop only decides; computing is behind three callables, so its decisions can
+When a draw does not depend on the tokens before it (greedy, or sampling without a repeat
+penalty) and the sampler can hand its tokens on the device (`draw`), the loop runs one step
+ahead: the next step starts from the tokens on the device while the host still waits for
+their copy, so the GPU does not idle while the host decides.  Ends by count (`max_new_tokens`,
+the context limit) are known beforehand; a sequence that drew a stop token has one more step
+on its way, whose result is dropped.
+
+The loop only decides; computing is behind a few callables, so its decisions can
 be tested without a GPU.  The reference's loop is `application/chat.cpp:221-275`
 over `ModelImp::decode_iter` (src/core/model_imp.cpp:55-79): one sequence, ended by
 token 2 or a full context, `n_predict` declared but unused (chat.cpp:23).
@@ -52,17 +59,26 @@ class _Live:
     seed: int
     out: List[int] = field(default_factory=list)
     history: List[int] = field(default_factory=list)
+    drawn: int = 0             # tokens drawn and read (the pipelined loop counts with it)
+    dead: bool = False
 
 
 class GenerationLoop:
     """`step(entries) -> logits`, `sample(logits, seeds, counters, histories) -> ids`,
-    `alloc_slot() -> slot`, `free_slot(slot)`; limits of the cache as numbers."""
+    `alloc_slot() -> slot`, `free_slot(slot)`; limits of the cache as numbers.
+
+    `draw(logits, seeds, counters, histories)` (optional): like `sample`, but returns an object
+    with `.device` (the tokens where the step function can take them from: `step(entries,
+    device_tokens=...)`), `.pick(rows)` (those of some rows) and `.tokens()` (the host list,
+    waiting if need be).  With it the loop runs one step ahead where the sampling allows."""
 
     def __init__(self, step: Callable, sample: Callable, alloc_slot: Callable[[], int],
                  free_slot: Callable[[int], None], max_batch: int, max_tokens: int,
                  max_seq_len: int, page_size: int = 64, sync: Optional[Callable[[], None]] = None,
-                 on_token: Optional[Callable[[int, int], None]] = None):
+                 on_token: Optional[Callable[[int, int], None]] = None,
+                 draw: Optional[Callable] = None):
         self.step, self.sample = step, sample
+        self.draw = draw
         self.alloc_slot, self.free_slot = alloc_slot, free_slot
         self.max_batch, self.max_tokens, self.max_seq_len = max_batch, max_tokens, max_seq_len
         self.page_size = page_size
@@ -125,8 +141,78 @@ class GenerationLoop:
         while waiting:
             batch = self.next_batch(waiting, lens, max_new_tokens)
             waiting = waiting[len(batch):]
-            self._run_batch(batch, prompts, params, max_new_tokens, stop_ids, include_stop, results)
+            ahead = self.draw is not None and (params.greedy or params.repeat_penalty == 1.0
+                                               or params.repeat_last_n <= 0)
+            run = self._run_batch_ahead if ahead else self._run_batch
+            run(batch, prompts, params, max_new_tokens, stop_ids, include_stop, results)
         return results
+
+    def _run_batch_ahead(self, batch, prompts, params, max_new_tokens, stop_ids, include_stop,
+                         results):
+        """The batch with every decode step started before the tokens of the step before it
+        have been read."""
+        everyone: List[_Live] = []
+        try:
+            for i in batch:
+                everyone.append(_Live(index=i, slot=self.alloc_slot(), prompt_len=len(prompts[i]),
+                                      seed=request_seed(params.seed, i)))
+            self.stats.batches += 1
+            self.sync()
+            t0 = time.perf_counter()
+            logits = self.step([StepEntry(s.slot, prompts[s.index], [s.prompt_len - 1])
+                                for s in everyone])
+            pending = self.draw(logits, [s.seed for s in everyone], [0] * len(everyone), None)
+            self.sync()
+            self.stats.prefill_seconds += time.perf_counter() - t0
+            self.stats.prompt_tokens += sum(s.prompt_len for s in everyone)
+            t0 = time.perf_counter()
+            rows = everyone                  # the sequences `pending` has a token for, in order
+            while True:
+                # who goes on after the pending token unless it is a stop token: known by count
+                cont: List[_Live] = []
+                places: List[int] = []
+                for i, s in enumerate(rows):
+                    if s.dead:
+                        continue
+                    if self.ended(-1, s.drawn + 1, s.prompt_len + s.drawn + 1, (), max_new_tokens,
+                                  self.max_seq_len) is None:
+                        cont.append(s)
+                        places.append(i)
+                following = None
+                if cont:
+                    tokens = pending.device if len(places) == len(rows) else pending.pick(places)
+                    logits = self.step([StepEntry(s.slot, [0], [0]) for s in cont],
+                                       device_tokens=tokens)
+                    following = self.draw(logits, [s.seed for s in cont],
+                                          [s.drawn + 1 for s in cont], None)
+                    self.stats.decode_steps += 1
+                for s, tok in zip(rows, pending.tokens()):
+                    if s.dead:
+                        continue             # it drew a stop token a step ago: this one is void
+                    tok = int(tok)
+                    s.drawn += 1
+                    self.stats.generated_tokens += 1
+                    why = self.ended(tok, s.drawn, s.prompt_len + s.drawn, stop_ids,
+                                     max_new_tokens, self.max_seq_len)
+                    if why != "stop" or include_stop:
+                        s.out.append(tok)
+                        if self.on_token is not None:
+                            self.on_token(s.index, tok)
+                    if why is not None:
+                        results[s.index] = s.out
+                        self.free_slot(s.slot)     # after the step that still used it was started
+                        s.slot = -1
+                        s.dead = True
+                if following is None:
+                    break
+                rows, pending = cont, following
+            self.sync()
+            self.stats.decode_seconds += time.perf_counter() - t0
+        finally:
+            for s in everyone:
+                if s.slot >= 0:
+                    self.free_slot(s.slot)
+                    s.slot = -1
 
     def _run_batch(self, batch, prompts, params, max_new_tokens, stop_ids, include_stop, results):
         live: List[_Live] = []

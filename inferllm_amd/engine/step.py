@@ -111,17 +111,29 @@ class StepRunner:
 
     # ------------------------------------------------------------ the step
     @torch.no_grad()
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry],
+             device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one step; float32 logits [wanted, vocab] in the order of the entries
-        and of their `want`, or None when nothing is wanted."""
+        and of their `want`, or None when nothing is wanted.
+
+        `device_tokens` (a step of single tokens only): int32 [len(entries)] on the device, the
+        token of every entry in order, in place of the entries' own (which are placeholders
+        then).  It lets a caller start the next step from tokens that were chosen on the device
+        before it has read them back."""
         prefill = self._phase(entries)
+        if device_tokens is not None:
+            if prefill:
+                raise StepError("tokens from the device are taken by steps of single tokens only")
+            if (device_tokens.dtype != torch.int32 or device_tokens.device != self.device
+                    or device_tokens.shape != (len(entries),)):
+                raise StepError(f"device_tokens must be int32 [{len(entries)}] on {self.device}")
         starts = [self.cache.length(e.slot) for e in entries]
         for e, s in zip(entries, starts):
             self.cache.extend(e.slot, s, len(e.tokens))
         self.cache.upload(lengths=prefill)
         if prefill:
             return self._prefill(entries)
-        return self._decode(entries, starts)
+        return self._decode(entries, starts, device_tokens)
 
     def _prefill(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         tokens: List[int] = []
@@ -152,7 +164,8 @@ class StepRunner:
             cache=self.cache)
         return self.model.forward(ctx, parts[6] if want else None)
 
-    def _decode(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> Optional[torch.Tensor]:
+    def _decode(self, entries: Sequence[StepEntry], starts: Sequence[int],
+                device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         B = len(entries)
         size = _bucket(B) if self.use_graphs else B
         pad = size - B
@@ -164,6 +177,8 @@ class StepRunner:
         wanted = [i for i, e in enumerate(entries) if len(e.want)]
         if not self.use_graphs:
             meta = torch.tensor(host, dtype=torch.int32).to(self.device)
+            if device_tokens is not None:
+                meta[:B].copy_(device_tokens)
             ctx = StepContext(
                 device=self.device, act_dtype=self.act_dtype, prefill=False, n_rows=B, n_seqs=B,
                 tokens=meta[:B], row_pos=meta[B:2 * B], row_slot=meta[2 * B:3 * B],
@@ -180,6 +195,8 @@ class StepRunner:
         g.stage_np[:] = host
         g.meta.copy_(g.stage, non_blocking=True)
         g.copied.record()
+        if device_tokens is not None:
+            g.meta[:B].copy_(device_tokens)
         g.in_flight = True
         if g.graph is None:
             self._capture(g)

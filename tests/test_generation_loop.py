@@ -25,11 +25,13 @@ class FakeModel:
         del self.seq[s]
         self.free.append(s)
 
-    def step(self, entries):
+    def step(self, entries, device_tokens=None):
         first = [len(self.seq[e.slot]) == 0 for e in entries]
         assert all(first) or (not any(first) and all(len(e.tokens) == 1 for e in entries))
-        for e in entries:
-            self.seq[e.slot].extend(e.tokens)
+        if device_tokens is not None:
+            assert not any(first) and len(device_tokens) == len(entries)
+        for i, e in enumerate(entries):
+            self.seq[e.slot].extend(e.tokens if device_tokens is None else [device_tokens[i]])
         self.steps.append([(e.slot, len(e.tokens)) for e in entries])
         self.max_live = max(self.max_live, len(self.seq))
         return [sum(self.seq[e.slot]) % 50 for e in entries]
@@ -37,6 +39,23 @@ class FakeModel:
     @staticmethod
     def sample(logits, seeds, counters, histories):
         return list(logits)
+
+    @staticmethod
+    def draw(logits, seeds, counters, histories):
+        return FakeDraw(list(logits))
+
+
+class FakeDraw:
+    """What a sampler's `draw` returns: the tokens "on the device", some of them, and on the host."""
+
+    def __init__(self, tokens):
+        self.device = tokens
+
+    def pick(self, rows):
+        return [self.device[i] for i in rows]
+
+    def tokens(self):
+        return list(self.device)
 
 
 def expected(prompt, n, stops=(), include_stop=False, limit=10**9):
@@ -54,17 +73,23 @@ def expected(prompt, n, stops=(), include_stop=False, limit=10**9):
     return out
 
 
-def loop_for(model, max_batch=3, max_tokens=64 * 12, max_seq_len=256):
+def loop_for(model, max_batch=3, max_tokens=64 * 12, max_seq_len=256, ahead=False):
+    """ahead: with a `draw`, so that the loop starts every step before it has read the last
+    step's tokens."""
     return GenerationLoop(model.step, model.sample, model.alloc, model.release, max_batch,
-                          max_tokens, max_seq_len)
+                          max_tokens, max_seq_len, draw=model.draw if ahead else None)
+
+
+AHEAD = pytest.mark.parametrize("ahead", [False, True])
 
 
 PROMPTS = [[1, 2, 3], [7], [4, 4, 4, 4, 9], [10, 11], [3, 3], [8, 1, 1, 1, 1, 1, 2], [5]]
 
 
-def test_every_request_gets_its_own_continuation_in_batches_of_three():
+@AHEAD
+def test_every_request_gets_its_own_continuation_in_batches_of_three(ahead):
     m = FakeModel(3)
-    loop = loop_for(m)
+    loop = loop_for(m, ahead=ahead)
     out = loop.run(PROMPTS, SamplingParams(), 6)
     assert out == [expected(p, 6) for p in PROMPTS]
     assert m.max_live <= 3 and not m.seq                    # slots all given back
@@ -74,21 +99,30 @@ def test_every_request_gets_its_own_continuation_in_batches_of_three():
     assert all(n == 1 for s in m.steps[1:6] for _, n in s)
 
 
-def test_stop_tokens_end_a_sequence_early_and_the_rest_goes_on():
+@AHEAD
+def test_stop_tokens_end_a_sequence_early_and_the_rest_goes_on(ahead):
     stops = {expected(PROMPTS[0], 6)[2], expected(PROMPTS[2], 6)[0]}
     m = FakeModel(3)
-    out = loop_for(m).run(PROMPTS[:3], SamplingParams(), 6, stops)
+    out = loop_for(m, ahead=ahead).run(PROMPTS[:3], SamplingParams(), 6, stops)
     assert out == [expected(p, 6, stops) for p in PROMPTS[:3]]
     assert out[2] == [] and len(out[0]) == 2 and len(out[1]) > 2
     sizes = [len(s) for s in m.steps]
-    assert sizes[0] == 3 and sizes[1] == 2 and sizes[-1] == 1   # the batch shrinks
-    out = loop_for(FakeModel(3)).run(PROMPTS[:3], SamplingParams(), 6, stops, include_stop=True)
+    if ahead:       # a stop token is seen one step late: that sequence has one void step more
+        assert sizes[:3] == [3, 3, 2] and sizes[-1] == 1
+        assert len(m.steps) <= 6                         # ends by max_new_tokens are known beforehand: no void step
+    else:
+        assert sizes[0] == 3 and sizes[1] == 2 and sizes[-1] == 1   # the batch shrinks
+    assert not m.seq
+    out = loop_for(FakeModel(3), ahead=ahead).run(PROMPTS[:3], SamplingParams(), 6, stops, include_stop=True)
     assert out == [expected(p, 6, stops, True) for p in PROMPTS[:3]]
 
 
-def test_context_limit_ends_a_sequence():
+@AHEAD
+def test_context_limit_ends_a_sequence(ahead):
     m = FakeModel(2)
-    out = loop_for(m, max_batch=2, max_seq_len=6).run([[1, 2, 3], [9, 9, 9, 9, 9, 9]], SamplingParams(), 10)
+    out = loop_for(m, max_batch=2, max_seq_len=6, ahead=ahead).run([[1, 2, 3], [9, 9, 9, 9, 9, 9]], SamplingParams(), 10)
+    assert max(len(v) for v in m.seq.values()) <= 6 if m.seq else True
+    assert all(n <= 1 for st in m.steps[1:] for _, n in st)
     assert out == [expected([1, 2, 3], 10, limit=6), expected([9] * 6, 10, limit=6)]
     assert len(out[0]) == 4 and len(out[1]) == 1
     with pytest.raises(ValueError, match="longer than"):
@@ -106,11 +140,12 @@ def test_batches_respect_cache_room():
     big = loop_for(FakeModel(8), max_batch=8, max_tokens=64 * 4, max_seq_len=2048)
     with pytest.raises(ValueError, match="more cache room"):
         big.next_batch([0], [1000], 6)
-    m = FakeModel(8)
-    loop = loop_for(m, max_batch=8, max_tokens=64 * 4)
-    prompts = [[1] * n for n in lens]
-    assert loop.run(prompts, SamplingParams(), 6) == [expected(p, 6) for p in prompts]
-    assert loop.stats.batches == 2
+    for ahead in (False, True):
+        m = FakeModel(8)
+        loop = loop_for(m, max_batch=8, max_tokens=64 * 4, ahead=ahead)
+        prompts = [[1] * n for n in lens]
+        assert loop.run(prompts, SamplingParams(), 6) == [expected(p, 6) for p in prompts]
+        assert loop.stats.batches == 2
 
 
 def test_zero_new_tokens_and_slots_returned_on_error():
@@ -119,10 +154,11 @@ def test_zero_new_tokens_and_slots_returned_on_error():
 
     def broken(entries):
         raise RuntimeError("boom")
-    loop = GenerationLoop(broken, m.sample, m.alloc, m.release, 2, 640, 64)
-    with pytest.raises(RuntimeError, match="boom"):
-        loop.run(PROMPTS[:2], SamplingParams(), 3)
-    assert not m.seq and len(m.free) == 2
+    for draw in (None, m.draw):
+        loop = GenerationLoop(broken, m.sample, m.alloc, m.release, 2, 640, 64, draw=draw)
+        with pytest.raises(RuntimeError, match="boom"):
+            loop.run(PROMPTS[:2], SamplingParams(), 3)
+        assert not m.seq and len(m.free) == 2
 
 
 def test_draws_depend_on_request_and_count_only():
@@ -149,13 +185,57 @@ def test_sampling_params_validation():
     assert SamplingParams().greedy and not SamplingParams(temperature=0.1).greedy
 
 
-def test_tokens_are_reported_as_they_are_kept():
+@AHEAD
+def test_tokens_are_reported_as_they_are_kept(ahead):
     seen = []
     m = FakeModel(3)
     loop = GenerationLoop(m.step, m.sample, m.alloc, m.release, 3, 6400, 256,
-                          on_token=lambda i, t: seen.append((i, t)))
+                          on_token=lambda i, t: seen.append((i, t)), draw=m.draw if ahead else None)
     stops = {expected(PROMPTS[0], 6)[2]}
     out = loop.run(PROMPTS[:3], SamplingParams(), 4, stops)
     for i in range(3):
         assert [t for j, t in seen if j == i] == out[i]
     assert [i for i, _ in seen[:3]] == [0, 1, 2]          # step by step, not request by request
+
+
+def test_the_loop_runs_ahead_only_when_draws_do_not_depend_on_earlier_tokens():
+    """With a repeat penalty a draw needs the tokens before it, which the host has only after
+    reading the last draw: the loop then takes step by step."""
+    m = FakeModel(3)
+    used = []
+
+    def draw(logits, seeds, counters, histories):
+        used.append("draw")
+        return m.draw(logits, seeds, counters, histories)
+
+    def sample(logits, seeds, counters, histories):
+        used.append("sample")
+        assert histories is not None
+        return m.sample(logits, seeds, counters, histories)
+    loop = GenerationLoop(m.step, sample, m.alloc, m.release, 3, 6400, 256, draw=draw)
+    loop.run(PROMPTS[:2], SamplingParams(temperature=0.5, repeat_penalty=1.1), 3)
+    assert set(used) == {"sample"}
+    del used[:]
+    loop.run(PROMPTS[:2], SamplingParams(temperature=0.5), 3)
+    assert set(used) == {"draw"}
+    del used[:]
+    loop.run(PROMPTS[:2], SamplingParams(repeat_penalty=1.3), 3)          # greedy ignores the penalty
+    assert set(used) == {"draw"}
+
+
+def test_random_stops_and_limits_give_the_same_with_and_without_running_ahead():
+    import random
+    rng = random.Random(5)
+    for trial in range(60):
+        prompts = [[rng.randrange(50) for _ in range(rng.randrange(1, 9))] for _ in range(rng.randrange(1, 8))]
+        stops = set(rng.sample(range(50), rng.randrange(0, 12)))
+        n_new = rng.randrange(1, 9)
+        limit = rng.choice([8, 10, 256])
+        include = rng.random() < 0.5
+        got = []
+        for ahead in (False, True):
+            m = FakeModel(3)
+            loop = loop_for(m, max_seq_len=limit, ahead=ahead)
+            got.append(loop.run(prompts, SamplingParams(), n_new, stops, include))
+            assert not m.seq and len(m.free) == 3
+        assert got[0] == got[1] == [expected(p, n_new, stops, include, limit) for p in prompts], trial

@@ -217,6 +217,62 @@ def test_padding_and_batch_company_change_nothing_float32(tmp_path_factory):
         eng.free_slot(sl)
 
 
+def test_a_step_takes_its_tokens_from_the_device(tmp_path_factory):
+    """`device_tokens`: the tokens of a step of single tokens as an int32 tensor on the device
+    (what the sampler left there) instead of the entries' own; the logits are the same bit for
+    bit, with and without graphs, and a step of whole prompts refuses them."""
+    from inferllm_amd import StepEntry
+    from inferllm_amd.engine.step import StepError
+    for graphs in (True, False):
+        eng, plain, config = setup(tmp_path_factory, "B", "bfloat16", use_graphs=graphs)
+        reqs = requests_for(config, [9, 4, 17], seed=6)
+        got = {}
+        for mode in ("host", "device"):
+            slots = [eng.alloc_slot() for _ in reqs]
+            eng.step([StepEntry(s, r[:-3], []) for s, r in zip(slots, reqs)])
+            rows = []
+            for t in range(3):
+                toks = [r[len(r) - 3 + t] for r in reqs]
+                if mode == "host":
+                    out = eng.step([StepEntry(s, [k], [0]) for s, k in zip(slots, toks)])
+                else:
+                    dev = torch.tensor(toks, dtype=torch.int32, device=DEV)
+                    out = eng.step([StepEntry(s, [0], [0]) for s in slots], device_tokens=dev)
+                rows.append(out.clone())
+            got[mode] = torch.stack(rows)
+            for s in slots:
+                eng.free_slot(s)
+        assert torch.equal(got["host"], got["device"])
+        for i, r in enumerate(reqs):
+            assert err(got["device"][:, i], plain(r)[-3:]) < BUDGET["bfloat16"]
+        s = eng.alloc_slot()
+        with pytest.raises(StepError, match="single tokens only"):
+            eng.step([StepEntry(s, [1, 2], [1])], device_tokens=torch.zeros(1, dtype=torch.int32, device=DEV))
+        eng.step([StepEntry(s, [1, 2], [1])])
+        for bad in (torch.zeros(2, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int64, device=DEV),
+                    torch.zeros(1, dtype=torch.int32)):
+            with pytest.raises(StepError, match="device_tokens"):
+                eng.step([StepEntry(s, [3], [0])], device_tokens=bad)
+        eng.free_slot(s)
+        eng.cache.check()
+
+
+def test_generation_with_stop_tokens_runs_ahead_and_equals_plain(tmp_path_factory):
+    """Greedy requests run one step ahead of the host; a sequence that draws a stop token has one
+    void step on its way when the host sees it.  Results and freed slots must be as without."""
+    eng, plain, config = setup(tmp_path_factory, "A", "float32", max_batch=3)
+    prompts = requests_for(config, [5, 11, 2, 7, 3], seed=2)
+    want = [plain_llama.generate_greedy(config, _cache[("A", "float32")][1], p, 12) for p in prompts]
+    stops = {want[0][3], want[2][0], want[3][7]}
+    cut = []
+    for w in want:
+        k = next((i for i, t in enumerate(w) if t in stops), len(w))
+        cut.append(w[:k])
+    assert eng.generate(prompts, max_new_tokens=12, stop_token_ids=sorted(stops)) == cut
+    eng.cache.check()
+    assert eng.cache.slots.n_held() == 0
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_greedy_generation_equals_plain(tmp_path_factory, name):
     import inferllm_amd as I
