@@ -7,12 +7,12 @@ sequence ends at a stop token, at its `max_new_tokens`, or when it reaches the
 longest length the cache allows; it then leaves the batch (its slot is given
 back) while the others go on.  No request joins a batch that has started.
 
-When a draw does not depend on the tokens before it (greedy, or sampling without a repeat
-penalty) and the sampler can hand its tokens on the device (`draw`), the loop runs one step
-ahead: the next step starts from the tokens on the device while the host still waits for
-their copy, so the GPU does not idle while the host decides.  Ends by count (`max_new_tokens`,
-the context limit) are known beforehand; a sequence that drew a stop token has one more step
-on its way, whose result is dropped.
+When the sampler can hand its tokens on the device (`draw`), the loop runs one step ahead:
+the next step starts from the tokens on the device while the host still waits for their copy,
+so the GPU does not idle while the host decides.  Ends by count (`max_new_tokens`, the context
+limit) are known beforehand; a sequence that drew a stop token has one more step on its way,
+whose result is dropped.  A draw that looks at the tokens before it (the repeat penalty) gets
+the newest one, which the host has not read yet, from the device as well (`latest`).
 
 The loop only decides; computing is behind a few callables, so its decisions can
 be tested without a GPU.  The reference's loop is `application/chat.cpp:221-275`
@@ -67,10 +67,11 @@ class GenerationLoop:
     """`step(entries) -> logits`, `sample(logits, seeds, counters, histories) -> ids`,
     `alloc_slot() -> slot`, `free_slot(slot)`; limits of the cache as numbers.
 
-    `draw(logits, seeds, counters, histories)` (optional): like `sample`, but returns an object
-    with `.device` (the tokens where the step function can take them from: `step(entries,
+    `draw(logits, seeds, counters, histories, latest)` (optional): like `sample`, but returns an
+    object with `.device` (the tokens where the step function can take them from: `step(entries,
     device_tokens=...)`), `.pick(rows)` (those of some rows) and `.tokens()` (the host list,
-    waiting if need be).  With it the loop runs one step ahead where the sampling allows."""
+    waiting if need be); `latest` are the newest tokens, still unread, in the same form, and
+    `histories` the ones before them.  With it the loop runs one step ahead."""
 
     def __init__(self, step: Callable, sample: Callable, alloc_slot: Callable[[], int],
                  free_slot: Callable[[int], None], max_batch: int, max_tokens: int,
@@ -141,9 +142,7 @@ class GenerationLoop:
         while waiting:
             batch = self.next_batch(waiting, lens, max_new_tokens)
             waiting = waiting[len(batch):]
-            ahead = self.draw is not None and (params.greedy or params.repeat_penalty == 1.0
-                                               or params.repeat_last_n <= 0)
-            run = self._run_batch_ahead if ahead else self._run_batch
+            run = self._run_batch_ahead if self.draw is not None else self._run_batch
             run(batch, prompts, params, max_new_tokens, stop_ids, include_stop, results)
         return results
 
@@ -155,13 +154,15 @@ class GenerationLoop:
         try:
             for i in batch:
                 everyone.append(_Live(index=i, slot=self.alloc_slot(), prompt_len=len(prompts[i]),
-                                      seed=request_seed(params.seed, i)))
+                                      seed=request_seed(params.seed, i),
+                                      history=[int(t) for t in prompts[i]]))
             self.stats.batches += 1
             self.sync()
             t0 = time.perf_counter()
             logits = self.step([StepEntry(s.slot, prompts[s.index], [s.prompt_len - 1])
                                 for s in everyone])
-            pending = self.draw(logits, [s.seed for s in everyone], [0] * len(everyone), None)
+            pending = self.draw(logits, [s.seed for s in everyone], [0] * len(everyone),
+                                [s.history for s in everyone], None)
             self.sync()
             self.stats.prefill_seconds += time.perf_counter() - t0
             self.stats.prompt_tokens += sum(s.prompt_len for s in everyone)
@@ -184,7 +185,8 @@ class GenerationLoop:
                     logits = self.step([StepEntry(s.slot, [0], [0]) for s in cont],
                                        device_tokens=tokens)
                     following = self.draw(logits, [s.seed for s in cont],
-                                          [s.drawn + 1 for s in cont], None)
+                                          [s.drawn + 1 for s in cont],
+                                          [s.history for s in cont], tokens)
                     self.stats.decode_steps += 1
                 for s, tok in zip(rows, pending.tokens()):
                     if s.dead:
@@ -198,6 +200,7 @@ class GenerationLoop:
                         s.out.append(tok)
                         if self.on_token is not None:
                             self.on_token(s.index, tok)
+                    s.history.append(tok)
                     if why is not None:
                         results[s.index] = s.out
                         self.free_slot(s.slot)     # after the step that still used it was started

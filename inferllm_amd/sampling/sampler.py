@@ -73,9 +73,14 @@ class Sampler:
         return (not p.greedy) and p.repeat_penalty != 1.0 and p.repeat_last_n > 0
 
     def draw(self, logits: torch.Tensor, seeds: Sequence[int], counters: Sequence[int],
-             histories: Optional[Sequence[Sequence[int]]] = None) -> Draw:
+             histories: Optional[Sequence[Sequence[int]]] = None,
+             latest: Optional[torch.Tensor] = None) -> Draw:
         """logits float32 [B, V] on the device -> one token id per row, chosen on the device; the
-        copy to the host is under way when this returns.  At most four draws may be unread."""
+        copy to the host is under way when this returns.  At most four draws may be unread.
+
+        `latest` (int32 [B] on the device): every sequence's newest token when the host has not
+        read it yet; `histories` then hold the tokens before it, and the repeat penalty's window
+        is completed on the device."""
         p = self.params
         self._turn = (self._turn + 1) % 4
         if p.greedy:
@@ -84,8 +89,15 @@ class Sampler:
             rows = None
             if self.needs_histories() and histories is not None:
                 n = p.repeat_last_n
-                rows = [[-1] * (n - min(n, len(h))) + list(h[-n:]) for h in histories]
+                if latest is None:
+                    rows = [[-1] * (n - min(n, len(h))) + list(h[-n:]) for h in histories]
+                else:
+                    m = n - 1
+                    rows = [[-1] * (m - min(m, len(h))) + (list(h[-m:]) if m else []) + [-1]
+                            for h in histories]
             seeds_t, counters_t, last = self._upload(seeds, counters, rows)
+            if last is not None and latest is not None:
+                last[:, -1].copy_(latest)
             dev = ops.sample(logits.contiguous(), p.temperature, p.top_k, p.top_p,
                              p.repeat_penalty, last, seeds_t, counters_t)
         B = dev.numel()

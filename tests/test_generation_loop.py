@@ -41,7 +41,7 @@ class FakeModel:
         return list(logits)
 
     @staticmethod
-    def draw(logits, seeds, counters, histories):
+    def draw(logits, seeds, counters, histories, latest=None):
         return FakeDraw(list(logits))
 
 
@@ -198,29 +198,27 @@ def test_tokens_are_reported_as_they_are_kept(ahead):
     assert [i for i, _ in seen[:3]] == [0, 1, 2]          # step by step, not request by request
 
 
-def test_the_loop_runs_ahead_only_when_draws_do_not_depend_on_earlier_tokens():
-    """With a repeat penalty a draw needs the tokens before it, which the host has only after
-    reading the last draw: the loop then takes step by step."""
-    m = FakeModel(3)
-    used = []
-
-    def draw(logits, seeds, counters, histories):
-        used.append("draw")
-        return m.draw(logits, seeds, counters, histories)
+def test_running_ahead_gives_every_draw_the_same_window_of_earlier_tokens():
+    """A draw that looks back (the repeat penalty) sees the same tokens either way: when the loop
+    runs ahead, the newest one comes as `latest` (unread) and the ones before it as history."""
+    seen = {False: [], True: []}
+    m = None
 
     def sample(logits, seeds, counters, histories):
-        used.append("sample")
-        assert histories is not None
+        seen[False].append([tuple(h) for h in histories])
         return m.sample(logits, seeds, counters, histories)
-    loop = GenerationLoop(m.step, sample, m.alloc, m.release, 3, 6400, 256, draw=draw)
-    loop.run(PROMPTS[:2], SamplingParams(temperature=0.5, repeat_penalty=1.1), 3)
-    assert set(used) == {"sample"}
-    del used[:]
-    loop.run(PROMPTS[:2], SamplingParams(temperature=0.5), 3)
-    assert set(used) == {"draw"}
-    del used[:]
-    loop.run(PROMPTS[:2], SamplingParams(repeat_penalty=1.3), 3)          # greedy ignores the penalty
-    assert set(used) == {"draw"}
+
+    def draw(logits, seeds, counters, histories, latest=None):
+        whole = [tuple(h) + ((latest[i],) if latest is not None else ()) for i, h in enumerate(histories)]
+        seen[True].append(whole)
+        return m.draw(logits, seeds, counters, histories)
+    outs = []
+    for ahead in (False, True):
+        m = FakeModel(3)
+        loop = GenerationLoop(m.step, sample, m.alloc, m.release, 3, 6400, 256, draw=draw if ahead else None)
+        outs.append(loop.run(PROMPTS[:3], SamplingParams(temperature=0.5, repeat_penalty=1.1), 5))
+    assert outs[0] == outs[1]
+    assert seen[False] == seen[True]
 
 
 def test_random_stops_and_limits_give_the_same_with_and_without_running_ahead():

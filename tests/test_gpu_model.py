@@ -292,6 +292,32 @@ def test_greedy_generation_equals_plain(tmp_path_factory, name):
     assert eng.cache.slots.n_held() == 0
 
 
+def test_sampling_with_a_repeat_penalty_is_the_same_step_by_step_and_running_ahead(tmp_path_factory):
+    """The repeat penalty's window ends with the newest token, which the loop that runs ahead has
+    only on the device: both loops must draw the same tokens."""
+    import inferllm_amd as I
+    from inferllm_amd.engine import GenerationLoop
+    from inferllm_amd.sampling import Sampler, SamplingParams
+    eng, plain, config = setup(tmp_path_factory, "B", "float32", max_batch=3)
+    prompts = requests_for(config, [5, 11, 2, 9], seed=8)
+    params = SamplingParams(temperature=0.9, top_k=20, top_p=0.9, repeat_penalty=1.4, repeat_last_n=5, seed=3)
+    outs = []
+    for ahead in (False, True):
+        sampler = Sampler(params, DEV)
+        loop = GenerationLoop(eng.step, sampler, eng.alloc_slot, eng.free_slot, max_batch=3,
+                              max_tokens=eng.cache.max_tokens, max_seq_len=eng.max_seq_len,
+                              draw=sampler.draw if ahead else None)
+        outs.append(loop.run(prompts, params, 10, [7, 9, 11]))
+        eng.cache.check()
+    assert outs[0] == outs[1] and any(len(o) > 3 for o in outs[0])
+    strong = eng.generate(prompts, temperature=0.9, top_k=20, top_p=0.9, repeat_penalty=1.4, repeat_last_n=5,
+                          seed=3, max_new_tokens=10, stop_token_ids=[7, 9, 11])
+    assert strong == outs[0]
+    none = eng.generate(prompts, temperature=0.9, top_k=20, top_p=0.9, seed=3, max_new_tokens=10,
+                        stop_token_ids=[7, 9, 11])
+    assert none != strong                                  # the penalty does change the draws
+
+
 def test_temperature_sampling_is_reproducible_and_batch_independent(tmp_path_factory):
     eng, plain, config = setup(tmp_path_factory, "B", "float32", max_batch=3)
     prompts = requests_for(config, [5, 11, 2], seed=1)
