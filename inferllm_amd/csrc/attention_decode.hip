@@ -27,6 +27,48 @@ __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
     f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
 }
 
+// Combining the results that the waves of a block left in LDS, for one head: row w (of wave w)
+// is at base + w * wstride floats and holds hd sums, then the wave's max and sum; rows are
+// 16-byte aligned (hd + 4 floats).  All reads are asked for at once (a wave beyond `waves` reads
+// the last one's row again, with weight zero): a loop that waits for each in turn took longer
+// than a tile of keys.  a: this lane's 8 dims from dim0 on (if dim_ok).
+#define DEC_MAXW 8
+__device__ __forceinline__ void combine_waves(const float* base, int wstride, int hd, int waves,
+                                              bool dim_ok, int dim0, float& m_out, float& l_out,
+                                              float (&a)[8]) {
+    float mw[DEC_MAXW], lw[DEC_MAXW];
+    float4 v0[DEC_MAXW], v1[DEC_MAXW];
+#pragma unroll
+    for (int w = 0; w < DEC_MAXW; ++w) {
+        const float* wr = base + (size_t)(w < waves ? w : waves - 1) * wstride;
+        mw[w] = wr[hd];
+        lw[w] = wr[hd + 1];
+        v0[w] = make_float4(0.f, 0.f, 0.f, 0.f);
+        v1[w] = v0[w];
+        if (dim_ok) {
+            v0[w] = *(const float4*)(wr + dim0);
+            v1[w] = *(const float4*)(wr + dim0 + 4);
+        }
+    }
+    float mm = NEG_INF;
+#pragma unroll
+    for (int w = 0; w < DEC_MAXW; ++w) mm = fmaxf(mm, w < waves ? mw[w] : NEG_INF);
+    float L = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_MAXW; ++w) {
+        const float wgt = (w < waves && mw[w] != NEG_INF) ? expf(mw[w] - mm) : 0.f;
+        L = fmaf(wgt, lw[w], L);
+        a[0] = fmaf(wgt, v0[w].x, a[0]); a[1] = fmaf(wgt, v0[w].y, a[1]);
+        a[2] = fmaf(wgt, v0[w].z, a[2]); a[3] = fmaf(wgt, v0[w].w, a[3]);
+        a[4] = fmaf(wgt, v1[w].x, a[4]); a[5] = fmaf(wgt, v1[w].y, a[5]);
+        a[6] = fmaf(wgt, v1[w].z, a[6]); a[7] = fmaf(wgt, v1[w].w, a[7]);
+    }
+    m_out = mm;
+    l_out = L;
+}
+
 // LPR: lanes per key row (power of two, 8 dims each, LPR * 8 >= head_dim).
 // GC: query heads handled together (power of two >= heads per kv head, at most 8).
 template <int LPR, int GC>
@@ -40,7 +82,7 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     constexpr int KPI = 64 / LPR;              // keys per load instruction
     constexpr int NI = LPR < 16 ? LPR : 16;    // load instructions per tile
     constexpr int TK = NI * KPI;               // keys per tile
-    extern __shared__ float wave_res[];        // [waves][GC][hd + 2], used when waves > 1
+    extern __shared__ __attribute__((aligned(16))) float wave_res[];   // [waves][GC][hd + 4], used when waves > 1
     const int lane = threadIdx.x & 63, wave = wave_index(), waves = blockDim.x >> 6;
     const int q = lane / LPR, c = lane % LPR;
     const int G = nh / nkv;
@@ -170,10 +212,10 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
         // every wave leaves its result in LDS; wave 0 combines them
 #pragma unroll
         for (int g = 0; g < GC; ++g) {
-            float* wr = wave_res + (size_t)(wave * GC + g) * (hd + 2);
+            float* wr = wave_res + (size_t)(wave * GC + g) * (hd + 4);
             if (q == 0 && dim_ok) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) wr[c * 8 + i] = acc[g][i];
+                *(float4*)(wr + c * 8) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+                *(float4*)(wr + c * 8 + 4) = make_float4(acc[g][4], acc[g][5], acc[g][6], acc[g][7]);
             }
             if (lane == 0) {
                 wr[hd] = m[g];
@@ -183,29 +225,9 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
         __syncthreads();
         if (wave != 0) return;
 #pragma unroll
-        for (int g = 0; g < GC; ++g) {
-            float mm = NEG_INF;
-            for (int w = 0; w < waves; ++w)
-                mm = fmaxf(mm, wave_res[(size_t)(w * GC + g) * (hd + 2) + hd]);
-            float L = 0.f, a[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) a[i] = 0.f;
-            for (int w = 0; w < waves; ++w) {
-                const float* wr = wave_res + (size_t)(w * GC + g) * (hd + 2);
-                const float mw = wr[hd];
-                if (mw == NEG_INF) continue;
-                const float wgt = expf(mw - mm);
-                L += wgt * wr[hd + 1];
-                if (q == 0 && dim_ok) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) a[i] = fmaf(wgt, wr[c * 8 + i], a[i]);
-                }
-            }
-            m[g] = mm;
-            l[g] = L;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[g][i] = a[i];
-        }
+        for (int g = 0; g < GC; ++g)
+            combine_waves(wave_res + (size_t)g * (hd + 4), GC * (hd + 4), hd, waves,
+                          q == 0 && dim_ok, c * 8, m[g], l[g], acc[g]);
     }
 #pragma unroll
     for (int g = 0; g < GC; ++g) {
@@ -463,6 +485,231 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
     }
 }
 
+// Grouped heads, head_dim % 32 == 0 and <= 128: both products on the matrix cores.
+//
+// S^T[key][head] = K . Q^T as in the kernel above.  For O[head][dim] = P . V with MFMA 16x16x32
+// the contraction runs over keys: lane (r, k-group q4) supplies 8 keys of head r as the A
+// operand and lane (n, q4) 8 keys of ONE dim as the B operand, while V lies in the cache with
+// the dims of a key contiguous.  Two things make that cheap.  The order of the keys within the
+// contraction is free as long as A and B agree, so the 32 keys of an MFMA are taken in the order
+// in which the first product left their scores: lane (r, q4) already holds head r's probabilities
+// of keys 16 sub + 4 q4 + i (sub = 0..3, i = 0..3), and two sub-tiles of them are its A operand
+// as they are: P never leaves the registers.  And lane (n, q4) loads, for the same 8 keys,
+// the 8 dims 8 n .. 8 n + 7 (16 bytes of a row), an 8 x 8 block that it transposes in its own
+// registers with byte permutes; row e of the transposed block is the B operand of the MFMA that
+// gives dims 8 n + e of all 16 heads.  Eight MFMAs per 32 keys cover 128 dims, and a lane ends
+// up with 4 heads x 8 consecutive dims.  A block takes up to 16 heads of a kv head.
+// Measured against the kernel above at 8 sequences of 650 keys, 32/8 heads: see DESIGN.md.
+template <int HD>
+__global__ void __launch_bounds__(512)
+attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
+                               const bf16_t* __restrict__ kcache,
+                               const bf16_t* __restrict__ vcache,
+                               const int32_t* __restrict__ page_table, int table_stride,
+                               int page_size, int ring, const int32_t* __restrict__ seq_slot,
+                               const int32_t* __restrict__ seq_len, float* __restrict__ partial,
+                               int nsplit, int nh, int nkv, float scale, int window) {
+    constexpr int TK = 64;                     // keys per tile
+    constexpr int KS = HD / 32;                // k-steps of 32 dims of the first product
+    extern __shared__ __attribute__((aligned(16))) float lds[];   // the waves' results at the end
+    const int lane = threadIdx.x & 63, wave = wave_index(), waves = blockDim.x >> 6;
+    const int r = lane & 15, q4 = lane >> 4;
+    const int G = nh / nkv;
+    const int chunks = (G + 15) / 16;
+    const int kvh = blockIdx.x / chunks, g0 = (blockIdx.x % chunks) * 16;
+    const int GH = min(16, G - g0);            // heads of this block
+    const int b = blockIdx.y, sp = blockIdx.z;
+    const int slot = seq_slot[b];
+    const int len = seq_len[b];
+    const int kf = window > 0 ? max(0, len - window) : 0;
+    const bool dim_ok = r * 8 < HD;            // this lane's 8 dims as an owner of V columns
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
+
+    uint4 qf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        qf[s] = make_uint4(0, 0, 0, 0);
+        if (r < GH)
+            qf[s] = *(const uint4*)(qkv + (size_t)b * rowlen + (size_t)(kvh * G + g0 + r) * HD +
+                                    s * 32 + q4 * 8);
+    }
+    float m = NEG_INF, l = 0.f;                // of head r (the same in the four k groups)
+    df32x4_t o[8];                             // o[e][i]: head 4 q4 + i, dim 8 r + e
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (df32x4_t){0.f, 0.f, 0.f, 0.f};
+
+    const int t_first = kf / TK;
+    const int n_tiles = (len + TK - 1) / TK - t_first;
+    const int per = (n_tiles + nsplit - 1) / nsplit;
+    const int t_lo = t_first + sp * per;
+    const int t_hi = min(t_first + n_tiles, t_lo + per);
+
+    for (int t = t_lo + wave; t < t_hi; t += waves) {
+        const int k0 = t * TK;
+        int lp = k0 / page_size;
+        if (ring > 0) lp %= ring;
+        const int phys = page_table[(size_t)slot * table_stride + lp];
+        const size_t tile = (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)HD;
+        uint4 ka[4][KS], vr[2][8];
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                ka[sub][s] = *(const uint4*)(kcache + tile + (size_t)(sub * 16 + r) * HD + s * 32 + q4 * 8);
+        // V: slot i of half hb is key (2 hb + i / 4) * 16 + 4 q4 + i % 4, the key whose score this
+        // k group's lanes get at place i % 4 of sub-tile 2 hb + i / 4
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int kt = (2 * hb + i / 4) * 16 + 4 * q4 + (i & 3);
+                vr[hb][i] = dim_ok ? *(const uint4*)(vcache + tile + (size_t)kt * HD + r * 8)
+                                   : make_uint4(0, 0, 0, 0);
+            }
+        if (k0 + TK > len || k0 < kf) {
+            // a tile with keys that do not count: their rows may hold anything (NaN too), and a
+            // probability of zero would not undo that
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int key = k0 + (2 * hb + i / 4) * 16 + 4 * q4 + (i & 3);
+                    if (!(key < len && key >= kf)) vr[hb][i] = make_uint4(0, 0, 0, 0);
+                }
+        }
+        // scores of 4 keys per sub-tile for head r
+        float sv[4][4];
+        float mx = NEG_INF;
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub) {
+            df32x4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+                a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const dbf16x8_t*)&ka[sub][s],
+                                                            *(const dbf16x8_t*)&qf[s], a, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = k0 + sub * 16 + 4 * q4 + i;
+                const bool ok = key < len && key >= kf;
+                sv[sub][i] = ok ? a[i] * scale : NEG_INF;
+                mx = fmaxf(mx, sv[sub][i]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, ILLM_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
+        const float alpha = expf(m - m_use);             // m = -inf gives 0 (nothing summed yet)
+        float rs = 0.f;
+        uint4 pa[2];                                     // head r's probabilities, two A operands
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+            float pf[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float sc = sv[2 * hb + i / 4][i & 3];
+                pf[i] = (sc == NEG_INF) ? 0.f : expf(sc - m_use);
+                rs += pf[i];
+            }
+            pa[hb] = make_uint4(pack_bf16x2(pf[0], pf[1]), pack_bf16x2(pf[2], pf[3]),
+                                pack_bf16x2(pf[4], pf[5]), pack_bf16x2(pf[6], pf[7]));
+        }
+        rs += __shfl_xor(rs, 16, ILLM_WAVE);
+        rs += __shfl_xor(rs, 32, ILLM_WAVE);
+        l = l * alpha + rs;
+        m = m_new;
+        // what this lane has summed belongs to heads 4 q4 + i, whose factors lanes 4 q4 + i hold
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float ai = __shfl(alpha, 4 * q4 + i, ILLM_WAVE);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e][i] *= ai;
+        }
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                // row e of the transposed 8 keys x 8 dims block: dim 8 r + e of the 8 keys
+                const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                uint4 tr;
+                const uint32_t* w0 = (const uint32_t*)&vr[hb][0];
+                tr.x = __builtin_amdgcn_perm(((const uint32_t*)&vr[hb][1])[e >> 1], w0[e >> 1], sel);
+                tr.y = __builtin_amdgcn_perm(((const uint32_t*)&vr[hb][3])[e >> 1],
+                                             ((const uint32_t*)&vr[hb][2])[e >> 1], sel);
+                tr.z = __builtin_amdgcn_perm(((const uint32_t*)&vr[hb][5])[e >> 1],
+                                             ((const uint32_t*)&vr[hb][4])[e >> 1], sel);
+                tr.w = __builtin_amdgcn_perm(((const uint32_t*)&vr[hb][7])[e >> 1],
+                                             ((const uint32_t*)&vr[hb][6])[e >> 1], sel);
+                o[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const dbf16x8_t*)&pa[hb],
+                                                               *(const dbf16x8_t*)&tr, o[e], 0, 0, 0);
+            }
+        }
+    }
+    // this lane's heads 4 q4 + i: their max and sum from the lanes that hold them
+    float lh[4], mh[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        lh[i] = __shfl(l, 4 * q4 + i, ILLM_WAVE);
+        mh[i] = __shfl(m, 4 * q4 + i, ILLM_WAVE);
+    }
+    if (waves > 1) {
+        // every wave leaves its result in LDS ([wave][head][HD + 4]); wave 0 combines them
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int hl = 4 * q4 + i;
+            if (hl >= GH) continue;
+            float* wr = lds + (size_t)(wave * GH + hl) * (HD + 4);
+            if (dim_ok) {
+                *(float4*)(wr + r * 8) = make_float4(o[0][i], o[1][i], o[2][i], o[3][i]);
+                *(float4*)(wr + r * 8 + 4) = make_float4(o[4][i], o[5][i], o[6][i], o[7][i]);
+            }
+            if (r == 0) {
+                wr[HD] = mh[i];
+                wr[HD + 1] = lh[i];
+            }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int hl = 4 * q4 + i;
+            if (hl >= GH) continue;
+            float a[8];
+            combine_waves(lds + (size_t)hl * (HD + 4), GH * (HD + 4), HD, waves, dim_ok, r * 8,
+                          mh[i], lh[i], a);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e][i] = a[e];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int hl = 4 * q4 + i;
+        if (hl >= GH) continue;
+        const int h = kvh * G + g0 + hl;
+        if (nsplit == 1) {
+            if (dim_ok) {
+                const float inv = 1.0f / lh[i];
+                uint4 ov;
+                ov.x = pack_bf16x2(o[0][i] * inv, o[1][i] * inv);
+                ov.y = pack_bf16x2(o[2][i] * inv, o[3][i] * inv);
+                ov.z = pack_bf16x2(o[4][i] * inv, o[5][i] * inv);
+                ov.w = pack_bf16x2(o[6][i] * inv, o[7][i] * inv);
+                *(uint4*)(out + ((size_t)b * nh + h) * HD + r * 8) = ov;
+            }
+        } else {
+            float* pp = partial + (((size_t)b * nh + h) * nsplit + sp) * (size_t)(HD + 2);
+            if (dim_ok) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pp[r * 8 + e] = o[e][i];
+            }
+            if (r == 0) {
+                pp[HD] = mh[i];
+                pp[HD + 1] = lh[i];
+            }
+        }
+    }
+}
+
 // grid (heads, sequences), one wave: lane s holds split s's max and sum (nsplit <= 64), the
 // weights are formed once, and splits that saw no key are skipped.
 __global__ void __launch_bounds__(64)
@@ -480,9 +727,19 @@ attn_decode_bf16_merge_kernel(const float* __restrict__ partial, bf16_t* __restr
     const float inv = 1.0f / wave_sum(w * ls);
     for (int d = lane; d < hd; d += 64) {
         float a = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float ws = __shfl(w, s, ILLM_WAVE);
-            if (ws != 0.f) a = fmaf(ws, pp[(size_t)s * (hd + 2) + d], a);
+        // eight splits' values are asked for at once (beyond the last: the last again, unused)
+        for (int s0 = 0; s0 < nsplit; s0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int s = s0 + u < nsplit ? s0 + u : nsplit - 1;
+                v[u] = pp[(size_t)s * (hd + 2) + d];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float ws = __shfl(w, (s0 + u) & 63, ILLM_WAVE);
+                a = (s0 + u < nsplit && ws != 0.f) ? fmaf(ws, v[u], a) : a;
+            }
         }
         out[((size_t)b * nh + h) * hd + d] = f32_to_bf16(a * inv);
     }
@@ -498,7 +755,7 @@ static int launch_decode(const void* qkv, void* out, const void* kcache, const v
     const int chunks = (G + GC - 1) / GC;
     const int maxw = GC <= 4 ? 8 : 4;
     waves = waves < 1 ? 1 : (waves > maxw ? maxw : waves);
-    const size_t smem = waves > 1 ? (size_t)waves * GC * (hd + 2) * sizeof(float) : 0;
+    const size_t smem = waves > 1 ? (size_t)waves * GC * (hd + 4) * sizeof(float) : 0;
     hipLaunchKernelGGL((attn_decode_bf16_kernel<LPR, GC>), dim3(nkv * chunks, B, nsplit),
                        dim3(64 * waves), smem, stream, (const bf16_t*)qkv, (bf16_t*)out, (const bf16_t*)kcache,
                        (const bf16_t*)vcache, page_table, table_stride, page_size, ring, seq_slot,
@@ -532,6 +789,9 @@ static int launch_decode_g(int gc, const void* qkv, void* out, const void* kcach
 // is a multiple of 64.  Anything else: ILLM_ERR_ARG (the caller uses the generic kernel).
 // `waves`: waves per block that share a key range (clamped to what registers and LDS allow);
 // `nsplit`: key ranges per sequence, combined by the merge kernel when > 1.
+static int GQA_PV_ON_MATRIX_CORES = 1;      // 0: the kernel with P.V on the vector units (tuning)
+extern "C" void illm_set_gqa_pv_on_matrix_cores(int on) { GQA_PV_ON_MATRIX_CORES = on; }
+
 extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache,
                                      const void* vcache, const int32_t* page_table,
                                      int table_stride, int page_size, int ring,
@@ -544,6 +804,30 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
     const int G = nh / nkv;
+    if (G > 1 && hd % 32 == 0 && hd <= 128 && GQA_PV_ON_MATRIX_CORES) {
+        const int chunks = (G + 15) / 16, gh = G < 16 ? G : 16;
+        const dim3 grid(nkv * chunks, B, nsplit);
+        int wq = waves < 1 ? 1 : (waves > 8 ? 8 : waves);
+        while (wq > 1 && (size_t)wq * gh * (hd + 4) * sizeof(float) > 64 * 1024) --wq;
+        const size_t smem = wq > 1 ? (size_t)wq * gh * (hd + 4) * sizeof(float) : 0;
+#define GQA_PV(HD_)                                                                                \
+    hipLaunchKernelGGL((attn_decode_bf16_gqa_pv_kernel<HD_>), grid, dim3(64 * wq), smem,           \
+                       (hipStream_t)stream, (const bf16_t*)qkv, (bf16_t*)out,                      \
+                       (const bf16_t*)kcache, (const bf16_t*)vcache, page_table, table_stride,     \
+                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, scale, window)
+        switch (hd) {
+            case 32: GQA_PV(32); break;
+            case 64: GQA_PV(64); break;
+            case 96: GQA_PV(96); break;
+            default: GQA_PV(128); break;
+        }
+#undef GQA_PV
+        if (nsplit > 1)
+            hipLaunchKernelGGL(attn_decode_bf16_merge_kernel, dim3(nh, B), dim3(64), 0,
+                               (hipStream_t)stream, (const float*)partial, (bf16_t*)out, nsplit, nh,
+                               hd);
+        return illm_launch_status();
+    }
     if (G > 1 && hd % 32 == 0) {
         int gcq = 2;
         while (gcq < G && gcq < 16) gcq <<= 1;

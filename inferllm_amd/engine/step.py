@@ -44,11 +44,23 @@ def _bucket(n: int) -> int:
     return b
 
 
-class _DecodeGraph:
-    """Static buffers and the captured graph for decode steps of one bucket size."""
+def _length_class(n: int, limit: int) -> int:
+    """The class of a decode step by its longest sequence: 1024, 2048, 4096, ... keys, at most
+    the cache's limit.  How attention cuts the keys among blocks is fixed when a graph is
+    captured, and what is best for 600 keys is not for 4000."""
+    c = 1024
+    while c < n:
+        c *= 2
+    return min(c, max(limit, 1))
 
-    def __init__(self, runner: "StepRunner", size: int):
+
+class _DecodeGraph:
+    """Static buffers and the captured graph for decode steps of one bucket size and one class
+    of lengths."""
+
+    def __init__(self, runner: "StepRunner", size: int, max_len: int):
         self.size = size
+        self.max_len = max_len
         dev = runner.device
         self.meta = torch.zeros(4 * size, dtype=torch.int32, device=dev)   # tokens | pos | slot | len
         # host side of `meta`: pinned, so that one asynchronous copy brings a step's numbers over
@@ -67,7 +79,7 @@ class _DecodeGraph:
             device=runner.device, act_dtype=runner.act_dtype, prefill=False, n_rows=n, n_seqs=n,
             tokens=self.meta[:n], row_pos=self.meta[n:2 * n], row_slot=self.meta[2 * n:3 * n],
             cu_seqlens=self.cu, seq_slot=self.meta[2 * n:3 * n], seq_len=self.meta[3 * n:],
-            max_len=runner.cache.max_seq_len, cache=runner.cache)
+            max_len=self.max_len, cache=runner.cache)
 
 
 class StepRunner:
@@ -80,7 +92,7 @@ class StepRunner:
         self.vocab_size = model.spec.vocab_size
         self.use_graphs = (use_graphs and model.graph_safe
                            and os.environ.get("INFERLLM_NO_GRAPH", "0") != "1")
-        self._graphs: Dict[int, _DecodeGraph] = {}
+        self._graphs: Dict[tuple, _DecodeGraph] = {}
 
     # ------------------------------------------------------------ checks
     def _phase(self, entries: Sequence[StepEntry]) -> bool:
@@ -187,9 +199,10 @@ class StepRunner:
                 cache=self.cache)
             rows = torch.tensor(wanted, dtype=torch.int32, device=self.device) if wanted else None
             return self.model.forward(ctx, rows)
-        g = self._graphs.get(size)
+        key = (size, _length_class(max(starts) + 1, self.cache.max_seq_len))
+        g = self._graphs.get(key)
         if g is None:
-            g = self._graphs[size] = _DecodeGraph(self, size)
+            g = self._graphs[key] = _DecodeGraph(self, *key)
         if g.in_flight:
             g.copied.synchronize()          # the last step's copy has left the pinned buffer
         g.stage_np[:] = host

@@ -130,7 +130,7 @@ def attn_prefill(qkv, cu_seqlens, n_seqs, max_len, nh, nkv, hd, scale, window):
     return out
 
 
-def decode_splits(B, nkv, max_len):
+def decode_splits(B, nkv, max_len, nh=0, hd=0):
     return 2, 1
 
 
