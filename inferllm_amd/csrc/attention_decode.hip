@@ -20,6 +20,13 @@
 
 #define NEG_INF (-INFINITY)
 
+// e^x for the softmax of bfloat16 rows: the hardware's base-2 exponential of x * log2(e), three
+// instructions instead of the library routine's thirty; its relative error, about |x| * 6e-8, is
+// far below what bfloat16 keeps.  (The float32 path has kernels of its own with expf.)
+__device__ __forceinline__ float fexp(float x) {
+    return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
+}
+
 __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
     f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
     f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
@@ -27,46 +34,56 @@ __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
     f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
 }
 
-// Combining the results that the waves of a block left in LDS, for one head: row w (of wave w)
-// is at base + w * wstride floats and holds hd sums, then the wave's max and sum; rows are
-// 16-byte aligned (hd + 4 floats).  All reads are asked for at once (a wave beyond `waves` reads
-// the last one's row again, with weight zero): a loop that waits for each in turn took longer
-// than a tile of keys.  a: this lane's 8 dims from dim0 on (if dim_ok).
+// Combining the results that the waves of a block left in LDS and writing them out, by the
+// whole block: row (w, head) is at lds + (w * n_heads + head) * (hd + 4) floats and holds hd
+// sums, then the wave's max and sum.  A thread takes 4 dims of one head and asks for all the
+// waves' values at once (a wave beyond `waves` reads the last one's row again, with weight
+// zero): one wave walking through heads and waves in turn took longer than a tile of keys.
+// The block's heads are bh0, bh0 + 1, ... in the numbering b * nh + head; a wave's rows are
+// row_heads apart, of which the first n_heads count.
 #define DEC_MAXW 8
-__device__ __forceinline__ void combine_waves(const float* base, int wstride, int hd, int waves,
-                                              bool dim_ok, int dim0, float& m_out, float& l_out,
-                                              float (&a)[8]) {
-    float mw[DEC_MAXW], lw[DEC_MAXW];
-    float4 v0[DEC_MAXW], v1[DEC_MAXW];
+__device__ __forceinline__ void combine_block(const float* lds, int row_heads, int n_heads, int hd,
+                                              int waves, bf16_t* out, float* partial, int nsplit,
+                                              int sp, size_t bh0) {
+    const int stride = hd + 4, per_head = hd / 4;
+    for (int idx = threadIdx.x; idx < n_heads * per_head; idx += blockDim.x) {
+        const int hl = idx / per_head, d = (idx % per_head) * 4;
+        float mw[DEC_MAXW], lw[DEC_MAXW];
+        float4 v[DEC_MAXW];
 #pragma unroll
-    for (int w = 0; w < DEC_MAXW; ++w) {
-        const float* wr = base + (size_t)(w < waves ? w : waves - 1) * wstride;
-        mw[w] = wr[hd];
-        lw[w] = wr[hd + 1];
-        v0[w] = make_float4(0.f, 0.f, 0.f, 0.f);
-        v1[w] = v0[w];
-        if (dim_ok) {
-            v0[w] = *(const float4*)(wr + dim0);
-            v1[w] = *(const float4*)(wr + dim0 + 4);
+        for (int w = 0; w < DEC_MAXW; ++w) {
+            const float* wr = lds + ((size_t)(w < waves ? w : waves - 1) * row_heads + hl) * stride;
+            mw[w] = wr[hd];
+            lw[w] = wr[hd + 1];
+            v[w] = *(const float4*)(wr + d);
+        }
+        float mm = NEG_INF;
+#pragma unroll
+        for (int w = 0; w < DEC_MAXW; ++w) mm = fmaxf(mm, w < waves ? mw[w] : NEG_INF);
+        float L = 0.f;
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int w = 0; w < DEC_MAXW; ++w) {
+            const float wgt = (w < waves && mw[w] != NEG_INF) ? fexp(mw[w] - mm) : 0.f;
+            L = fmaf(wgt, lw[w], L);
+            a.x = fmaf(wgt, v[w].x, a.x); a.y = fmaf(wgt, v[w].y, a.y);
+            a.z = fmaf(wgt, v[w].z, a.z); a.w = fmaf(wgt, v[w].w, a.w);
+        }
+        const size_t bh = bh0 + hl;
+        if (nsplit == 1) {
+            const float inv = 1.0f / L;
+            *(uint2*)(out + bh * hd + d) =
+                make_uint2(pack_bf16x2(a.x * inv, a.y * inv), pack_bf16x2(a.z * inv, a.w * inv));
+        } else {
+            float* pp = partial + (bh * nsplit + sp) * (size_t)(hd + 2);
+            *(float2*)(pp + d) = make_float2(a.x, a.y);
+            *(float2*)(pp + d + 2) = make_float2(a.z, a.w);
+            if (d == 0) {
+                pp[hd] = mm;
+                pp[hd + 1] = L;
+            }
         }
     }
-    float mm = NEG_INF;
-#pragma unroll
-    for (int w = 0; w < DEC_MAXW; ++w) mm = fmaxf(mm, w < waves ? mw[w] : NEG_INF);
-    float L = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) a[i] = 0.f;
-#pragma unroll
-    for (int w = 0; w < DEC_MAXW; ++w) {
-        const float wgt = (w < waves && mw[w] != NEG_INF) ? expf(mw[w] - mm) : 0.f;
-        L = fmaf(wgt, lw[w], L);
-        a[0] = fmaf(wgt, v0[w].x, a[0]); a[1] = fmaf(wgt, v0[w].y, a[1]);
-        a[2] = fmaf(wgt, v0[w].z, a[2]); a[3] = fmaf(wgt, v0[w].w, a[3]);
-        a[4] = fmaf(wgt, v1[w].x, a[4]); a[5] = fmaf(wgt, v1[w].y, a[5]);
-        a[6] = fmaf(wgt, v1[w].z, a[6]); a[7] = fmaf(wgt, v1[w].w, a[7]);
-    }
-    m_out = mm;
-    l_out = L;
 }
 
 // LPR: lanes per key row (power of two, 8 dims each, LPR * 8 >= head_dim).
@@ -175,8 +192,8 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
         for (int g = 0; g < GC; ++g) {
             const float s = own_ok ? s_own[g] : NEG_INF;
             const float m_new = fmaxf(m[g], wave_max(s));
-            const float alpha = (m_new == NEG_INF) ? 1.f : expf(m[g] - m_new);
-            const float p = own_ok ? expf(s - m_new) : 0.f;
+            const float alpha = (m_new == NEG_INF) ? 1.f : fexp(m[g] - m_new);
+            const float p = own_ok ? fexp(s - m_new) : 0.f;
             p_own[g] = p;
             l[g] = l[g] * alpha + wave_sum(p);
             m[g] = m_new;
@@ -223,11 +240,9 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
             }
         }
         __syncthreads();
-        if (wave != 0) return;
-#pragma unroll
-        for (int g = 0; g < GC; ++g)
-            combine_waves(wave_res + (size_t)g * (hd + 4), GC * (hd + 4), hd, waves,
-                          q == 0 && dim_ok, c * 8, m[g], l[g], acc[g]);
+        combine_block(wave_res, GC, min(GC, G - g0), hd, waves, out, partial, nsplit, sp,
+                      (size_t)b * nh + kvh * G + g0);
+        return;
     }
 #pragma unroll
     for (int g = 0; g < GC; ++g) {
@@ -357,7 +372,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
         mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
-        const float alpha = expf(m - m_use);             // m = -inf gives 0 (nothing summed yet)
+        const float alpha = fexp(m - m_use);             // m = -inf gives 0 (nothing summed yet)
         float rs = 0.f;
         // P is private to the wave, whose LDS accesses run in program order: no barrier, only
         // a fence for the compiler
@@ -366,7 +381,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
         for (int sub = 0; sub < NSUB; ++sub)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float p = (sv[sub][i] == NEG_INF) ? 0.f : expf(sv[sub][i] - m_use);
+                const float p = (sv[sub][i] == NEG_INF) ? 0.f : fexp(sv[sub][i] - m_use);
                 rs += p;
                 ps[(sub * 16 + 4 * q4 + i) * PLD + r] = p;
             }
@@ -444,7 +459,7 @@ attn_decode_bf16_gqa_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__
                 const float* wr = lds + (size_t)(w * GC + g) * (HD + 2);
                 const float mw = wr[HD];
                 if (mw == NEG_INF) continue;
-                const float wgt = expf(mw - mm);
+                const float wgt = fexp(mw - mm);
                 L += wgt * wr[HD + 1];
                 if (q == 0 && dim_ok) {
 #pragma unroll
@@ -599,7 +614,7 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
         mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
-        const float alpha = expf(m - m_use);             // m = -inf gives 0 (nothing summed yet)
+        const float alpha = fexp(m - m_use);             // m = -inf gives 0 (nothing summed yet)
         float rs = 0.f;
         uint4 pa[2];                                     // head r's probabilities, two A operands
 #pragma unroll
@@ -608,7 +623,7 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const float sc = sv[2 * hb + i / 4][i & 3];
-                pf[i] = (sc == NEG_INF) ? 0.f : expf(sc - m_use);
+                pf[i] = (sc == NEG_INF) ? 0.f : fexp(sc - m_use);
                 rs += pf[i];
             }
             pa[hb] = make_uint4(pack_bf16x2(pf[0], pf[1]), pack_bf16x2(pf[2], pf[3]),
@@ -669,17 +684,9 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
             }
         }
         __syncthreads();
-        if (wave != 0) return;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int hl = 4 * q4 + i;
-            if (hl >= GH) continue;
-            float a[8];
-            combine_waves(lds + (size_t)hl * (HD + 4), GH * (HD + 4), HD, waves, dim_ok, r * 8,
-                          mh[i], lh[i], a);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[e][i] = a[e];
-        }
+        combine_block(lds, GH, GH, HD, waves, out, partial, nsplit, sp,
+                      (size_t)b * nh + kvh * G + g0);
+        return;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -723,7 +730,7 @@ attn_decode_bf16_merge_kernel(const float* __restrict__ partial, bf16_t* __restr
         ls = pp[(size_t)lane * (hd + 2) + hd + 1];
     }
     const float m = wave_max(ms);
-    const float w = (ms == NEG_INF) ? 0.f : expf(ms - m);
+    const float w = (ms == NEG_INF) ? 0.f : fexp(ms - m);
     const float inv = 1.0f / wave_sum(w * ls);
     for (int d = lane; d < hd; d += 64) {
         float a = 0.f;

@@ -591,24 +591,16 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
 def decode_splits(B: int, nkv: int, max_len: int, nh: int = 0, hd: int = 0):
     """(nsplit, waves): how to cut the keys of a decode step among blocks (`nsplit` ranges per
     sequence, combined by a merge kernel) and among the waves of a block (combined in LDS).
-    Measured on MI355X at head size 128, 1 to 64 sequences of 650 to 4000 keys:
-
-    * grouped heads on the kernel with both products on the matrix cores (nh > nkv, hd a
-      multiple of 32 up to 128): blocks of one wave, about 512 of them; a block of several waves
-      costs 3 us more than it saves until there are fewer sequences than that;
-    * one head per kv head: the same for fewer than 256 (sequence, head) pairs and at most 16
-      tiles of keys; otherwise about 2048 waves, up to 8 in a block, then ranges."""
-    blocks = max(1, B * nkv)
+    Measured on MI355X at head size 128, 32/32, 32/8 and 64/8 heads, 1 to 64 sequences of 650
+    to 4000 keys: about as many blocks as the chip has compute units (256) is best or within a
+    microsecond of it, in at most 16 ranges; 8 waves a block (idle ones cost nothing) until
+    there are 512 blocks, then 4."""
+    base = max(1, B * nkv)
+    if nh > nkv > 0 and hd % 32 == 0 and 0 < hd <= 128:
+        base *= -(-(nh // nkv) // 16)          # the grouped kernel takes 16 heads a block
     tiles = max(1, (max_len + 63) // 64)
-    grouped = nh > nkv > 0 and hd % 32 == 0 and 0 < hd <= 128
-    if grouped:
-        blocks *= -(-(nh // nkv) // 16)
-        return max(1, min(-(-512 // blocks), tiles, 16)), 1
-    if blocks < 256 and tiles <= 16:
-        return max(1, min(-(-1024 // blocks), tiles)), 1
-    want = max(1, min(-(-2048 // blocks), tiles))
-    waves = min(8, want)
-    return max(1, min(-(-want // waves), 32)), waves
+    nsplit = max(1, min(-(-256 // base), 16, tiles))
+    return nsplit, (8 if base * nsplit < 512 else 4)
 
 
 def attn_decode(qkv: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
