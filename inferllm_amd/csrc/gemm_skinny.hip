@@ -63,7 +63,10 @@ struct SkResidual {
 // with tile = blockIdx.x holding the 16 rows that block works on (in its mode's order): a load
 // instruction then reads 1 KB that is contiguous and already in operand order, so the lines need
 // no reordering in LDS.  Measured at the 7B shapes: 6 to 17 % less time than from row-major W.
-template <int MT, int NTB, int SK_U, int MAXW, int MODE, bool TILED>
+// ONE_SHOT: a wave asks for its whole share of K at once and holds no second piece (for K that
+// the block's waves cover in one piece each: the product of a short K is bound by the round
+// trips of a wave's pieces, not by bandwidth).
+template <int MT, int NTB, int SK_U, int MAXW, int MODE, bool TILED, bool ONE_SHOT = false>
 __global__ void __launch_bounds__(64 * MAXW)
 gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                    void* __restrict__ Y, int y_dt, int M, int N, int K, SkRope rope,
@@ -251,9 +254,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
     if (s0 < ksteps) load(s0, a, b);
     for (; s0 < ksteps; s0 += stride) {
         // the next piece is on its way while this one is multiplied
-        uint4 an[NTB][SK_U], bn[MT][SK_U];
-        const bool more = s0 + stride < ksteps;
-        if (more) load(s0 + stride, an, bn);
+        uint4 an[ONE_SHOT ? 1 : NTB][SK_U], bn[ONE_SHOT ? 1 : MT][SK_U];
+        const bool more = !ONE_SHOT && s0 + stride < ksteps;
+        if constexpr (ONE_SHOT) {
+            if (s0 != wave * SK_U) load(s0, a, b);       // (a K longer than one piece a wave)
+        } else {
+            if (more) load(s0 + stride, an, bn);
+        }
         if (!TILED) {
 #pragma unroll
             for (int u = 0; u < SK_U; ++u) {
@@ -276,13 +283,15 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                     acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                         *(const bf16x8_t*)&am, *(bf16x8_t*)&b[mt][u], acc[nt][mt], 0, 0, 0);
             }
-        if (more) {
+        if constexpr (!ONE_SHOT) {
+            if (more) {
 #pragma unroll
-            for (int u = 0; u < SK_U; ++u) {
+                for (int u = 0; u < SK_U; ++u) {
 #pragma unroll
-                for (int nt = 0; nt < NTB; ++nt) a[nt][u] = an[nt][u];
+                    for (int nt = 0; nt < NTB; ++nt) a[nt][u] = an[nt][u];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) b[mt][u] = bn[mt][u];
+                    for (int mt = 0; mt < MT; ++mt) b[mt][u] = bn[mt][u];
+                }
             }
         }
     }
@@ -432,19 +441,19 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
 
 static const SkResidual SK_NO_RESIDUAL = {0, nullptr, ILLM_BF16, nullptr, nullptr, nullptr, 0, 0.f};
 
-template <int MT, int NTB, int U, int MODE = SK_PLAIN, bool TILED = false>
+template <int MT, int NTB, int U, int MODE = SK_PLAIN, bool TILED = false, bool ONE_SHOT = false>
 static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M, int N, int K,
                          int waves, hipStream_t st, SkRope rope = SkRope(),
                          SkResidual res = SK_NO_RESIDUAL) {
     constexpr bool DUAL = MODE == SK_GATE_UP;
-    // registers a lane needs: operands of two pieces in flight and the accumulators
-    constexpr int REGS = 2 * (NTB + MT) * U * 4 + NTB * 8 + NTB * MT * 4 + 40;
+    // registers a lane needs: operands of two pieces in flight (one if ONE_SHOT) and the accumulators
+    constexpr int REGS = (ONE_SHOT ? 1 : 2) * (NTB + MT) * U * 4 + NTB * 8 + NTB * MT * 4 + 40;
     constexpr int MAXW = REGS <= 128 ? 16 : (REGS <= 256 ? 8 : 4);
     waves = waves > MAXW ? MAXW : waves;
     const int rows_per_block = DUAL ? 8 * NTB : 16 * NTB;
     const int blocks = (N + rows_per_block - 1) / rows_per_block;
     const size_t smem = (size_t)waves * NTB * ((!TILED && U > MT) ? U : MT) * 1024 + 64;
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, MODE, TILED>), dim3(blocks), dim3(64 * waves),
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NTB, U, MAXW, MODE, TILED, ONE_SHOT>), dim3(blocks), dim3(64 * waves),
                        smem, st, (const bf16_t*)X, (const bf16_t*)W, Y, y_dt, M, N, K, rope, res);
     return illm_launch_status();
 }
@@ -454,6 +463,8 @@ static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M,
 static const int SK_WAVES_ON_CHIP = 2400;
 // Tiles a block of the tiled gate|up and plain products takes: 0 = by the number of tiles (two
 // from 1024 tiles on), 1 or 2 = forced (tuning).
+static int SK_ONE_SHOT = 1;           // tuning: 0 switches the one-piece-per-wave variant off
+extern "C" void illm_set_skinny_one_shot(int on) { SK_ONE_SHOT = on; }
 static int SK_TILES_PER_BLOCK = 0;
 extern "C" void illm_set_skinny_tiles_per_block(int n) { SK_TILES_PER_BLOCK = (n == 1 || n == 2) ? n : 0; }
 static const int SK_WAVES_ON_CHIP_TILED = 3072;      // from the tiled copy (no staging in LDS)
@@ -543,9 +554,15 @@ extern "C" int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt
     waves = clamp_waves(waves < 1 ? 1 : waves, 1, 1, 4, K);
     SkResidual res = SK_NO_RESIDUAL;
     res.accumulate = 1; res.nw = nw; res.nw_dt = nw_dt; res.xb = (bf16_t*)xb; res.ssq_out = ssq_out;
-    if (use_tiled(Wt, M, K))
+    if (use_tiled(Wt, M, K)) {
+        // a K of at most 8 pieces of 16 k-steps (4096) and few enough tiles that a block has the
+        // chip's compute unit to itself: 8 waves, each with its whole share of K in flight at once
+        if (SK_ONE_SHOT && K <= 8 * 16 * 32 && blocks <= 512 && waves_wanted <= 0)
+            return launch_skinny<1, 1, 16, SK_PLAIN, true, true>(
+                X, Wt, Y, ILLM_F32, M, N, K, (K / 32 + 15) / 16, (hipStream_t)stream, SkRope(), res);
         return launch_skinny<1, 1, 4, SK_PLAIN, true>(X, Wt, Y, ILLM_F32, M, N, K, waves,
                                                       (hipStream_t)stream, SkRope(), res);
+    }
     return launch_skinny<1, 1, 4>(X, W, Y, ILLM_F32, M, N, K, waves, (hipStream_t)stream, SkRope(),
                                   res);
 }
