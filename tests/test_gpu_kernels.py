@@ -392,6 +392,13 @@ def test_products_of_many_rows_are_planned_once_and_stay_right():
     for plan in o._split_candidates(N):                    # every candidate gives the product
         assert all(0 < c < N for c in plan)
         close(o._run_plan(x.to(DEV), w.to(DEV), plan), R.linear(x, w), torch.bfloat16, scale=math.sqrt(K))
+    big = rnd(2048, K, dtype=torch.bfloat16, seed=3)       # many rows: also as two halves
+    plans = o._split_candidates(N, 2048)
+    assert ("rows", 2) in plans and ("rows", 2) not in o._split_candidates(N, 1100)
+    close(o._run_plan(big.to(DEV), w.to(DEV), ("rows", 2)), R.linear(big, w), torch.bfloat16, scale=math.sqrt(K))
+    o._PLANS[(8, N, K)] = ("rows", 2)                      # ragged rows of that class run whole
+    close(o.linear(big[:1900].to(DEV), w.to(DEV)), R.linear(big[:1900], w), torch.bfloat16, scale=math.sqrt(K))
+    del o._PLANS[(8, N, K)]
     o.linear(x.to(DEV), w.to(DEV))
     assert len(o._PLANS) == 1                              # measured once
     o.linear(x[:1000].to(DEV), w.to(DEV))                  # fewer rows than planning is for
