@@ -375,6 +375,31 @@ def test_long_prompt_then_decoding_at_head_size_128(tmp_path_factory, dtype):
     eng.cache.check()
 
 
+def test_decoding_across_a_class_of_lengths(tmp_path_factory):
+    """Decode graphs are captured per class of lengths (up to 1024 keys, 2048, ...), since how
+    attention cuts the keys among blocks is fixed at capture: two sequences decode from 1,010
+    and 1,020 keys to beyond 1,024, through the change of graph."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "D", "bfloat16", max_batch=2, max_seq_len=2048,
+                               max_tokens=2 * 1088)
+    reqs = requests_for(config, [1040, 1050], seed=21)
+    heads = [1010, 1020]
+    slots = [eng.alloc_slot() for _ in reqs]
+    eng.step([StepEntry(s, r[:h], []) for s, r, h in zip(slots, reqs, heads)])
+    got = [[], []]
+    for t in range(30):
+        out = eng.step([StepEntry(s, [r[h + t]], [0]) for s, r, h in zip(slots, reqs, heads)])
+        got[0].append(out[0:1].clone()); got[1].append(out[1:2].clone())
+    assert len(eng.runner._graphs) == 2 and {k[1] for k in eng.runner._graphs} == {1024, 2048}
+    for i, (r, h) in enumerate(zip(reqs, heads)):
+        want = plain(r[:h + 30])[h:h + 30]
+        per = (torch.cat(got[i]).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+        assert float(per.max()) < BUDGET["bfloat16"], f"request {i}: first bad position {h + int((per >= BUDGET['bfloat16']).nonzero()[0])}"
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
+
+
 def test_kernel_timing_reports_every_op(tmp_path_factory):
     from inferllm_amd.kernels.profile import kernel_timing
     eng, plain, config = setup(tmp_path_factory, "A", "bfloat16", use_graphs=False)
