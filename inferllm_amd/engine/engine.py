@@ -42,7 +42,8 @@ class Engine:
     float32 (own multiply-add kernels; no matrix-core or reduced-precision mode).
 
     `decode_copies`: keep a second copy of every matrix in the layout of the few-rows kernels
-    (decoding reads that one, prompts the row-major one); default: if it fits comfortably.
+    (decoding reads that one, prompts the row-major one), or with "thin" of the down projections
+    alone; default: all if they fit comfortably, else the thin ones if those do.
 
     Cache size: `max_tokens` is the most tokens live sequences hold together (each
     rounded up to 64), `max_batch` the most live sequences, `max_seq_len` the longest
@@ -52,7 +53,7 @@ class Engine:
     def __init__(self, config, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  max_batch: int = 8, max_seq_len: Optional[int] = None,
                  max_tokens: Optional[int] = None, use_graphs: bool = True,
-                 poison_freed: bool = False, decode_copies: Optional[bool] = None):
+                 poison_freed: bool = False, decode_copies=None):
         self.config = config
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
@@ -65,11 +66,20 @@ class Engine:
         self.model = DecoderModel(self.spec)
         if decode_copies is None:
             # a second copy of the matrices, laid out for the few-rows kernels of decoding, if it
-            # takes no more than a quarter of the memory that is free now
-            nbytes = sum(t.numel() * t.element_size() for t in tensors.values() if t.dim() == 2)
+            # takes no more than a quarter of the memory that is free now; else of the long thin
+            # ones alone (the down projections) if that takes no more than a third
+            sizes = [(t.numel() * t.element_size(), t.shape) for t in tensors.values() if t.dim() == 2]
             free, _total = torch.cuda.mem_get_info(self.device)
-            decode_copies = self.dtype == torch.bfloat16 and nbytes <= free // 4
-        self.decode_copies = bool(decode_copies) and self.dtype == torch.bfloat16
+            thin = sum(n for n, shape in sizes if shape[1] >= 2 * shape[0])
+            if self.dtype != torch.bfloat16:
+                decode_copies = False
+            elif sum(n for n, _ in sizes) <= free // 4:
+                decode_copies = True
+            else:
+                decode_copies = "thin" if 0 < thin <= free // 3 else False
+        if self.dtype != torch.bfloat16:
+            decode_copies = False
+        self.decode_copies = decode_copies if decode_copies == "thin" else bool(decode_copies)
         ops.DECODE_COPIES = self.decode_copies
         try:
             self.model.load(tensors)

@@ -211,7 +211,10 @@ class Weight:
         return self.plain.dtype
 
 
-DECODE_COPIES = False         # whether `decode_weight` makes the second copy (set by the engine)
+# Whether `decode_weight` makes the second copy (set by the engine): False, True (of every matrix)
+# or "thin" (only of matrices with K >= 2 N, the down projections: where the vendor GEMM is weakest
+# at 17 to 64 rows and `linear_planes` needs the copy; for models whose copies do not all fit).
+DECODE_COPIES = False
 
 
 def _w(w, mode: str = "plain"):
@@ -265,7 +268,8 @@ def decode_weight(w: torch.Tensor, mode: str = "plain", **geometry):
     """The weight as the parts keep it: with a tiled copy for the few-rows kernels if the engine
     asked for decode copies and the matrix allows it, else the tensor itself."""
     if (DECODE_COPIES and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0
-            and w.is_cuda and (mode != "qkv" or geometry.get("hd", 0) % 16 == 0)):
+            and w.is_cuda and (mode != "qkv" or geometry.get("hd", 0) % 16 == 0)
+            and (DECODE_COPIES != "thin" or (mode == "plain" and w.shape[1] >= 2 * w.shape[0]))):
         return Weight(w, tile_weight(w, tile_rows(w.shape[0], mode, **geometry)), mode)
     return w
 

@@ -375,6 +375,27 @@ def test_long_prompt_then_decoding_at_head_size_128(tmp_path_factory, dtype):
     eng.cache.check()
 
 
+def test_decode_copies_of_the_thin_matrices_alone(tmp_path_factory):
+    """`decode_copies="thin"` (what the engine chooses when copies of all matrices do not fit):
+    only the down projections, which have K >= 2 N, get the second copy."""
+    from inferllm_amd import StepEntry
+    from inferllm_amd.kernels import ops
+    eng, plain, config = setup(tmp_path_factory, "B", "bfloat16", decode_copies="thin", max_batch=24)
+    assert eng.decode_copies == "thin"
+    for layer in eng.model.layers:
+        assert isinstance(layer.feed_forward.w_down, ops.Weight) and layer.feed_forward.w_down.mode == "plain"
+        assert not isinstance(layer.feed_forward.w_gate_up, ops.Weight)
+        assert not isinstance(layer.mixer.w_qkv, ops.Weight) and not isinstance(layer.mixer.w_o, ops.Weight)
+    for n in (1, 9, 40):                                  # few-rows kernels, and the split product
+        ids = requests_for(config, [n + 3], seed=30 + n)[0]
+        s = eng.alloc_slot()
+        got = [eng.step([StepEntry(s, ids[:n], list(range(n)))]).clone()]
+        for t in ids[n:]:
+            got.append(eng.step([StepEntry(s, [t], [0])]).clone())
+        assert err(torch.cat(got), plain(ids)) < BUDGET["bfloat16"], n
+        eng.free_slot(s)
+
+
 def test_decoding_across_a_class_of_lengths(tmp_path_factory):
     """Decode graphs are captured per class of lengths (up to 1024 keys, 2048, ...), since how
     attention cuts the keys among blocks is fixed at capture: two sequences decode from 1,010
