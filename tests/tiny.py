@@ -1,7 +1,7 @@
 """Tiny configurations and helpers shared by the tests.
 
-A and B are the two tiny LLaMA shapes of the build's baseline; C adds what those
-two share (another head count, tied embeddings, a head size in steps of 16 with
+A and B are two tiny LLaMA shapes (4 heads of 16 on 4 kv heads; 4 heads of 24 on 2 kv heads);
+C adds what those two lack (another head count, tied embeddings, a head size in steps of 16 with
 8-fold groups).  They differ in every size and constant.
 """
 from __future__ import annotations
