@@ -114,6 +114,15 @@ void illm_set_mid_tiles_per_wave(int n);      // tuning: 1 or 2 (0: by the numbe
 // two when there are at least 1024 tiles).
 void illm_set_skinny_tiles_per_block(int n);
 
+// Tuning and tests: 0 switches off the variant of the residual-adding product in which, for K up
+// to 4096 and at most 512 tiles, 8 waves each take their whole share of K at once (default 1).
+void illm_set_skinny_one_shot(int on);
+
+// Tuning and tests: 0 sends grouped heads of head sizes up to 128 to the decode attention kernel
+// with P.V on the vector units, which larger head sizes use, instead of the one with both
+// products on the matrix cores (default 1).
+void illm_set_gqa_pv_on_matrix_cores(int on);
+
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
 // product, `ssq` included.  waves_wanted: waves per block (0: the default choice).
 int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const void* Wt, void* Y, int y_dt,

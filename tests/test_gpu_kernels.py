@@ -283,6 +283,55 @@ def test_attn_decode_bf16_pages_of_64(nh, nkv, hd, lens, window, nsplit):
         close(got, want, dtype, scale=2)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,lens,window,nsplit", [(32, 8, 128, [650, 90, 3000], 0, 4), (12, 4, 32, [90, 17, 700], 13, 2),
+                                                          (64, 8, 128, [1000, 63], 0, 5), (34, 2, 64, [200, 129], 0, 1)])
+def test_both_grouped_head_decode_kernels_agree(nh, nkv, hd, lens, window, nsplit):
+    """Grouped heads up to head size 128 run with both products on the matrix cores; the kernel
+    with P.V on the vector units (which larger head sizes still use) must give the same."""
+    o = ops()
+    dtype, page = torch.bfloat16, 64
+    ring = (window + page - 2) // page + 1 if window else 0
+    pt, kc, vc, slots, seq_len = paged_case(dtype, nkv, hd, lens, page, ring)
+    qkv = rnd(len(lens), (nh + 2 * nkv) * hd, dtype=dtype, seed=11)
+    args = (qkv.to(DEV), kc.to(DEV), vc.to(DEV), pt.to(DEV), page, ring, slots.to(DEV), seq_len.to(DEV),
+            nh, nkv, hd, 1.0 / math.sqrt(hd), window, nsplit, 4)
+    new = o.attn_decode(*args)
+    try:
+        o._lib().illm_set_gqa_pv_on_matrix_cores(0)
+        old = o.attn_decode(*args)
+    finally:
+        o._lib().illm_set_gqa_pv_on_matrix_cores(1)
+    want = R.attn_decode(qkv, kc, vc, pt, page, ring, slots, seq_len, nh, nkv, hd, 1.0 / math.sqrt(hd), window, nsplit)
+    close(new, want, dtype, scale=2)
+    close(old, want, dtype, scale=2)
+    close(new, old.float(), dtype, scale=2)
+
+
+def test_linear_add_over_a_short_k_in_one_piece_a_wave():
+    """K up to 4096 with at most 512 tiles runs with 8 waves that each take their share of K at
+    once; the looping variant sums in another order and must agree to rounding."""
+    o = ops()
+    for M, N, K in ((8, 4096, 4096), (16, 2048, 1024), (3, 520, 4096), (1, 8192, 2048)):
+        x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
+        nw = (1 + rnd(N, seed=4) * 0.3).to(torch.bfloat16)
+        into = rnd(M, N, seed=3) * 10
+        wc = _plain_copy(w.to(DEV))
+        outs = []
+        for on in (1, 0):
+            try:
+                o._lib().illm_set_skinny_one_shot(on)
+                dev = into.clone().to(DEV)
+                rows = o.linear_add(x.to(DEV), wc, dev, (nw.to(DEV), 1e-5))
+            finally:
+                o._lib().illm_set_skinny_one_shot(1)
+            outs.append((dev, rows))
+        want = into.double() + R.linear(x, w, torch.float64)
+        for dev, rows in outs:
+            torch.testing.assert_close(dev.double().cpu(), want, atol=2e-4 * math.sqrt(K), rtol=1e-5)
+            close(rows.xb, want * nw.double(), torch.bfloat16, scale=float(want.abs().max()))
+            torch.testing.assert_close(rows.ssq.double().sum(1).cpu(), (want ** 2).sum(1), rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("ydt", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 2, 128), (4, 128, 128), (8, 4096, 4096), (1, 32000, 4096), (16, 411, 80),
                                    (17, 100, 1000), (33, 64, 1008), (48, 31, 8), (64, 4096, 11008), (7, 12288, 4096),
