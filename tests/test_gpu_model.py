@@ -375,6 +375,32 @@ def test_long_prompt_then_decoding_at_head_size_128(tmp_path_factory, dtype):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_of_a_hundred_sequences(tmp_path_factory, dtype):
+    """More sequences than any few-rows kernel takes (100: a decode bucket of 128 rows, products
+    by the vendor GEMM in bfloat16): prompts of unequal lengths in one step, then three tokens
+    each; every sequence is compared with the plain implementation."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "B", dtype, max_batch=100, max_seq_len=64)
+    reqs = requests_for(config, [4 + (7 * i) % 13 for i in range(100)], seed=40)
+    heads = [len(r) - 3 for r in reqs]
+    slots = [eng.alloc_slot() for _ in reqs]
+    out = eng.step([StepEntry(s, r[:h], [h - 1]) for s, r, h in zip(slots, reqs, heads)])
+    got = [[out[i:i + 1].clone()] for i in range(100)]
+    for t in range(3):
+        out = eng.step([StepEntry(s, [r[h + t]], [0]) for s, r, h in zip(slots, reqs, heads)])
+        for i in range(100):
+            got[i].append(out[i:i + 1].clone())
+    worst = 0.0
+    for i, (r, h) in enumerate(zip(reqs, heads)):
+        want = plain(r)[h - 1:]
+        worst = max(worst, err(torch.cat(got[i]), want))
+    assert worst < BUDGET[dtype]
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
+
+
 def test_decode_copies_of_the_thin_matrices_alone(tmp_path_factory):
     """`decode_copies="thin"` (what the engine chooses when copies of all matrices do not fit):
     only the down projections, which have K >= 2 N, get the second copy."""
