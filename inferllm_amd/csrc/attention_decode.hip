@@ -141,15 +141,19 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
         const int phys = page_table[(size_t)slot * table_stride + lp];
         const size_t base = (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)hd +
                             (size_t)q * hd + c * 8;
+        // rows beyond the sequence's length are not read (the last tile of a sequence is half
+        // empty on average: 5 % of the bytes at 640 keys)
         uint4 kreg[NI], vreg[NI];
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-            kreg[j] = dim_ok ? ld16_stream(kcache + base + (size_t)j * KPI * hd)
-                             : make_uint4(0, 0, 0, 0);
+            kreg[j] = (dim_ok && k0 + j * KPI + q < len)
+                          ? ld16_stream(kcache + base + (size_t)j * KPI * hd)
+                          : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-            vreg[j] = dim_ok ? ld16_stream(vcache + base + (size_t)j * KPI * hd)
-                             : make_uint4(0, 0, 0, 0);
+            vreg[j] = (dim_ok && k0 + j * KPI + q < len)
+                          ? ld16_stream(vcache + base + (size_t)j * KPI * hd)
+                          : make_uint4(0, 0, 0, 0);
 
         // scores: lane (q, c) ends up owning key k0 + c * KPI + q (if c < NI).  Every lane has a
         // share of NI dot products; instead of NI full reductions over the LPR lanes of a row,
@@ -566,12 +570,15 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
         if (ring > 0) lp %= ring;
         const int phys = page_table[(size_t)slot * table_stride + lp];
         const size_t tile = (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)HD;
+        // rows beyond the sequence's length are not read
         uint4 ka[4][KS], vr[2][8];
 #pragma unroll
         for (int sub = 0; sub < 4; ++sub)
 #pragma unroll
             for (int s = 0; s < KS; ++s)
-                ka[sub][s] = *(const uint4*)(kcache + tile + (size_t)(sub * 16 + r) * HD + s * 32 + q4 * 8);
+                ka[sub][s] = k0 + sub * 16 + r < len
+                                 ? *(const uint4*)(kcache + tile + (size_t)(sub * 16 + r) * HD + s * 32 + q4 * 8)
+                                 : make_uint4(0, 0, 0, 0);
         // V: slot i of half hb is key (2 hb + i / 4) * 16 + 4 q4 + i % 4, the key whose score this
         // k group's lanes get at place i % 4 of sub-tile 2 hb + i / 4
 #pragma unroll
@@ -579,18 +586,19 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int kt = (2 * hb + i / 4) * 16 + 4 * q4 + (i & 3);
-                vr[hb][i] = dim_ok ? *(const uint4*)(vcache + tile + (size_t)kt * HD + r * 8)
-                                   : make_uint4(0, 0, 0, 0);
+                vr[hb][i] = (dim_ok && k0 + kt < len)
+                                ? *(const uint4*)(vcache + tile + (size_t)kt * HD + r * 8)
+                                : make_uint4(0, 0, 0, 0);
             }
-        if (k0 + TK > len || k0 < kf) {
-            // a tile with keys that do not count: their rows may hold anything (NaN too), and a
-            // probability of zero would not undo that
+        if (k0 < kf) {
+            // a tile with keys before the window: their rows may hold anything (NaN too), and a
+            // probability of zero would not undo that (rows beyond the length were not read)
 #pragma unroll
             for (int hb = 0; hb < 2; ++hb)
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int key = k0 + (2 * hb + i / 4) * 16 + 4 * q4 + (i & 3);
-                    if (!(key < len && key >= kf)) vr[hb][i] = make_uint4(0, 0, 0, 0);
+                    if (key < kf) vr[hb][i] = make_uint4(0, 0, 0, 0);
                 }
         }
         // scores of 4 keys per sub-tile for head r
