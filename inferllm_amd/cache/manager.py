@@ -203,6 +203,28 @@ class CacheManager:
         self._len[slot] = new_len
         self._len_dirty = True
 
+    def extend_all(self, items: Sequence[Tuple[int, int, int]]) -> None:
+        """`extend` for every (slot, start_pos, n_tokens) of a step, or for none of them: if the
+        step as a whole does not fit, CacheFull is raised and the cache is as it was."""
+        for g in self.groups:
+            more = 0
+            for slot, start, n in items:
+                more += max(0, g.pages_needed(start + n) - len(g.held.get(slot, ())))
+            if more > g.pool.n_free():
+                raise CacheFull(f"cache full: this step needs {more} more pages of "
+                                f"{g.page_size} tokens, {g.pool.n_free()} of {g.n_pages} are free")
+        for slot, start, n in items:
+            if slot not in self.slots._held:
+                raise CacheError(f"slot {slot} is not held")
+            if start != int(self._len[slot]):
+                raise CacheError(f"slot {slot} holds {int(self._len[slot])} tokens; a step "
+                                 f"starting at {start} does not follow")
+            if start + n > self.max_seq_len:
+                raise CacheFull(f"sequence would reach {start + n} tokens; the limit is "
+                                f"{self.max_seq_len}")
+        for slot, start, n in items:
+            self.extend(slot, start, n)
+
     def upload(self, lengths: bool = True) -> None:
         """Bring page tables (and, unless `lengths` is False, the per-slot lengths) on the
         device up to date with the host.  Steps of single tokens carry their sequences'

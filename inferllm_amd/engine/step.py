@@ -140,8 +140,7 @@ class StepRunner:
                     or device_tokens.shape != (len(entries),)):
                 raise StepError(f"device_tokens must be int32 [{len(entries)}] on {self.device}")
         starts = [self.cache.length(e.slot) for e in entries]
-        for e, s in zip(entries, starts):
-            self.cache.extend(e.slot, s, len(e.tokens))
+        self.cache.extend_all([(e.slot, s, len(e.tokens)) for e, s in zip(entries, starts)])
         self.cache.upload(lengths=prefill)
         if prefill:
             return self._prefill(entries)

@@ -92,6 +92,25 @@ def test_room_is_counted_in_pages_of_64():
     m.check()
 
 
+def test_a_step_that_does_not_fit_leaves_the_cache_as_it_was():
+    m = manager(max_tokens=64 * 3, max_slots=3)
+    a, b, c = m.alloc_slot(), m.alloc_slot(), m.alloc_slot()
+    with pytest.raises(CacheFull, match="needs 4 more pages"):
+        m.extend_all([(a, 0, 64), (b, 0, 65), (c, 0, 1)])      # a and b alone would fit
+    assert [m.length(x) for x in (a, b, c)] == [0, 0, 0]
+    assert all(g.pool.n_held() == 0 for g in m.groups)
+    m.extend_all([(a, 0, 64), (b, 0, 64), (c, 0, 1)])
+    with pytest.raises(CacheFull, match="needs 2 more pages"):
+        m.extend_all([(a, 64, 1), (b, 64, 1), (c, 1, 1)])      # one of the three would fit
+    assert [m.length(x) for x in (a, b, c)] == [64, 64, 1]
+    with pytest.raises(CacheError, match="does not follow"):
+        m.extend_all([(c, 1, 1), (a, 63, 1)])
+    assert m.length(c) == 1
+    m.extend_all([(c, 1, 1)])
+    assert m.length(c) == 2
+    m.check()
+
+
 def test_groups_with_different_needs_have_their_own_storage():
     lines = {0: KVSpec("full", 2, 16), 1: KVSpec("window", 2, 16, window=70), 2: KVSpec("full", 4, 8),
              3: KVSpec("window", 2, 16, window=70)}
