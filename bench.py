@@ -92,7 +92,8 @@ def main() -> int:
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     dev = "cuda:0"
     max_b = max(args.batch, 1 if args.no_points else 64)
-    room = max(max_b * 1024, 4096)
+    per_seq = -(-(args.prompt + args.steps + args.warmup + 2) // 64) * 64     # whole cache pages
+    room = max(max_b * max(per_seq, 1024), 4096)
     t0 = time.time()
     eng = Engine.from_random(cfg, seed=0, dtype=args.dtype, device=dev, max_batch=max_b,
                              max_seq_len=ctx_len, max_tokens=room)
