@@ -1,4 +1,4 @@
-// Y[M, N] = X[M, K] . W[N, K]^T for 17 to 64 rows (decoding larger batches), bfloat16 operands,
+// Y[M, N] = X[M, K] . W[N, K]^T for up to 64 rows (decoding larger batches), bfloat16 operands,
 // float32 accumulation on the matrix cores, from the tiled copy of W
 // ([tile of 16 rows][K / 32][16 rows][32 k], see gemm_skinny.hip).
 //

@@ -15,8 +15,9 @@ uses a vendor GEMM too (cublasSgemm, src/kern/gpu/kernel_gpu.cu:420-435).
 Four things ride on the products.  `Weight`: a matrix with a second copy in the
 kernels' own tile order (`decode_weight`).  `linear_add` / `NormedRows`: the
 residual add in the product's epilogue and the RMS norm that follows it taken by
-the next product (up to 16 rows).  `linear_planes`: the product of 17 to 64 rows
-with a long thin matrix, K cut into ranges whose float32 planes `add_rmsnorm` adds.
+the next product (up to 16 rows).  `linear_planes`: the product of up to 64 rows (from
+17, or from fewer where that is measured to pay) with a long thin matrix, K cut into
+ranges whose float32 planes `add_rmsnorm` adds.
 `_planned_matmul`: products of many rows measured once per shape, whole against
 cut along the output columns.
 """
@@ -360,21 +361,72 @@ def linear_add(x: torch.Tensor, w, into: torch.Tensor, norm=None,
     return NormedRows(into, weight, eps, act_dtype, xb, ssq)
 
 
-MID_MIN_ROWS = 17        # rows from which `linear_planes` stands in for the vendor GEMM
 MID_MAX_ROWS = 64
 MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the norm that adds the
                          # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
                          # K >= 2 N (the down projection) and the same time when K = N
+MEASURE_PLANES = True    # whether `linear_planes_pays` may measure a shape it has not seen
+_PLANES_FROM: dict = {}  # (N, K) -> fewest rows (1, 5, 9, 13 or 17) from which the planes pay
 
 
 def linear_planes_fits(x, w) -> bool:
-    """Whether `linear_planes` takes these operands: 17 to 64 bfloat16 rows and a matrix with a
+    """Whether `linear_planes` takes these operands: up to 64 bfloat16 rows and a matrix with a
     decode copy in plain tile order that has few rows for its length (K >= 2 N)."""
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == "plain"
             and isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and x.dim() == 2
-            and MID_MIN_ROWS <= x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.plain.shape[1]
+            and 1 <= x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.plain.shape[1]
             and w.plain.shape[0] % 4 == 0 and w.plain.shape[0] <= MID_MAX_COLS
             and w.plain.shape[1] >= 2 * w.plain.shape[0])
+
+
+def _measure_planes_from(w: "Weight") -> int:
+    """Fewest rows from which `linear_planes` and the norm that adds its planes take less time
+    than `linear_add` (whose norm the next product takes), measured at 16, 12, 8 and 4 rows."""
+    N, K = w.plain.shape
+    dev = w.plain.device
+    x = torch.zeros((SKINNY_BEST_ROWS, K), dtype=torch.bfloat16, device=dev)
+    into = torch.zeros((SKINNY_BEST_ROWS, N), dtype=torch.float32, device=dev)
+    nw = torch.ones(N, dtype=torch.bfloat16, device=dev)
+
+    def timed(fn) -> float:
+        fn()
+        fn()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(8):
+            fn()
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end)
+
+    first = SKINNY_BEST_ROWS + 1
+    for rows in (16, 12, 8, 4):
+        xs, dst = x[:rows], into[:rows]
+        t_add = timed(lambda: linear_add(xs, w, dst, (nw, 1e-5)))
+        t_planes = timed(lambda: add_rmsnorm(dst, linear_planes(xs, w), nw, 1e-5, torch.bfloat16))
+        if t_planes >= 0.97 * t_add:              # the planes have to pay clearly
+            break
+        first = rows - 3
+    return first
+
+
+def linear_planes_pays(x, w) -> bool:
+    """Whether the planes are the faster way for these operands (which `linear_planes_fits`).
+    Beyond the few-rows kernels' 16 rows always.  Up to 16 rows `linear_add` reads X once per
+    block of W rows, so its time grows with the rows, and a matrix whose tiles do not fill the
+    chip evenly is slow at any (measured: LLaMA-2-7B's down projection 23.3 against 21.7 us at
+    16 rows, the 70B's 105 against 77, a 5120 x 13824 one 34 against 30 at 4 rows): measured
+    once per shape, outside graph capture."""
+    rows = x.shape[0]
+    if rows > SKINNY_BEST_ROWS:
+        return True
+    key = tuple(w.plain.shape)
+    first = _PLANES_FROM.get(key)
+    if first is None:
+        if not MEASURE_PLANES or torch.cuda.is_current_stream_capturing():
+            return False
+        first = _PLANES_FROM[key] = _measure_planes_from(w)
+    return rows >= first
 
 
 def linear_planes(x: torch.Tensor, w: "Weight", splits: int = 0) -> torch.Tensor:

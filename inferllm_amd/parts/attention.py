@@ -96,10 +96,11 @@ class Attention(Mixer):
             o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
                                 ctx.seq_slot, ctx.seq_len, nh, nkv, hd, self.scale, window,
                                 nsplit, waves)
+        if (next_norm is not None and getattr(next_norm, "adds_planes", False)
+                and ops.linear_planes_fits(o, self.w_o) and ops.linear_planes_pays(o, self.w_o)):
+            return ops.linear_planes(o, self.w_o)
         if residual is not None and ops.linear_add_fits(o, self.w_o, residual):
             return ops.linear_add(o, self.w_o, residual,
                                   next_norm.rms_params() if next_norm is not None else None,
                                   ctx.act_dtype)
-        if next_norm is not None and getattr(next_norm, "adds_planes", False) and ops.linear_planes_fits(o, self.w_o):
-            return ops.linear_planes(o, self.w_o)
         return ops.linear(o, self.w_o)

@@ -40,10 +40,11 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, ctx: StepContext, residual=None, next_norm=None):
         a = ops.gate_up_silu(h, self.w_gate_up)
+        if (next_norm is not None and getattr(next_norm, "adds_planes", False)
+                and ops.linear_planes_fits(a, self.w_down) and ops.linear_planes_pays(a, self.w_down)):
+            return ops.linear_planes(a, self.w_down)
         if residual is not None and ops.linear_add_fits(a, self.w_down, residual):
             return ops.linear_add(a, self.w_down, residual,
                                   next_norm.rms_params() if next_norm is not None else None,
                                   ctx.act_dtype)
-        if next_norm is not None and getattr(next_norm, "adds_planes", False) and ops.linear_planes_fits(a, self.w_down):
-            return ops.linear_planes(a, self.w_down)
         return ops.linear(a, self.w_down)

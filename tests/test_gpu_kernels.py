@@ -519,14 +519,15 @@ def _plain_copy(w):
     return o.Weight(w, o.tile_weight(w, o.tile_rows(w.shape[0], "plain")), "plain")
 
 
-# rows 17..64 in every count of 16-row tiles; N with a last tile of 4 rows, with fewer tiles than
+# rows in every count of 16-row tiles; N with a last tile of 4 rows, with fewer tiles than
 # a block's waves, with tiles beyond a multiple of 4; K of one piece, of a partial last piece
 @pytest.mark.parametrize("tiles_per_wave", [0, 1, 2])
 @pytest.mark.parametrize("M,N,K,splits", [(17, 40, 96, 0), (33, 100, 224, 0), (64, 4096, 11008, 0),
                                           (50, 84, 1184, 5), (48, 20, 64, 1), (31, 72, 352, 3),
-                                          (64, 36, 2048, 16), (20, 8192, 16384, 0)])
+                                          (64, 36, 2048, 16), (20, 8192, 16384, 0),
+                                          (1, 40, 96, 0), (7, 100, 224, 2), (16, 4096, 11008, 0)])
 def test_linear_planes(M, N, K, splits, tiles_per_wave):
-    """The product for 17 to 64 rows, K cut into ranges: the planes add up to x . w^T, and what
+    """The product for up to 64 rows, K cut into ranges: the planes add up to x . w^T, and what
     `add_rmsnorm` makes of them is the residual add and norm of the product."""
     o = ops()
     if N >= 8192 and tiles_per_wave:
@@ -558,7 +559,7 @@ def test_linear_planes_refuses_what_it_does_not_take():
     x = rnd(20, 256, dtype=torch.bfloat16).to(DEV)
     assert o.linear_planes_fits(x, _plain_copy(w))
     assert not o.linear_planes_fits(x, w)                                  # no decode copy
-    assert not o.linear_planes_fits(x[:16], _plain_copy(w))                # the few-rows kernels' rows
+    assert o.linear_planes_fits(x[:16], _plain_copy(w)) and o.linear_planes_pays(x, _plain_copy(w))
     assert not o.linear_planes_fits(rnd(65, 256, dtype=torch.bfloat16).to(DEV), _plain_copy(w))
     assert not o.linear_planes_fits(x.float(), _plain_copy(w))
     wide = rnd(256, 256, dtype=torch.bfloat16).to(DEV)                      # K < 2 N: the vendor GEMM's

@@ -113,6 +113,55 @@ def test_steps_of_17_to_64_rows(tmp_path_factory, monkeypatch):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("first", [1, 5, 17])
+def test_few_rows_through_the_planes_where_they_pay(tmp_path_factory, monkeypatch, first):
+    """From how few rows the down projection goes through planes is measured per shape; here it
+    is pinned (1: every step; 5: steps of 5 rows or more; 17: never below 17), and prompts of 3
+    and 9 tokens and six sequences decoding together must come out as the plain model's in each."""
+    from inferllm_amd import StepEntry
+    from inferllm_amd.kernels import ops
+    eng, plain, config = setup(tmp_path_factory, "B", "bfloat16", max_batch=8, decode_copies=True)
+    shape = (config["hidden_size"], config["intermediate_size"])
+    monkeypatch.setitem(ops._PLANES_FROM, shape, first)
+    calls = []
+    real = ops.linear_planes
+    monkeypatch.setattr(ops, "linear_planes", lambda x, w, *a: calls.append(x.shape[0]) or real(x, w, *a))
+    for n in (3, 9):
+        ids = requests_for(config, [n], seed=n)[0]
+        s = eng.alloc_slot()
+        assert err(eng.step([StepEntry(s, ids, list(range(n)))]), plain(ids)) < BUDGET["bfloat16"]
+        eng.free_slot(s)
+    reqs = requests_for(config, [4, 9, 3, 7, 5, 3], seed=8)
+    slots = [eng.alloc_slot() for _ in reqs]
+    got = [[eng.step([StepEntry(s, r[:-2], list(range(len(r) - 2)))])] for s, r in zip(slots, reqs)]
+    for t in (2, 1):
+        out = eng.step([StepEntry(s, [r[-t]], [0]) for s, r in zip(slots, reqs)])
+        for i in range(len(reqs)):
+            got[i].append(out[i:i + 1].clone())
+    for i, r in enumerate(reqs):
+        assert err(torch.cat(got[i]), plain(r)) < BUDGET["bfloat16"], i
+    for s in slots:
+        eng.free_slot(s)
+    if first == 17:
+        assert not calls
+    else:
+        assert calls and min(calls) >= first and (first > 1 or 1 in calls or 2 in calls)
+
+
+def test_the_rows_from_which_planes_pay_are_measured_once_per_shape():
+    from inferllm_amd.kernels import ops
+    m = torch.randn(128, 512, device="cuda", dtype=torch.bfloat16)
+    w = ops.Weight(m, ops.tile_weight(m, ops.tile_rows(128, "plain")), "plain")
+    ops._PLANES_FROM.pop((128, 512), None)
+    x = torch.zeros(8, 512, device="cuda", dtype=torch.bfloat16)
+    assert ops.linear_planes_fits(x, w)
+    a = ops.linear_planes_pays(x, w)
+    assert ops._PLANES_FROM[(128, 512)] in (1, 5, 9, 13, 17)
+    assert a == (8 >= ops._PLANES_FROM[(128, 512)])
+    assert ops.linear_planes_pays(torch.zeros(17, 512, device="cuda", dtype=torch.bfloat16), w)
+    ops._PLANES_FROM.pop((128, 512), None)
+
+
 @pytest.mark.parametrize("copies", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C", "D"])
