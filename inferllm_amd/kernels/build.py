@@ -13,6 +13,7 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -142,6 +143,39 @@ def build(verbose: bool = True, force: bool = True) -> str:
     return os.path.join(out_dir, LIB_NAME)
 
 
+_C_TYPES = {"int": ctypes.c_int, "float": ctypes.c_float, "double": ctypes.c_double,
+            "size_t": ctypes.c_size_t, "unsigned": ctypes.c_uint, "uint32_t": ctypes.c_uint32,
+            "int32_t": ctypes.c_int32, "uint64_t": ctypes.c_uint64, "int64_t": ctypes.c_int64,
+            "unsigned long long": ctypes.c_ulonglong, "long long": ctypes.c_longlong}
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    """Give every entry point of api.h its argument and result types, so that a call with the
+    wrong number or kind of arguments raises here instead of reading garbage over there."""
+    with open(os.path.join(CSRC, "api.h")) as f:
+        text = re.sub(r"//[^\n]*", "", f.read())
+    for ret, name, params in re.findall(r"\b(int|void)\s+(illm_\w+)\s*\(([^)]*)\)\s*;", text):
+        types = []
+        for prm in (p.strip() for p in params.split(",")):
+            if not prm or prm == "void":
+                continue
+            if "*" in prm:
+                types.append(ctypes.c_void_p)
+                continue
+            ctype = " ".join(w for w in prm.split()[:-1] if w != "const")
+            if ctype not in _C_TYPES:
+                raise KernelLibraryError(f"api.h: {name} has a parameter of type {ctype!r} that "
+                                         "the loader does not know")
+            types.append(_C_TYPES[ctype])
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            raise KernelLibraryError(f"{LIB_NAME} lacks {name}, which api.h declares: "
+                                     "the library is not the one these sources build") from None
+        fn.argtypes = types
+        fn.restype = ctypes.c_int if ret == "int" else None
+
+
 def library() -> ctypes.CDLL:
     """The loaded kernel library; built first if no current build exists."""
     global _lib
@@ -150,9 +184,11 @@ def library() -> ctypes.CDLL:
             return _lib
         path = build(verbose=True, force=False)
         try:
-            _lib = ctypes.CDLL(path)
+            lib = ctypes.CDLL(path)
         except OSError as e:
             raise KernelLibraryError(f"cannot load {path}: {e}") from None
+        _declare(lib)
+        _lib = lib
         return _lib
 
 

@@ -34,6 +34,20 @@ def rnd(*shape, dtype=torch.float32, seed=0, std=1.0):
     return (torch.randn(*shape, generator=g) * std).to(dtype)
 
 
+def test_every_entry_point_is_declared_and_a_wrong_call_raises():
+    """The loader gives each function of api.h its argument types: a call with too few arguments
+    or with a float where a size is meant raises instead of launching on garbage."""
+    import ctypes
+    lib = ops()._lib()
+    assert lib.illm_version.argtypes == [] and lib.illm_embed.argtypes[-1] is ctypes.c_void_p
+    with pytest.raises(TypeError):
+        lib.illm_version(1)
+    with pytest.raises(TypeError):
+        lib.illm_silu_mul(None, None, 0, 4)
+    with pytest.raises(ctypes.ArgumentError):
+        lib.illm_silu_mul(None, None, 0, 4.5, 8, None)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("V,E,ids", [(10, 128, [1, 9, 3, 3]), (411, 80, [0, 410, 7]), (1000, 4100, [999])])
 def test_embed(dtype, V, E, ids):
