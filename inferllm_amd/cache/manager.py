@@ -189,7 +189,7 @@ class CacheManager:
     # ------------------------------------------------------------ steps
     def extend(self, slot: int, start_pos: int, n_tokens: int) -> None:
         """Make room for `n_tokens` more tokens of `slot`, which must now hold `start_pos`."""
-        if slot not in self.slots._held:
+        if not self.slots.holds(slot):
             raise CacheError(f"slot {slot} is not held")
         have = int(self._len[slot])
         if start_pos != have:
@@ -214,7 +214,7 @@ class CacheManager:
                 raise CacheFull(f"cache full: this step needs {more} more pages of "
                                 f"{g.page_size} tokens, {g.pool.n_free()} of {g.n_pages} are free")
         for slot, start, n in items:
-            if slot not in self.slots._held:
+            if not self.slots.holds(slot):
                 raise CacheError(f"slot {slot} is not held")
             if start != int(self._len[slot]):
                 raise CacheError(f"slot {slot} holds {int(self._len[slot])} tokens; a step "

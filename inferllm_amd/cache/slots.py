@@ -55,6 +55,9 @@ class FreeList:
     def n_free(self) -> int:
         return len(self._free)
 
+    def holds(self, i: int) -> bool:
+        return i in self._held
+
     def n_held(self) -> int:
         return len(self._held)
 
