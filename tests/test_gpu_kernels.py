@@ -205,7 +205,9 @@ def test_attn_prefill(dtype, nh, nkv, hd, lens, window):
 
 @pytest.mark.parametrize("nh,nkv,hd,lens,window", [
     (4, 4, 128, [300, 129, 128, 1], 0), (8, 1, 64, [257, 64], 0), (3, 3, 96, [200], 0), (6, 2, 32, [127, 130], 0),
-    (2, 1, 160, [70], 0), (4, 2, 128, [400], 100), (2, 2, 64, [333, 5], 64), (5, 5, 224, [66], 0), (2, 2, 192, [129], 7)])
+    (2, 1, 160, [70], 0), (4, 2, 128, [400], 100), (2, 2, 64, [333, 5], 64), (5, 5, 224, [66], 0), (2, 2, 192, [129], 7),
+    # more blocks than the chip holds at once (heaviest first, not paired), and a long sequence
+    (32, 8, 128, [600, 130, 577, 64], 0), (2, 1, 128, [2500, 40], 0)])
 def test_attn_prefill_mfma(nh, nkv, hd, lens, window):
     """The matrix-core kernel over several blocks of 128 query rows and tiles of 64 keys."""
     dtype = torch.bfloat16
@@ -271,7 +273,9 @@ def test_attn_decode(dtype, nh, nkv, hd, lens, window, nsplit):
     (8, 1, 64, [1000], 0, 32), (6, 2, 24, [5, 11, 130], 0, 2), (16, 1, 256, [257, 31], 0, 2),
     (5, 5, 96, [130, 520], 70, 5), (12, 4, 32, [90, 17, 700], 13, 2), (3, 3, 8, [129], 0, 1),
     (20, 2, 48, [333], 0, 4), (64, 8, 128, [1000, 63], 0, 5), (32, 8, 64, [129], 0, 1), (6, 3, 96, [70, 700], 0, 3),
-    (34, 2, 32, [200], 0, 2), (8, 2, 160, [90, 300], 50, 2), (10, 5, 224, [65], 0, 1)])
+    (34, 2, 32, [200], 0, 2), (8, 2, 160, [90, 300], 50, 2), (10, 5, 224, [65], 0, 1),
+    # long contexts, the most splits, both kernels (plain and grouped heads)
+    (8, 8, 128, [8192, 16001], 0, 16), (16, 2, 128, [12000, 5], 0, 16)])
 def test_attn_decode_bf16_pages_of_64(nh, nkv, hd, lens, window, nsplit):
     """The fast bfloat16 kernel (pages of 64 rows, as the engine's cache has them); stale rows
     of the pages are NaN and must not leak into the result."""
