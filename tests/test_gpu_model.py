@@ -424,6 +424,31 @@ def test_long_prompt_then_decoding_at_head_size_128(tmp_path_factory, dtype):
     eng.cache.check()
 
 
+def test_a_context_beyond_4096_beside_a_short_one(tmp_path_factory):
+    """A prompt of 4,300 tokens and one of 70 in one step, then six tokens each: the long
+    sequence's keys lie in the class of lengths up to 8,192, the most splits, and rotation
+    angles at positions that a table of 4,096 would not hold."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "E", "bfloat16", max_batch=2, max_seq_len=8192,
+                               max_tokens=4480 + 128)
+    reqs = requests_for(config, [4306, 76], seed=3)
+    wants = [plain(r) for r in reqs]
+    slots = [eng.alloc_slot() for _ in reqs]
+    probes = [[0, 63, 64, 2047, 2048, 4095, 4096, 4299], [0, 69]]
+    got = eng.step([StepEntry(s, r[:-6], p) for s, r, p in zip(slots, reqs, probes)])
+    at = 0
+    for w, p in zip(wants, probes):
+        assert err(got[at:at + len(p)], w[p]) < BUDGET["bfloat16"]
+        at += len(p)
+    for t in range(6, 0, -1):
+        out = eng.step([StepEntry(s, [r[-t]], [0]) for s, r in zip(slots, reqs)])
+        for i, (w, r) in enumerate(zip(wants, reqs)):
+            assert err(out[i:i + 1], w[len(r) - t:len(r) - t + 1]) < BUDGET["bfloat16"], (i, t)
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_batch_of_a_hundred_sequences(tmp_path_factory, dtype):
     """More sequences than any few-rows kernel takes (100: a decode bucket of 128 rows, products

@@ -2,7 +2,8 @@
 
 A and B are two tiny LLaMA shapes (4 heads of 16 on 4 kv heads; 4 heads of 24 on 2 kv heads);
 C adds what those two lack (another head count, tied embeddings, a head size in steps of 16 with
-8-fold groups).  They differ in every size and constant.
+8-fold groups); D has the head size and grouping of the large models, E positions beyond 4,096.
+They differ in every size and constant.
 """
 from __future__ import annotations
 
@@ -32,7 +33,14 @@ TINY_D = {"architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermedia
           "head_dim": 128, "vocab_size": 1000, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
           "max_position_embeddings": 4096, "tie_word_embeddings": False,
           "bos_token_id": 1, "eos_token_id": 2}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+# positions beyond 4,096: one layer of two heads of 128 on one kv head, so that the plain model
+# can afford thousands of tokens
+TINY_E = {"architectures": ["LlamaForCausalLM"], "hidden_size": 256, "intermediate_size": 300,
+          "num_hidden_layers": 1, "num_attention_heads": 2, "num_key_value_heads": 1,
+          "head_dim": 128, "vocab_size": 500, "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+          "max_position_embeddings": 8192, "tie_word_embeddings": False,
+          "bos_token_id": 1, "eos_token_id": 2}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
 
 
 def make_model_dir(tmp_path, config: dict, seed: int, dtype=torch.float32, gain: float = 1.0) -> str:
