@@ -366,6 +366,8 @@ MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the no
                          # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
                          # K >= 2 N (the down projection) and the same time when K = N
 MEASURE_PLANES = True    # whether `linear_planes_pays` may measure a shape it has not seen
+PLANES_MIN_ELEMENTS = 1 << 22   # smaller matrices are not measured (both ways take a few
+                                # microseconds and the clock would decide): no planes below 17 rows
 _PLANES_FROM: dict = {}  # (N, K) -> fewest rows (1, 5, 9, 13 or 17) from which the planes pay
 
 
@@ -383,6 +385,8 @@ def _measure_planes_from(w: "Weight") -> int:
     """Fewest rows from which `linear_planes` and the norm that adds its planes take less time
     than `linear_add` (whose norm the next product takes), measured at 16, 12, 8 and 4 rows."""
     N, K = w.plain.shape
+    if N * K < PLANES_MIN_ELEMENTS:
+        return SKINNY_BEST_ROWS + 1
     dev = w.plain.device
     x = torch.zeros((SKINNY_BEST_ROWS, K), dtype=torch.bfloat16, device=dev)
     into = torch.zeros((SKINNY_BEST_ROWS, N), dtype=torch.float32, device=dev)

@@ -150,16 +150,18 @@ def test_few_rows_through_the_planes_where_they_pay(tmp_path_factory, monkeypatc
 
 def test_the_rows_from_which_planes_pay_are_measured_once_per_shape():
     from inferllm_amd.kernels import ops
-    m = torch.randn(128, 512, device="cuda", dtype=torch.bfloat16)
-    w = ops.Weight(m, ops.tile_weight(m, ops.tile_rows(128, "plain")), "plain")
-    ops._PLANES_FROM.pop((128, 512), None)
-    x = torch.zeros(8, 512, device="cuda", dtype=torch.bfloat16)
-    assert ops.linear_planes_fits(x, w)
-    a = ops.linear_planes_pays(x, w)
-    assert ops._PLANES_FROM[(128, 512)] in (1, 5, 9, 13, 17)
-    assert a == (8 >= ops._PLANES_FROM[(128, 512)])
-    assert ops.linear_planes_pays(torch.zeros(17, 512, device="cuda", dtype=torch.bfloat16), w)
-    ops._PLANES_FROM.pop((128, 512), None)
+    for shape, measured in (((128, 512), False), ((1024, 4096), True)):
+        m = torch.randn(*shape, device="cuda", dtype=torch.bfloat16)
+        w = ops.Weight(m, ops.tile_weight(m, ops.tile_rows(shape[0], "plain")), "plain")
+        ops._PLANES_FROM.pop(shape, None)
+        x = torch.zeros(8, shape[1], device="cuda", dtype=torch.bfloat16)
+        assert ops.linear_planes_fits(x, w)
+        a = ops.linear_planes_pays(x, w)
+        first = ops._PLANES_FROM[shape]
+        assert first in (1, 5, 9, 13, 17) and (measured or first == 17)    # small ones: never
+        assert a == (8 >= first)
+        assert ops.linear_planes_pays(torch.zeros(17, shape[1], device="cuda", dtype=torch.bfloat16), w)
+        ops._PLANES_FROM.pop(shape, None)
 
 
 @pytest.mark.parametrize("copies", [True, False])
