@@ -24,7 +24,7 @@ The reference keeps, per attention op, two tensors [n_ctx, embd] and a cursor
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch

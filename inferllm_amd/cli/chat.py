@@ -109,7 +109,7 @@ def main(argv=None) -> int:
 
     import json
 
-    from .. import Engine, load_config
+    from .. import Engine
     from ..config import config_from_dict
 
     seed = args.seed if args.seed >= 0 else int(time.time())
@@ -120,7 +120,6 @@ def main(argv=None) -> int:
             config = config_from_dict(json.load(f))
         eng = Engine.from_random(config, seed=args.weights_seed, **kw)
     else:
-        config = load_config(args.model)
         eng = Engine.from_pretrained(args.model, **kw)
     if args.mtype is not None:
         family = {"LlamaForCausalLM": ("llama", "llama2")}.get(eng.spec.architecture, ())

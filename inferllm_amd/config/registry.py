@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import json
 import os
-from typing import Callable, Dict, Type
+from typing import Callable, Dict
 
 
 class ConfigError(ValueError):

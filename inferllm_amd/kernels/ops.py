@@ -24,7 +24,6 @@ cut along the output columns.
 from __future__ import annotations
 
 import ctypes
-import math
 from typing import Optional
 
 import torch

@@ -2,8 +2,7 @@
 encoding turns it into a change of q and k (rotary) or does nothing."""
 from __future__ import annotations
 
-import math
-from typing import Dict, Optional, Tuple
+from typing import Dict, Tuple
 
 import torch
 

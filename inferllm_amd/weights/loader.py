@@ -15,7 +15,7 @@ int32.  An engine that runs in float32 widens every floating tensor to float32.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Iterable, List, Optional, Tuple
+from typing import Dict, Iterable, List, Tuple
 
 import torch
 
