@@ -101,7 +101,7 @@ int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y,
 int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M, int N,
                               int K, int ntb, int u, int waves, void* stream);
 
-// Y = X[M, K] . W[N, K]^T for M up to 64 (meant for 17..64) from the tiled copy Wt of W, K a
+// Y = X[M, K] . W[N, K]^T for M up to 128 (64 rows a launch) from the tiled copy Wt of W, K a
 // multiple of 32, X shared by a block's waves through LDS.  splits == 1: Y is [M, N] of y_dt;
 // splits > 1: K is cut into that many ranges and Y is float32 [splits][M][N], the planes to be
 // added by the caller (illm_add_rmsnorm takes them).  illm_gemm_mid_splits: the splits to use.

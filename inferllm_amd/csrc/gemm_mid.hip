@@ -1,4 +1,4 @@
-// Y[M, N] = X[M, K] . W[N, K]^T for up to 64 rows (decoding larger batches), bfloat16 operands,
+// Y[M, N] = X[M, K] . W[N, K]^T for up to 64 rows a launch (decoding larger batches), bfloat16 operands,
 // float32 accumulation on the matrix cores, from the tiled copy of W
 // ([tile of 16 rows][K / 32][16 rows][32 k], see gemm_skinny.hip).
 //
@@ -27,7 +27,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 template <int MT, int NTB>
 __global__ void __launch_bounds__(256)
 gemm_mid_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, void* __restrict__ Y,
-                int y_dt, int M, int N, int K, int pieces_per_split) {
+                int y_dt, int M, int N, int K, int pieces_per_split, size_t plane_stride) {
     __shared__ uint4 xs[2][MT * 256];    // [buffer][row][16 units of 8 k]
     const int lane = threadIdx.x & 63, wave = wave_index();
     const int r = lane & 15, q = lane >> 4;
@@ -118,7 +118,7 @@ gemm_mid_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, voi
     // acc[nt][mt][i] = sum for X row mt * 16 + r and W row (tile0 + nt) * 16 + 4 q + i
     const bool planes = gridDim.y > 1;
     const int dt = planes ? ILLM_F32 : y_dt;
-    const size_t plane = planes ? (size_t)blockIdx.y * M * N : 0;
+    const size_t plane = planes ? (size_t)blockIdx.y * plane_stride : 0;
 #pragma unroll
     for (int nt = 0; nt < NTB; ++nt) {
         if (!tile_ok[nt]) continue;
@@ -171,12 +171,13 @@ extern "C" int illm_gemm_mid_splits(int N, int K) {
     return (pieces + per - 1) / per;
 }
 
-// Takes bfloat16 X [M, K] with M in 1..64 and the tiled copy Wt of W [N, K], K a multiple of
-// 32.  splits == 1: Y is [M, N] of y_dt.  splits > 1: Y is float32 [splits][M][N], whose planes
-// the caller adds up.  Otherwise ILLM_ERR_ARG.
+// Takes bfloat16 X [M, K] with M in 1..128 (more than 64 rows: 64 at a time, W read again for
+// each) and the tiled copy Wt of W [N, K], K a multiple of 32.  splits == 1: Y is [M, N] of y_dt.
+// splits > 1: Y is float32 [splits][M][N], whose planes the caller adds up.  Otherwise
+// ILLM_ERR_ARG.
 extern "C" int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M, int N,
                                   int K, int splits, void* stream) {
-    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 32) || splits < 1 || !illm_dtype_ok(y_dt) ||
+    if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K % 32) || splits < 1 || !illm_dtype_ok(y_dt) ||
         !X || !Wt || !Y)
         return ILLM_ERR_ARG;
     const int pieces = (K / 32 + MID_PIECE_STEPS - 1) / MID_PIECE_STEPS;
@@ -184,14 +185,26 @@ extern "C" int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_
     const int per = (pieces + splits - 1) / splits;
     const dim3 grid(mid_blocks_x(N), splits);
     hipStream_t st = (hipStream_t)stream;
-    const int mt = (M + 15) / 16, ntb = mid_ntb(N);
+    const int ntb = mid_ntb(N);
+    const size_t y_elem = (splits > 1 || y_dt == ILLM_F32) ? 4 : 2;
+    const size_t plane_stride = (size_t)M * N;
+    for (int m0 = 0; m0 < M; m0 += 64) {
+        const int rows = M - m0 < 64 ? M - m0 : 64;
+        const int mt = (rows + 15) / 16;
+        const bf16_t* x = (const bf16_t*)X + (size_t)m0 * K;
+        void* y = (char*)Y + (size_t)m0 * N * y_elem;
+        bool launched = false;
 #define GO(MT_, NTB_)                                                                         \
-    if (mt == MT_ && ntb == NTB_) {                                                           \
-        hipLaunchKernelGGL((gemm_mid_kernel<MT_, NTB_>), grid, dim3(256), 0, st,              \
-                           (const bf16_t*)X, (const bf16_t*)Wt, Y, y_dt, M, N, K, per);       \
-        return illm_launch_status();                                                          \
-    }
-    GO(1, 1) GO(2, 1) GO(3, 1) GO(4, 1) GO(1, 2) GO(2, 2) GO(3, 2) GO(4, 2)
+        if (mt == MT_ && ntb == NTB_) {                                                       \
+            hipLaunchKernelGGL((gemm_mid_kernel<MT_, NTB_>), grid, dim3(256), 0, st, x,       \
+                               (const bf16_t*)Wt, y, y_dt, rows, N, K, per, plane_stride);    \
+            launched = true;                                                                  \
+        }
+        GO(1, 1) GO(2, 1) GO(3, 1) GO(4, 1) GO(1, 2) GO(2, 2) GO(3, 2) GO(4, 2)
 #undef GO
-    return ILLM_ERR_ARG;
+        if (!launched) return ILLM_ERR_ARG;
+        const int rc = illm_launch_status();
+        if (rc != ILLM_OK) return rc;
+    }
+    return ILLM_OK;
 }

@@ -15,7 +15,7 @@ uses a vendor GEMM too (cublasSgemm, src/kern/gpu/kernel_gpu.cu:420-435).
 Four things ride on the products.  `Weight`: a matrix with a second copy in the
 kernels' own tile order (`decode_weight`).  `linear_add` / `NormedRows`: the
 residual add in the product's epilogue and the RMS norm that follows it taken by
-the next product (up to 16 rows).  `linear_planes`: the product of up to 64 rows (from
+the next product (up to 16 rows).  `linear_planes`: the product of up to 128 rows (from
 17, or from fewer where that is measured to pay) with a long thin matrix, K cut into
 ranges whose float32 planes `add_rmsnorm` adds.
 `_planned_matmul`: products of many rows measured once per shape, whole against
@@ -360,10 +360,12 @@ def linear_add(x: torch.Tensor, w, into: torch.Tensor, norm=None,
     return NormedRows(into, weight, eps, act_dtype, xb, ssq)
 
 
-MID_MAX_ROWS = 64
+MID_MAX_ROWS = 128       # beyond 64 rows the kernel runs once per 64 (the vendor GEMM reads the
+                         # thin matrices at 1.6 TB/s at 128 rows: 58.6 us for the 7B down projection)
 MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the norm that adds the
                          # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
                          # K >= 2 N (the down projection) and the same time when K = N
+PLANES_TWICE_MIN_ROWS = 112
 MEASURE_PLANES = True    # whether `linear_planes_pays` may measure a shape it has not seen
 PLANES_MIN_ELEMENTS = 1 << 22   # smaller matrices are not measured (both ways take a few
                                 # microseconds and the clock would decide): no planes below 17 rows
@@ -371,7 +373,7 @@ _PLANES_FROM: dict = {}  # (N, K) -> fewest rows (1, 5, 9, 13 or 17) from which 
 
 
 def linear_planes_fits(x, w) -> bool:
-    """Whether `linear_planes` takes these operands: up to 64 bfloat16 rows and a matrix with a
+    """Whether `linear_planes` takes these operands: up to 128 bfloat16 rows and a matrix with a
     decode copy in plain tile order that has few rows for its length (K >= 2 N)."""
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == "plain"
             and isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and x.dim() == 2
@@ -415,12 +417,17 @@ def _measure_planes_from(w: "Weight") -> int:
 
 def linear_planes_pays(x, w) -> bool:
     """Whether the planes are the faster way for these operands (which `linear_planes_fits`).
-    Beyond the few-rows kernels' 16 rows always.  Up to 16 rows `linear_add` reads X once per
+    From 17 to 64 rows always.  Up to 16 rows `linear_add` reads X once per
     block of W rows, so its time grows with the rows, and a matrix whose tiles do not fill the
     chip evenly is slow at any (measured: LLaMA-2-7B's down projection 23.3 against 21.7 us at
     16 rows, the 70B's 105 against 77, a 5120 x 13824 one 34 against 30 at 4 rows): measured
     once per shape, outside graph capture."""
     rows = x.shape[0]
+    if rows > 64:
+        # two launches of the kernel, W read twice: that beats the vendor GEMM when the second
+        # is nearly full (128 rows, the bucket of 65 to 128 sequences: 50 against 63 us for the
+        # 7B down projection, 164 against 205 for the 70B one) and loses at 80 rows
+        return rows >= PLANES_TWICE_MIN_ROWS
     if rows > SKINNY_BEST_ROWS:
         return True
     key = tuple(w.plain.shape)

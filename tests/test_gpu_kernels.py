@@ -541,9 +541,10 @@ def _plain_copy(w):
 @pytest.mark.parametrize("M,N,K,splits", [(17, 40, 96, 0), (33, 100, 224, 0), (64, 4096, 11008, 0),
                                           (50, 84, 1184, 5), (48, 20, 64, 1), (31, 72, 352, 3),
                                           (64, 36, 2048, 16), (20, 8192, 16384, 0),
-                                          (1, 40, 96, 0), (7, 100, 224, 2), (16, 4096, 11008, 0)])
+                                          (1, 40, 96, 0), (7, 100, 224, 2), (16, 4096, 11008, 0),
+                                          (65, 40, 96, 0), (100, 84, 1184, 4), (128, 4096, 11008, 0)])
 def test_linear_planes(M, N, K, splits, tiles_per_wave):
-    """The product for up to 64 rows, K cut into ranges: the planes add up to x . w^T, and what
+    """The product for up to 128 rows (64 a launch), K cut into ranges: the planes add up to x . w^T, and what
     `add_rmsnorm` makes of them is the residual add and norm of the product."""
     o = ops()
     if N >= 8192 and tiles_per_wave:
@@ -576,7 +577,7 @@ def test_linear_planes_refuses_what_it_does_not_take():
     assert o.linear_planes_fits(x, _plain_copy(w))
     assert not o.linear_planes_fits(x, w)                                  # no decode copy
     assert o.linear_planes_fits(x[:16], _plain_copy(w)) and o.linear_planes_pays(x, _plain_copy(w))
-    assert not o.linear_planes_fits(rnd(65, 256, dtype=torch.bfloat16).to(DEV), _plain_copy(w))
+    assert not o.linear_planes_fits(rnd(129, 256, dtype=torch.bfloat16).to(DEV), _plain_copy(w))
     assert not o.linear_planes_fits(x.float(), _plain_copy(w))
     wide = rnd(256, 256, dtype=torch.bfloat16).to(DEV)                      # K < 2 N: the vendor GEMM's
     assert not o.linear_planes_fits(x, _plain_copy(wide))
@@ -586,7 +587,7 @@ def test_linear_planes_refuses_what_it_does_not_take():
         o.linear_planes(x, w)
     y = torch.empty(2, 20, 64, device=DEV)
     assert o._lib().illm_gemm_mid_bf16(o._p(x), o._p(_plain_copy(w).tiled), o._p(y), 0, 20, 64, 250, 2, None) != 0
-    assert o._lib().illm_gemm_mid_bf16(o._p(x), o._p(_plain_copy(w).tiled), o._p(y), 0, 65, 64, 256, 2, None) != 0
+    assert o._lib().illm_gemm_mid_bf16(o._p(x), o._p(_plain_copy(w).tiled), o._p(y), 0, 129, 64, 256, 2, None) != 0
     assert o._lib().illm_gemm_mid_bf16(o._p(x), o._p(_plain_copy(w).tiled), o._p(y), 0, 20, 64, 256, 3, None) != 0
 
 

@@ -75,7 +75,7 @@ def test_short_prompts_at_head_size_128(tmp_path_factory, copies):
 
 
 def test_steps_of_17_to_64_rows(tmp_path_factory, monkeypatch):
-    """Steps of 17 to 64 rows (a prompt of that length, or that many sequences decoding) read the
+    """Steps of 17 to 128 rows (here 24 to 64: a prompt of that length, or that many sequences decoding) read the
     decode copy of the down projection with K cut into ranges, whose planes the next norm adds
     (configuration B: 96 x 256).  24 sequences decode together after prompts of unequal lengths;
     one prompt of 40 tokens runs alone."""
@@ -100,7 +100,7 @@ def test_steps_of_17_to_64_rows(tmp_path_factory, monkeypatch):
     for i, h in enumerate(heads):
         got[i].append(out[at:at + h].clone())
         at += h
-    assert not calls                                     # more than 64 rows: the vendor GEMM
+    assert not calls                                     # 139 rows, more than 128: the vendor GEMM
     for t in range(2):
         out = eng.step([StepEntry(s, [r[h + t]], [0]) for s, r, h in zip(slots, reqs, heads)])
         for i in range(len(reqs)):
