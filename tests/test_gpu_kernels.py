@@ -468,6 +468,17 @@ def test_products_of_many_rows_are_planned_once_and_stay_right():
     assert len(o._PLANS) == 1                              # measured once
     o.linear(x[:1000].to(DEV), w.to(DEV))                  # fewer rows than planning is for
     assert len(o._PLANS) == 1
+    # 65 to 255 rows: whole against filled up to 256 rows, once per shape and 32 rows
+    few = x[:100].to(DEV)
+    close(o.linear(few, w.to(DEV)), R.linear(x[:100], w), torch.bfloat16, scale=math.sqrt(K))
+    assert o._PLANS.get(("pad", 4, N, K)) in ((), ("pad", 256)) and len(o._PLANS) == 2
+    close(o._run_plan(few, w.to(DEV), ("pad", 256)), R.linear(x[:100], w), torch.bfloat16, scale=math.sqrt(K))
+    into = torch.empty(100, N, dtype=torch.bfloat16, device=DEV)
+    assert o._run_plan(few, w.to(DEV), ("pad", 256), into) is into
+    close(into, R.linear(x[:100], w), torch.bfloat16, scale=math.sqrt(K))
+    o.linear(x[:64].to(DEV), w.to(DEV))
+    o.linear(x[:256].to(DEV), w.to(DEV))
+    assert len(o._PLANS) == 2
 
 
 def _prepared_rows(M, K, nw_dtype, eps, seed=5):
