@@ -120,21 +120,34 @@ def main() -> int:
         draw = sampler.draw(eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)]),
                             [0] * batch, [0] * batch)
 
+        seen = []
+
         def one():
             nonlocal draw
             logits = eng.step([StepEntry(s, [0], [0]) for s in slots], device_tokens=draw.device)
             following = sampler.draw(logits, [0] * batch, [0] * batch)
-            draw.tokens()
+            seen.append(draw.tokens())
             draw = following
+            return logits
 
         for _ in range(warmup):
             one()
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(steps):
-            one()
+            logits = one()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
+        # what was timed must have computed something: finite logits, and greedy tokens that
+        # change from step to step (a run on NaN or constant logits would be as fast)
+        if not bool(torch.isfinite(logits).all()):
+            raise SystemExit(f"bench: non-finite logits in the decode run at batch {batch}")
+        distinct = {int(t) for row in seen for t in row}
+        print(f"[bench] batch {batch}: {len(distinct)} distinct greedy tokens in {len(seen)} steps",
+              file=sys.stderr, flush=True)
+        if len(seen) >= 16 and len(distinct) < 2:
+            raise SystemExit(f"bench: the greedy token is {sorted(distinct)} in every step of every "
+                             f"sequence at batch {batch}: the logits are degenerate")
         mean_ctx = args.prompt + 1 + warmup + (steps + 1) / 2.0
         for s in slots:
             eng.free_slot(s)
@@ -151,6 +164,8 @@ def main() -> int:
             ops.argmax(logits).tolist()
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t)
+            if not bool(torch.isfinite(logits).all()):
+                raise SystemExit("bench: non-finite logits in the prefill")
             eng.free_slot(s)
         pt = min(times[1:])
         fl = prefill_flops(cfg, layers, T)

@@ -122,7 +122,7 @@ def main(argv=None) -> int:
     else:
         eng = Engine.from_pretrained(args.model, **kw)
     if args.mtype is not None:
-        family = {"LlamaForCausalLM": ("llama", "llama2")}.get(eng.spec.architecture, ())
+        family = tuple(getattr(type(eng.config), "cli_type_names", ()))
         if args.mtype not in family:
             print(f"chat: --type {args.mtype!r} does not fit the model's architecture "
                   f"{eng.spec.architecture!r}", file=sys.stderr)

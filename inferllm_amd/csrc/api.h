@@ -96,11 +96,6 @@ int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y,
                          int K, const void* nw, int nw_dt, void* xb, float* ssq_out,
                          int waves_wanted, void* stream);
 
-// Tuning entry of the same product: rows of W per block 16 * ntb (ntb 1, 2, 4), u * 64 bytes
-// of a W row per wave iteration (u 4, 8), waves per block.
-int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M, int N,
-                              int K, int ntb, int u, int waves, void* stream);
-
 // Y = X[M, K] . W[N, K]^T for M up to 128 (64 rows a launch) from the tiled copy Wt of W, K a
 // multiple of 32, X shared by a block's waves through LDS.  splits == 1: Y is [M, N] of y_dt;
 // splits > 1: K is cut into that many ranges and Y is float32 [splits][M][N], the planes to be
@@ -109,10 +104,6 @@ int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M, 
                        int splits, void* stream);
 int illm_gemm_mid_splits(int N, int K);
 void illm_set_mid_tiles_per_wave(int n);      // tuning: 1 or 2 (0: by the number of tiles)
-
-// Tuning: tiles a block of the tiled plain and gate|up products takes (1 or 2; 0: the default,
-// two when there are at least 1024 tiles).
-void illm_set_skinny_tiles_per_block(int n);
 
 // Tuning and tests: 0 switches off the variant of the residual-adding product in which, for K up
 // to 4096 and at most 512 tiles, 8 waves each take their whole share of K at once (default 1).

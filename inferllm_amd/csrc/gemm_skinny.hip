@@ -461,12 +461,10 @@ static int launch_skinny(const void* X, const void* W, void* Y, int y_dt, int M,
 // Measured on MI355X at the LLaMA-2-7B shapes: 16 W rows per block and about this many waves
 // on the chip are best for M <= 16; wider row tiles only pay when X has many rows.
 static const int SK_WAVES_ON_CHIP = 2400;
-// Tiles a block of the tiled gate|up and plain products takes: 0 = by the number of tiles (two
-// from 1024 tiles on), 1 or 2 = forced (tuning).
+// A block of the tiled gate|up and plain products takes two tiles from 1024 tiles on.
+static bool two_tiles_a_block(int blocks) { return blocks >= 1024; }
 static int SK_ONE_SHOT = 1;           // tuning: 0 switches the one-piece-per-wave variant off
 extern "C" void illm_set_skinny_one_shot(int on) { SK_ONE_SHOT = on; }
-static int SK_TILES_PER_BLOCK = 0;
-extern "C" void illm_set_skinny_tiles_per_block(int n) { SK_TILES_PER_BLOCK = (n == 1 || n == 2) ? n : 0; }
 static const int SK_WAVES_ON_CHIP_TILED = 3072;      // from the tiled copy (no staging in LDS)
 
 static int clamp_waves(int w, int ntb, int mt, int u, int K) {
@@ -479,10 +477,11 @@ static int clamp_waves(int w, int ntb, int mt, int u, int K) {
     return w < 1 ? 1 : w;
 }
 
-// Tuning entry: the same product with the tile shape given: ntb in {1, 2, 4}, u in {4, 8},
-// waves per block (clamped to what LDS and K allow).  Used to choose the defaults below.
-extern "C" int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, int y_dt, int M,
-                                         int N, int K, int ntb, int u, int waves, void* stream) {
+// The product from the matrix itself (no tiled copy) with the tile shape given: 16 * ntb rows of
+// W a block, u * 64 bytes of a W row per wave iteration, waves per block (clamped to what LDS
+// and K allow).  Up to 16 rows of X take ntb = 1, more take 2; u = 4 (measured best).
+static int skinny_from_matrix(const void* X, const void* W, void* Y, int y_dt, int M,
+                              int N, int K, int ntb, int u, int waves, void* stream) {
     if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8) || !illm_dtype_ok(y_dt))
         return ILLM_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
@@ -491,10 +490,7 @@ extern "C" int illm_gemm_skinny_bf16_cfg(const void* X, const void* W, void* Y, 
 #define GO(MT_, NTB_, U_)                                                                     \
     if (mt == MT_ && ntb == NTB_ && u == U_)                                                  \
         return launch_skinny<MT_, NTB_, U_>(X, W, Y, y_dt, M, N, K, waves, st)
-    GO(1, 1, 4); GO(1, 2, 4); GO(1, 4, 4); GO(1, 1, 8); GO(1, 2, 8); GO(1, 4, 8);
-    GO(2, 1, 4); GO(2, 2, 4); GO(2, 4, 4); GO(2, 2, 8);
-    GO(3, 2, 4); GO(3, 4, 4);
-    GO(4, 1, 4); GO(4, 2, 4); GO(4, 4, 4);
+    GO(1, 1, 4); GO(2, 2, 4); GO(3, 2, 4); GO(4, 2, 4);
 #undef GO
     return ILLM_ERR_ARG;
 }
@@ -520,13 +516,13 @@ extern "C" int illm_gemm_skinny_bf16(const void* X, const void* W, const void* W
     int waves = waves_wanted > 0 ? waves_wanted : (on_chip + blocks / 2) / blocks;
     waves = waves < 1 ? 1 : waves;
     if (!ssq && !use_tiled(Wt, M, K))
-        return illm_gemm_skinny_bf16_cfg(X, W, Y, y_dt, M, N, K, ntb, u, waves, stream);
+        return skinny_from_matrix(X, W, Y, y_dt, M, N, K, ntb, u, waves, stream);
     SkResidual res = SK_NO_RESIDUAL;
     res.ssq = ssq; res.parts = parts; res.eps = eps;
     waves = clamp_waves(waves, 1, 1, 4, K);
     if (use_tiled(Wt, M, K)) {
         // with many tiles (the head) a block takes two: X is read half as often
-        if (SK_TILES_PER_BLOCK == 2 || (SK_TILES_PER_BLOCK == 0 && blocks >= 1024)) {
+        if (two_tiles_a_block(blocks)) {
             const int blocks2 = (blocks + 1) / 2;
             int w2 = waves_wanted > 0 ? waves_wanted : (on_chip + blocks2 / 2) / blocks2;
             return launch_skinny<1, 2, 4, SK_PLAIN, true>(X, Wt, Y, y_dt, M, N, K,
@@ -589,7 +585,7 @@ extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const 
     if (use_tiled(Wt, M, K)) {
         // with many tiles a block takes two: X is read half as often (measured at F = 11008, 8 and
         // 16 rows: 36 -> 31 us and 46 -> 33 us; one row: no change)
-        if (SK_TILES_PER_BLOCK == 2 || (SK_TILES_PER_BLOCK == 0 && blocks >= 1024)) {
+        if (two_tiles_a_block(blocks)) {
             const int blocks2 = (F + 15) / 16;
             int w2 = waves_wanted > 0 ? waves_wanted : (1400 + blocks2 / 2) / blocks2;
             w2 = clamp_waves(w2 < 1 ? 1 : w2, 2, mt, 4, K);
@@ -597,7 +593,7 @@ extern "C" int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const 
         }
         return launch_skinny<1, 1, 4, SK_GATE_UP, true>(X, Wt, Y, y_dt, M, F, K, waves, st, SkRope(), res);
     }
-    if (mt == 1 && (SK_TILES_PER_BLOCK == 2 || (SK_TILES_PER_BLOCK == 0 && blocks >= 1024))) {
+    if (mt == 1 && two_tiles_a_block(blocks)) {
         const int blocks2 = (F + 15) / 16;
         int w2 = waves_wanted > 0 ? waves_wanted : (1400 + blocks2 / 2) / blocks2;
         w2 = clamp_waves(w2 < 1 ? 1 : w2, 2, mt, 4, K);

@@ -7,11 +7,13 @@ decode_summary) with batches of sequences in place of its single one.
 """
 from __future__ import annotations
 
+import warnings
 from typing import Dict, List, Optional, Sequence, Union
 
 import torch
 
 from ..kernels import ops
+from ..kernels.plan import Plan
 from ..cache.manager import PAGE_SIZE, CacheManager, round_up
 from ..config.registry import config_from_dict, load_config
 from ..sampling.params import SamplingParams
@@ -37,13 +39,19 @@ def parse_dtype(dtype) -> torch.dtype:
 class Engine:
     """One model on one GPU with its cache, step function and generation loop.
 
-    dtype "bfloat16": weights as stored, bfloat16 activations and cache, float32
-    residual stream, statistics and logits.  dtype "float32": everything in true
+    dtype "bfloat16": bfloat16 matrices, activations and cache, float32 residual
+    stream, statistics and logits.  dtype "float32": everything in true
     float32 (own multiply-add kernels; no matrix-core or reduced-precision mode).
 
     `decode_copies`: keep a second copy of every matrix in the layout of the few-rows kernels
     (decoding reads that one, prompts the row-major one), or with "thin" of the down projections
     alone; default: all if they fit comfortably, else the thin ones if those do.
+
+    `tune`, `plan`: some bfloat16 products have several equivalent ways that differ in speed by
+    shape and in rounding.  By default the way is taken from fixed tables (`kernels.plan`), so the
+    same request gives the same bits in every process and nothing is timed.  `tune=True` times
+    the ways for shapes the tables lack (thin matrices now, many-row products at first use) and
+    keeps the winners in `engine.plan`; `plan=` (a `Plan` or what its `to_dict()` gave) pins them.
 
     Cache size: `max_tokens` is the most tokens live sequences hold together (each
     rounded up to 64), `max_batch` the most live sequences, `max_seq_len` the longest
@@ -53,7 +61,7 @@ class Engine:
     def __init__(self, config, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  max_batch: int = 8, max_seq_len: Optional[int] = None,
                  max_tokens: Optional[int] = None, use_graphs: bool = True,
-                 poison_freed: bool = False, decode_copies=None):
+                 poison_freed: bool = False, decode_copies=None, tune: bool = False, plan=None):
         self.config = config
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
@@ -80,11 +88,19 @@ class Engine:
         if self.dtype != torch.bfloat16:
             decode_copies = False
         self.decode_copies = decode_copies if decode_copies == "thin" else bool(decode_copies)
-        ops.DECODE_COPIES = self.decode_copies
-        try:
-            self.model.load(tensors)
-        finally:
-            ops.DECODE_COPIES = False
+        self.model.load(tensors, decode_copies=self.decode_copies)
+        if isinstance(plan, dict):
+            plan = Plan.from_dict(plan)
+        self.plan: Plan = plan if plan is not None else Plan.fixed(measure=bool(tune))
+        if self.plan.measure and self.dtype == torch.bfloat16:
+            ops.use_plan(self.plan)
+            for part in self.model.every_part():
+                for w in vars(part).values():
+                    if (isinstance(w, ops.Weight) and w.tiled is not None and w.mode == "plain"
+                            and tuple(w.shape) not in self.plan.planes_from
+                            and w.shape[1] >= 2 * w.shape[0] and w.shape[0] <= ops.MID_MAX_COLS
+                            and w.shape[0] % 4 == 0):
+                        self.plan.planes_from[tuple(w.shape)] = ops.measure_planes_from(w)
         limit = self.spec.max_positions
         self.max_seq_len = min(int(max_seq_len), limit) if max_seq_len else limit
         self.max_batch = int(max_batch)
@@ -94,17 +110,33 @@ class Engine:
                                   max_tokens=int(max_tokens), max_slots=self.max_batch,
                                   max_seq_len=self.max_seq_len, dtype=self.dtype,
                                   device=self.device, poison_freed=poison_freed)
-        self.runner = StepRunner(self.model, self.cache, self.dtype, self.device, use_graphs)
+        self.runner = StepRunner(self.model, self.cache, self.dtype, self.device, use_graphs,
+                                 plan=self.plan)
         self.last_stats: Optional[GenerationStats] = None
 
     # ------------------------------------------------------------ construction
     @classmethod
-    def from_pretrained(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
-        """From a folder with config.json and model.safetensors (or its shards)."""
+    def from_pretrained(cls, model_dir: str, dtype="bfloat16", device="cuda:0",
+                        keep_stored: bool = False, **kw) -> "Engine":
+        """From a folder with config.json and model.safetensors (or its shards).
+
+        Matrices take the engine's dtype as they are loaded, whatever the file stores them in
+        (float16 and float32 are rounded to bfloat16, to nearest even, in a bfloat16 engine; the
+        reference gives a tensor the runtime type of its file code, src/core/graph.cpp:216-231).
+        `keep_stored=True` keeps 32-bit and float16 matrices as float32 instead: their products
+        then run on the float32 multiply-add kernel, at twice the memory and a fraction of the
+        speed (a warning says so)."""
         config = load_config(model_dir)
         model = DecoderModel(config.to_spec())
-        tensors = load_named_tensors(model_dir, model.wants(), parse_dtype(dtype), device,
-                                     config.to_spec().ignored_tensor_suffixes)
+        dt = parse_dtype(dtype)
+        tensors = load_named_tensors(model_dir, model.wants(), dt, device,
+                                     config.to_spec().ignored_tensor_suffixes, keep_stored)
+        if keep_stored and dt == torch.bfloat16:
+            wide = [n for n, t in tensors.items() if t.dim() == 2 and t.dtype == torch.float32]
+            if wide:
+                warnings.warn(f"{len(wide)} matrices stay float32 in a bfloat16 engine "
+                              f"(keep_stored): their products run on the float32 kernel, not on "
+                              f"the matrix cores")
         return cls(config, tensors, dtype, device, **kw)
 
     @classmethod

@@ -24,8 +24,15 @@ class DecoderModel:
         self.spec = spec
         self.embedding = build_part("embedding", spec.embedding)
         self.layers: List[Block] = []
+        # position parts whose `on_embedding` hook runs on the embedded rows: one per distinct
+        # position spec among the layers (layers that name the same encoding share one call)
+        self.embedding_hooks: List = []
+        hooked: List = []
         for ls in spec.layers:
             position = build_part("position", ls.position) if ls.position is not None else None
+            if position is not None and ls.position not in hooked:
+                hooked.append(ls.position)
+                self.embedding_hooks.append(position)
             self.layers.append(part_class("block", ls.block)(
                 mixer=build_part("mixer", ls.mixer),
                 feed_forward=build_part("feed_forward", ls.feed_forward),
@@ -45,10 +52,10 @@ class DecoderModel:
             elif e.cache_line not in writers:
                 raise ValueError(f"schedule: cache line {e.cache_line} is read before any run writes it")
         self.loaded = False
-        every = [self.embedding, self.final_norm, self.head]
-        for layer in self.layers:
-            every.extend([layer] + layer.parts())
-        self.graph_safe = all(getattr(p, "graph_safe", True) for p in every)
+        self.graph_safe = all(getattr(p, "graph_safe", True) for p in self.every_part())
+        # mixers that cannot go on from their cache by more than one token a step
+        self.one_token_mixers = sorted({type(l.mixer).__name__ for l in self.layers
+                                        if not getattr(l.mixer, "takes_continuations", False)})
 
     # ------------------------------------------------------------ weights
     def wants(self) -> Dict[str, TensorWant]:
@@ -63,7 +70,17 @@ class DecoderModel:
                 out[name] = want
         return out
 
-    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+    def every_part(self) -> List:
+        every = [self.embedding, self.final_norm, self.head]
+        for layer in self.layers:
+            every.extend([layer] + layer.parts())
+        return every
+
+    def load(self, tensors: Dict[str, torch.Tensor], decode_copies=False) -> None:
+        """Hand every part its tensors.  `decode_copies`: whether the parts keep second copies of
+        their matrices for the few-rows kernels (False, True or "thin")."""
+        for part in self.every_part():
+            part.decode_copies = decode_copies
         for part in [self.embedding, *self.layers, self.final_norm, self.head]:
             part.load(tensors)
         self.loaded = True
@@ -93,10 +110,8 @@ class DecoderModel:
         """Run the step's rows through every scheduled layer; logits (float32
         [len(out_rows), vocab]) for the rows asked for, or None if none is."""
         x = self.embedding.forward(ctx)
-        for layer in self.layers:
-            if layer.position is not None:
-                layer.position.on_embedding(x, ctx)
-                break
+        for position in self.embedding_hooks:
+            position.on_embedding(x, ctx)
         pending = None
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]

@@ -20,6 +20,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from ..cache.manager import CacheManager
+from ..kernels import ops
 from ..parts.base import StepContext
 from .model import DecoderModel
 
@@ -86,8 +87,9 @@ class StepRunner:
     """Owns the model, the cache and the decode graphs; `step` is the one entry."""
 
     def __init__(self, model: DecoderModel, cache: CacheManager, act_dtype: torch.dtype,
-                 device: torch.device, use_graphs: bool = True):
+                 device: torch.device, use_graphs: bool = True, plan=None):
         self.model, self.cache = model, cache
+        self.plan = plan
         self.act_dtype, self.device = act_dtype, device
         self.vocab_size = model.spec.vocab_size
         self.use_graphs = (use_graphs and model.graph_safe
@@ -118,8 +120,11 @@ class StepRunner:
             return True
         if not any(starts) and all(len(e.tokens) == 1 for e in entries):
             return False
+        if not self.model.one_token_mixers:
+            return True            # every mixer goes on from what it kept by any number of tokens
         raise StepError("the sequences of a step must either all start at their first token "
-                        "or all go on by one token")
+                        "or all go on by one token: this model's "
+                        f"{', '.join(self.model.one_token_mixers)} cannot go on by several")
 
     # ------------------------------------------------------------ the step
     @torch.no_grad()
@@ -132,7 +137,9 @@ class StepRunner:
         token of every entry in order, in place of the entries' own (which are placeholders
         then).  It lets a caller start the next step from tokens that were chosen on the device
         before it has read them back."""
-        prefill = self._phase(entries)
+        prefill = self._phase(entries)          # True: a step of several tokens per sequence
+        if self.plan is not None:
+            ops.use_plan(self.plan)
         if device_tokens is not None:
             if prefill:
                 raise StepError("tokens from the device are taken by steps of single tokens only")
@@ -143,25 +150,26 @@ class StepRunner:
         self.cache.extend_all([(e.slot, s, len(e.tokens)) for e, s in zip(entries, starts)])
         self.cache.upload(lengths=prefill)
         if prefill:
-            return self._prefill(entries)
+            return self._prefill(entries, starts)
         return self._decode(entries, starts, device_tokens)
 
-    def _prefill(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _prefill(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> Optional[torch.Tensor]:
         tokens: List[int] = []
         pos: List[int] = []
         slot: List[int] = []
         cu = [0]
         want: List[int] = []
-        for e in entries:
+        for e, start in zip(entries, starts):
             n = len(e.tokens)
             want.extend(cu[-1] + int(w) for w in e.want)
             tokens.extend(int(t) for t in e.tokens)
-            pos.extend(range(n))
+            pos.extend(range(start, start + n))
             slot.extend([e.slot] * n)
             cu.append(cu[-1] + n)
         T, B = len(tokens), len(entries)
         host = torch.tensor(tokens + pos + slot + cu + [e.slot for e in entries]
-                            + [len(e.tokens) for e in entries] + want, dtype=torch.int32)
+                            + [s + len(e.tokens) for e, s in zip(entries, starts)] + want,
+                            dtype=torch.int32)
         meta = host.to(self.device)
         o = 0
         parts = []
@@ -171,7 +179,8 @@ class StepRunner:
         ctx = StepContext(
             device=self.device, act_dtype=self.act_dtype, prefill=True, n_rows=T, n_seqs=B,
             tokens=parts[0], row_pos=parts[1], row_slot=parts[2], cu_seqlens=parts[3],
-            seq_slot=parts[4], seq_len=parts[5], max_len=max(len(e.tokens) for e in entries),
+            seq_slot=parts[4], seq_len=parts[5],
+            max_len=max(s + len(e.tokens) for e, s in zip(entries, starts)),
             cache=self.cache)
         return self.model.forward(ctx, parts[6] if want else None)
 
@@ -202,6 +211,8 @@ class StepRunner:
         g = self._graphs.get(key)
         if g is None:
             g = self._graphs[key] = _DecodeGraph(self, *key)
+        if g.graph is None:
+            self._capture(g)
         if g.in_flight:
             g.copied.synchronize()          # the last step's copy has left the pinned buffer
         g.stage_np[:] = host
@@ -210,8 +221,6 @@ class StepRunner:
         if device_tokens is not None:
             g.meta[:B].copy_(device_tokens)
         g.in_flight = True
-        if g.graph is None:
-            self._capture(g)
         g.graph.replay()
         if not wanted:
             return None
@@ -220,11 +229,19 @@ class StepRunner:
         return g.logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
 
     def _capture(self, g: _DecodeGraph) -> None:
-        ctx = g.context(self)
+        """Capture the step's graph.  Before a capture the libraries must have set themselves up,
+        which takes one eager run of the same shapes: that run has every row on the cache's spare
+        slot and spare page, so that no real sequence's cache or state is written twice (a part
+        that updates per-sequence state is not idempotent as the store of keys is).  The capture
+        itself executes nothing; the caller fills in the step's numbers and replays."""
+        n = g.size
+        spare = self.cache.spare_slot
+        warm = torch.tensor([0] * n + [0] * n + [spare] * n + [1] * n, dtype=torch.int32)
+        g.meta.copy_(warm.to(self.device))
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(side):
-            self.model.forward(ctx, g.rows)        # warm-up: the libraries set themselves up
+            self.model.forward(g.context(self), g.rows)
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()

@@ -16,10 +16,11 @@ Four things ride on the products.  `Weight`: a matrix with a second copy in the
 kernels' own tile order (`decode_weight`).  `linear_add` / `NormedRows`: the
 residual add in the product's epilogue and the RMS norm that follows it taken by
 the next product (up to 16 rows).  `linear_planes`: the product of up to 128 rows (from
-17, or from fewer where that is measured to pay) with a long thin matrix, K cut into
+17, or from fewer where the plan says that pays) with a long thin matrix, K cut into
 ranges whose float32 planes `add_rmsnorm` adds.
-`_planned_matmul`: products of many rows measured once per shape, whole against
-cut along the output columns.
+`_planned_matmul`: products of many rows whole or cut along the output columns, as the
+current plan's table says for the shape (`kernels.plan`: fixed tables by default, so that
+nothing depends on a stopwatch).
 """
 from __future__ import annotations
 
@@ -29,6 +30,7 @@ from typing import Optional
 import torch
 
 from . import build
+from .plan import NEVER_BELOW, Plan
 
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
@@ -211,12 +213,6 @@ class Weight:
         return self.plain.dtype
 
 
-# Whether `decode_weight` makes the second copy (set by the engine): False, True (of every matrix)
-# or "thin" (only of matrices with K >= 2 N, the down projections: where the vendor GEMM is weakest
-# at 17 to 64 rows and `linear_planes` needs the copy; for models whose copies do not all fit).
-DECODE_COPIES = False
-
-
 def _w(w, mode: str = "plain"):
     """(plain tensor, pointer of the tiled copy or None) of a weight argument, for the kernel
     whose tiles are `mode`; a copy made for another kernel's tiles is not used."""
@@ -264,12 +260,15 @@ def tile_weight(w: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
     return picked.view(rows.shape[0], 16, K // 32, 32).permute(0, 2, 1, 3).contiguous()
 
 
-def decode_weight(w: torch.Tensor, mode: str = "plain", **geometry):
+def decode_weight(w: torch.Tensor, mode: str = "plain", copies=False, **geometry):
     """The weight as the parts keep it: with a tiled copy for the few-rows kernels if the engine
-    asked for decode copies and the matrix allows it, else the tensor itself."""
-    if (DECODE_COPIES and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0
+    asked for decode copies and the matrix allows it, else the tensor itself.  `copies`: False,
+    True (of every matrix) or "thin" (only of matrices with K >= 2 N, the down projections:
+    where the vendor GEMM is weakest at 17 to 64 rows and `linear_planes` needs the copy; for
+    models whose copies do not all fit)."""
+    if (copies and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 32 == 0
             and w.is_cuda and (mode != "qkv" or geometry.get("hd", 0) % 16 == 0)
-            and (DECODE_COPIES != "thin" or (mode == "plain" and w.shape[1] >= 2 * w.shape[0]))):
+            and (copies != "thin" or (mode == "plain" and w.shape[1] >= 2 * w.shape[0]))):
         return Weight(w, tile_weight(w, tile_rows(w.shape[0], mode, **geometry)), mode)
     return w
 
@@ -366,10 +365,21 @@ MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the no
                          # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
                          # K >= 2 N (the down projection) and the same time when K = N
 PLANES_TWICE_MIN_ROWS = 112
-MEASURE_PLANES = True    # whether `linear_planes_pays` may measure a shape it has not seen
 PLANES_MIN_ELEMENTS = 1 << 22   # smaller matrices are not measured (both ways take a few
                                 # microseconds and the clock would decide): no planes below 17 rows
-_PLANES_FROM: dict = {}  # (N, K) -> fewest rows (1, 5, 9, 13 or 17) from which the planes pay
+
+# The tables that products with more than one way are dispatched by (`kernels.plan`).  An engine
+# makes its own current at the start of each of its steps; nothing is timed unless the plan asks.
+_plan: Plan = Plan.fixed()
+
+
+def use_plan(plan: Plan) -> None:
+    global _plan
+    _plan = plan
+
+
+def current_plan() -> Plan:
+    return _plan
 
 
 def linear_planes_fits(x, w) -> bool:
@@ -382,12 +392,12 @@ def linear_planes_fits(x, w) -> bool:
             and w.plain.shape[1] >= 2 * w.plain.shape[0])
 
 
-def _measure_planes_from(w: "Weight") -> int:
+def measure_planes_from(w: "Weight") -> int:
     """Fewest rows from which `linear_planes` and the norm that adds its planes take less time
     than `linear_add` (whose norm the next product takes), measured at 16, 12, 8 and 4 rows."""
     N, K = w.plain.shape
     if N * K < PLANES_MIN_ELEMENTS:
-        return SKINNY_BEST_ROWS + 1
+        return NEVER_BELOW
     dev = w.plain.device
     x = torch.zeros((SKINNY_BEST_ROWS, K), dtype=torch.bfloat16, device=dev)
     into = torch.zeros((SKINNY_BEST_ROWS, N), dtype=torch.float32, device=dev)
@@ -404,7 +414,7 @@ def _measure_planes_from(w: "Weight") -> int:
         end.synchronize()
         return start.elapsed_time(end)
 
-    first = SKINNY_BEST_ROWS + 1
+    first = NEVER_BELOW
     for rows in (16, 12, 8, 4):
         xs, dst = x[:rows], into[:rows]
         t_add = timed(lambda: linear_add(xs, w, dst, (nw, 1e-5)))
@@ -420,8 +430,8 @@ def linear_planes_pays(x, w) -> bool:
     From 17 to 64 rows always.  Up to 16 rows `linear_add` reads X once per
     block of W rows, so its time grows with the rows, and a matrix whose tiles do not fill the
     chip evenly is slow at any (measured: LLaMA-2-7B's down projection 23.3 against 21.7 us at
-    16 rows, the 70B's 105 against 77, a 5120 x 13824 one 34 against 30 at 4 rows): measured
-    once per shape, outside graph capture."""
+    16 rows, the 70B's 105 against 77, a 5120 x 13824 one 34 against 30 at 4 rows): by the
+    plan's table; a plan that measures times a shape it lacks once, outside graph capture."""
     rows = x.shape[0]
     if rows > 64:
         # two launches of the kernel, W read twice: that beats the vendor GEMM when the second
@@ -431,11 +441,11 @@ def linear_planes_pays(x, w) -> bool:
     if rows > SKINNY_BEST_ROWS:
         return True
     key = tuple(w.plain.shape)
-    first = _PLANES_FROM.get(key)
+    first = _plan.planes_from.get(key)
     if first is None:
-        if not MEASURE_PLANES or torch.cuda.is_current_stream_capturing():
-            return False
-        first = _PLANES_FROM[key] = _measure_planes_from(w)
+        if not _plan.measure or torch.cuda.is_current_stream_capturing():
+            return rows >= NEVER_BELOW
+        first = _plan.planes_from[key] = measure_planes_from(w)
     return rows >= first
 
 
@@ -486,14 +496,13 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
 
 # The vendor GEMM's own choice of kernel is now and then a poor one for a shape (measured on
 # MI355X: 2048 x 22016 x 4096 takes 408 us whole and 253 us as 8192 + 13824 columns; most shapes
-# gain nothing).  So products of many rows are planned by measurement, once per shape: the whole
-# product against a few cuts of the output columns, each part written into its slice of one
-# result.  Every output element is still one kernel's sum; plans differ in rounding only.
-PLAN_PRODUCTS = True
+# gain nothing).  So products of many rows are planned per shape: the whole product or a cut of
+# the output columns, each part written into its slice of one result, as the current plan's
+# table says (`kernels.plan`; a plan that measures times the candidates for a shape it lacks).
+# Every output element is still one kernel's sum; plans differ in rounding only.
 PLAN_MIN_ROWS = 1024          # below this no cut ever paid
 PLAN_MIN_COLS = 8192
 PAD_MIN_ROWS, PAD_ROWS = 64, 256     # rows between these may be filled up to PAD_ROWS
-_PLANS: dict = {}             # (rows / 256 rounded up, N, K) -> cut points (empty: whole)
 
 
 def _split_candidates(N: int, M: int = 0):
@@ -532,7 +541,7 @@ def _run_plan(x: torch.Tensor, w: torch.Tensor, plan, out: Optional[torch.Tensor
     return out
 
 
-def _measure_plan(x: torch.Tensor, w: torch.Tensor, candidates=None):
+def measure_plan(x: torch.Tensor, w: torch.Tensor, candidates=None):
     out = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
     best, best_t = (), None
     for plan in candidates or _split_candidates(w.shape[0], x.shape[0]):
@@ -552,24 +561,26 @@ def _measure_plan(x: torch.Tensor, w: torch.Tensor, candidates=None):
 def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     M, K = x.shape
     N = w.shape[0]
-    if PLAN_PRODUCTS and PAD_MIN_ROWS < M < PAD_ROWS:
+    capturing = torch.cuda.is_current_stream_capturing()
+    if PAD_MIN_ROWS < M < PAD_ROWS:
         # the vendor GEMM takes 65 to 255 rows of some shapes slower than 256 (measured: 4096 x
-        # 11008 at 192 rows 82 us, at 256 rows 51): whole against filled up to 256, once per
-        # shape and 32 rows
+        # 11008 at 192 rows 82 us, at 256 rows 51): whole or filled up to 256, per shape and
+        # 32 rows
         key = ("pad", -(-M // 32), N, K)
-        plan = _PLANS.get(key)
+        plan = _plan.cuts.get(key)
         if plan is None:
-            if torch.cuda.is_current_stream_capturing():
+            if not _plan.measure or capturing:
                 return torch.matmul(x, w.t())
-            plan = _PLANS[key] = _measure_plan(x, w, [(), ("pad", PAD_ROWS)])
+            plan = _plan.cuts[key] = measure_plan(x, w, [(), ("pad", PAD_ROWS)])
         return _run_plan(x, w, plan)
-    if (not PLAN_PRODUCTS or M < PLAN_MIN_ROWS or N < PLAN_MIN_COLS
-            or torch.cuda.is_current_stream_capturing()):
+    if M < PLAN_MIN_ROWS or N < PLAN_MIN_COLS:
         return torch.matmul(x, w.t())
     key = (-(-M // 256), N, K)
-    plan = _PLANS.get(key)
+    plan = _plan.cuts.get(key)
     if plan is None:
-        plan = _PLANS[key] = _measure_plan(x, w)
+        if not _plan.measure or capturing:
+            return torch.matmul(x, w.t())
+        plan = _plan.cuts[key] = measure_plan(x, w)
     if plan and plan[0] == "rows" and M % (256 * plan[1]):
         plan = ()                                # measured at the class's full size; M is ragged
     return _run_plan(x, w, plan)

@@ -49,6 +49,9 @@ class LlamaConfig:
     rope_scaling: Optional[dict] = None
 
     architecture = "LlamaForCausalLM"
+    # what the command line's --type may name for this architecture (the reference's model-type
+    # strings, src/graph/graph_imp.cpp:6-21: "llama" and "llama2" are its two LLaMA graphs)
+    cli_type_names = ("llama", "llama2")
 
     # ------------------------------------------------------------ reading
     @classmethod

@@ -58,8 +58,10 @@ class Attention(Mixer):
 
     def load(self, tensors) -> None:
         self.w_qkv = ops.decode_weight(_fuse([self._take(tensors, n) for n in ("q", "k", "v")]),
-                                       "qkv", nh=self.nh, nkv=self.nkv, hd=self.hd)
-        self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous())
+                                       "qkv", self.decode_copies, nh=self.nh, nkv=self.nkv,
+                                       hd=self.hd)
+        self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous(), "plain",
+                                     self.decode_copies)
 
     def forward(self, h, ctx: StepContext, line, writes_cache, position, residual=None,
                 next_norm=None):

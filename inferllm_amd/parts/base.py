@@ -64,6 +64,9 @@ class Part:
     # A part with `takes_normed_rows` accepts `ops.NormedRows` as its `h`.
     adds_residual = False
     takes_normed_rows = False
+    # Set by the model before `load`: whether the engine wants second copies of the matrices in
+    # the few-rows kernels' tile order (False, True or "thin"; see `ops.decode_weight`).
+    decode_copies = False
 
     def __init__(self, tensors: Optional[Dict[str, str]] = None):
         self.tensors: Dict[str, str] = dict(tensors or {})
@@ -84,6 +87,12 @@ class Part:
 
 
 class Mixer(Part):
+    # True: in a step of several tokens per sequence (`ctx.prefill`) the mixer also serves
+    # sequences that already hold tokens, reading what it kept of them (rows then start at
+    # `ctx.row_pos`, not at 0).  False: such a step must start every sequence at its first
+    # token; the step function refuses anything else and names the mixer.
+    takes_continuations = False
+
     def kv_spec(self) -> Optional[KVSpec]:
         """Keys/values the mixer keeps per token, or None."""
         return None

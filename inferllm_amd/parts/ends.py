@@ -55,7 +55,8 @@ class LMHead(Head):
     def load(self, tensors) -> None:
         own = self.tensors["weight"]
         self.weight = ops.decode_weight(
-            (tensors[own] if own in tensors else tensors[self.tied_fallback]).contiguous())
+            (tensors[own] if own in tensors else tensors[self.tied_fallback]).contiguous(),
+            "plain", self.decode_copies)
 
     def forward(self, h, ctx: StepContext):
         return ops.linear(h, self.weight, out_dtype=torch.float32)

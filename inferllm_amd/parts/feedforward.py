@@ -35,8 +35,9 @@ class SwiGLU(FeedForward):
 
     def load(self, tensors) -> None:
         self.w_gate_up = ops.decode_weight(_fuse([self._take(tensors, "gate"), self._take(tensors, "up")]),
-                                           "gate_up")
-        self.w_down = ops.decode_weight(self._take(tensors, "down").contiguous())
+                                           "gate_up", self.decode_copies)
+        self.w_down = ops.decode_weight(self._take(tensors, "down").contiguous(), "plain",
+                                        self.decode_copies)
 
     def forward(self, h, ctx: StepContext, residual=None, next_norm=None):
         a = ops.gate_up_silu(h, self.w_gate_up)

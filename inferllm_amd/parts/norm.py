@@ -26,7 +26,7 @@ class RMSNorm(Norm):
         self.weight: Optional[torch.Tensor] = None
 
     def shapes(self) -> Dict[str, TensorWant]:
-        return {"weight": TensorWant((self.size,), init="ones_normal")}
+        return {"weight": TensorWant((self.size,), init="ones_normal", keep_stored=True)}
 
     def load(self, tensors) -> None:
         self.weight = self._take(tensors, "weight").contiguous()

@@ -8,9 +8,17 @@ file (src/core/graph.cpp:285-331), skips unknown names with a log line
 (:311-317), asserts on a wrong element count (:322-326) and never notices a
 missing weight; here all three are errors.
 
-Stored precision is kept: bfloat16 stays bfloat16, a tensor stored in 32-bit
-stays 32-bit, float16 is widened to float32 (exact), integer tables become
-int32.  An engine that runs in float32 widens every floating tensor to float32.
+Precision in memory.  The reference gives every tensor the runtime type that the
+file's type code names (src/core/graph.cpp:216-231).  Here a floating tensor becomes
+the engine's dtype as it is loaded: in a bfloat16 engine float16 and float32
+matrices are rounded to bfloat16 (to nearest, ties to even, on the device), so that
+a checkpoint stored in float16 runs on the same kernels as one stored in bfloat16.
+Tensors that the model marks `keep_stored` (norm weights and the like: small, and
+read by kernels that take either type) keep what the file holds: bfloat16 stays
+bfloat16, 32-bit stays 32-bit, float16 is widened to float32 (exact).  With
+`keep_stored=True` for the whole load every tensor is treated so.  Integer tables
+become int32.  An engine that runs in float32 widens every floating tensor to
+float32 (exact for all three stored types).
 """
 from __future__ import annotations
 
@@ -49,6 +57,7 @@ class TensorWant:
     kind: str = "float"          # "float" or "int"
     init: str = "normal"         # random-weights rule: "normal" N(0, s) or "ones_normal" 1 + N(0, s)
     optional: bool = False       # absent is fine (e.g. a head tied to the embedding)
+    keep_stored: bool = False    # keeps the file's precision in a bfloat16 engine (norm weights)
 
 
 _FLOATS = {"F64", "F32", "F16", "BF16"}
@@ -74,21 +83,24 @@ def check_names(expected: Dict[str, TensorWant],
         raise WeightsError(sorted(missing), sorted(unexpected), wrong_shape, wrong_dtype)
 
 
-def kept_dtype(stored: torch.dtype, kind: str, engine_dtype: torch.dtype) -> torch.dtype:
+def kept_dtype(stored: torch.dtype, kind: str, engine_dtype: torch.dtype,
+               keep_stored: bool = False) -> torch.dtype:
     """The dtype a stored tensor has in memory (see the module text)."""
     if kind == "int":
         return torch.int32
     if engine_dtype == torch.float32:
         return torch.float32
-    if stored == torch.bfloat16:
+    if stored == torch.bfloat16 or not keep_stored:
         return torch.bfloat16
     return torch.float32
 
 
 def load_named_tensors(model_dir: str, expected: Dict[str, TensorWant], engine_dtype: torch.dtype,
                        device: torch.device | str,
-                       ignored_suffixes: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
-    """All expected tensors that the folder holds, on `device`, after the whole-folder check."""
+                       ignored_suffixes: Iterable[str] = (),
+                       keep_stored: bool = False) -> Dict[str, torch.Tensor]:
+    """All expected tensors that the folder holds, on `device`, after the whole-folder check.
+    `keep_stored`: no floating tensor is rounded to the engine's dtype (see the module text)."""
     files: List[SafetensorsFile] = open_model_files(model_dir)
     try:
         where: Dict[str, SafetensorsFile] = {}
@@ -111,7 +123,8 @@ def load_named_tensors(model_dir: str, expected: Dict[str, TensorWant], engine_d
                 t = where[n].read(n)
                 if w.kind == "int" and t.numel() and (int(t.max()) > 2**31 - 1 or int(t.min()) < -2**31):
                     raise WeightsError([], [], [], [(n, "integers beyond int32")])
-            out[n] = t.to(device=device, dtype=kept_dtype(t.dtype, w.kind, engine_dtype))
+            out[n] = t.to(device=device, dtype=kept_dtype(t.dtype, w.kind, engine_dtype,
+                                                          keep_stored or w.keep_stored))
         if stage is not None:
             stage.finish()
         return out

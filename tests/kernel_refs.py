@@ -180,8 +180,28 @@ def kept_distribution(logits_row, temperature, top_k, top_p, repeat_penalty, las
     return order, p
 
 
+_M64 = (1 << 64) - 1
+_GOLDEN = 0x9E3779B97F4A7C15
+
+
+def mix64(z):
+    """The output function of the splitmix64 generator (public domain, Vigna): its published
+    first outputs from state 0 are mix64(1 * golden), mix64(2 * golden), ... =
+    0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F (pinned in the kernel tests)."""
+    z &= _M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+def uniform(seed, counter):
+    """The sampler's contract, restated here and shared with nothing of the product: draw
+    `counter` of a request with 64-bit `seed` uses the top 24 bits of
+    mix64(seed + golden * (counter + 1)) as a number in [0, 1)."""
+    return (mix64((seed + _GOLDEN * (counter + 1)) & _M64) >> 40) / 16777216.0
+
+
 def sample(logits, temperature, top_k, top_p, repeat_penalty, last_tokens, seeds, counters):
-    from inferllm_amd.sampling.params import uniform
     out = []
     for b in range(logits.shape[0]):
         ids, p = kept_distribution(logits[b], temperature, top_k, top_p, repeat_penalty,

@@ -443,42 +443,55 @@ def test_products_from_the_decode_copy_equal_those_from_the_matrix(M, N, K, monk
         assert torch.equal(o.linear(x, other), o.linear(x, w))
 
 
-def test_products_of_many_rows_are_planned_once_and_stay_right():
-    """A product of many rows is measured whole and cut along its output columns, once per
-    shape; whatever plan wins, every element is the plain product."""
+def test_products_of_many_rows_follow_the_plan_and_stay_right(monkeypatch):
+    """A product of many rows runs whole or cut along its output columns as the plan's table
+    says; a plan that measures times the candidates once per shape; whatever plan is taken,
+    every element is the plain product."""
     o = ops()
+    from inferllm_amd.kernels.plan import Plan
     M, N, K = 1100, 9000, 64
     x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2)
-    o._PLANS.clear()
+    fixed = Plan()
+    monkeypatch.setattr(o, "_plan", fixed)
+    whole = o.linear(x.to(DEV), w.to(DEV))
+    assert not fixed.cuts                                  # no table entry: whole, nothing timed
+    assert torch.equal(whole, torch.matmul(x.to(DEV), w.to(DEV).t()))
+    fixed.cuts[(-(-M // 256), N, K)] = (4096,)
+    cut = o.linear(x.to(DEV), w.to(DEV))
+    close(cut, R.linear(x, w), torch.bfloat16, scale=math.sqrt(K))
+    assert torch.equal(cut[:, :4096], torch.matmul(x.to(DEV), w.to(DEV)[:4096].t()))
+    plan = Plan(measure=True)
+    monkeypatch.setattr(o, "_plan", plan)
     got = o.linear(x.to(DEV), w.to(DEV))
     key = (-(-M // 256), N, K)
-    assert key in o._PLANS and len(o._PLANS) == 1
+    assert key in plan.cuts and len(plan.cuts) == 1
     close(got, R.linear(x, w), torch.bfloat16, scale=math.sqrt(K))
-    for plan in o._split_candidates(N):                    # every candidate gives the product
-        assert all(0 < c < N for c in plan)
-        close(o._run_plan(x.to(DEV), w.to(DEV), plan), R.linear(x, w), torch.bfloat16, scale=math.sqrt(K))
+    for cand in o._split_candidates(N):                    # every candidate gives the product
+        assert all(0 < c < N for c in cand)
+        close(o._run_plan(x.to(DEV), w.to(DEV), cand), R.linear(x, w), torch.bfloat16, scale=math.sqrt(K))
     big = rnd(2048, K, dtype=torch.bfloat16, seed=3)       # many rows: also as two halves
-    plans = o._split_candidates(N, 2048)
-    assert ("rows", 2) in plans and ("rows", 2) not in o._split_candidates(N, 1100)
+    cands = o._split_candidates(N, 2048)
+    assert ("rows", 2) in cands and ("rows", 2) not in o._split_candidates(N, 1100)
     close(o._run_plan(big.to(DEV), w.to(DEV), ("rows", 2)), R.linear(big, w), torch.bfloat16, scale=math.sqrt(K))
-    o._PLANS[(8, N, K)] = ("rows", 2)                      # ragged rows of that class run whole
+    plan.cuts[(8, N, K)] = ("rows", 2)                     # ragged rows of that class run whole
     close(o.linear(big[:1900].to(DEV), w.to(DEV)), R.linear(big[:1900], w), torch.bfloat16, scale=math.sqrt(K))
-    del o._PLANS[(8, N, K)]
+    del plan.cuts[(8, N, K)]
     o.linear(x.to(DEV), w.to(DEV))
-    assert len(o._PLANS) == 1                              # measured once
+    assert len(plan.cuts) == 1                             # measured once
     o.linear(x[:1000].to(DEV), w.to(DEV))                  # fewer rows than planning is for
-    assert len(o._PLANS) == 1
+    assert len(plan.cuts) == 1
     # 65 to 255 rows: whole against filled up to 256 rows, once per shape and 32 rows
     few = x[:100].to(DEV)
     close(o.linear(few, w.to(DEV)), R.linear(x[:100], w), torch.bfloat16, scale=math.sqrt(K))
-    assert o._PLANS.get(("pad", 4, N, K)) in ((), ("pad", 256)) and len(o._PLANS) == 2
+    assert plan.cuts.get(("pad", 4, N, K)) in ((), ("pad", 256)) and len(plan.cuts) == 2
     close(o._run_plan(few, w.to(DEV), ("pad", 256)), R.linear(x[:100], w), torch.bfloat16, scale=math.sqrt(K))
     into = torch.empty(100, N, dtype=torch.bfloat16, device=DEV)
     assert o._run_plan(few, w.to(DEV), ("pad", 256), into) is into
     close(into, R.linear(x[:100], w), torch.bfloat16, scale=math.sqrt(K))
     o.linear(x[:64].to(DEV), w.to(DEV))
     o.linear(x[:256].to(DEV), w.to(DEV))
-    assert len(o._PLANS) == 2
+    assert len(plan.cuts) == 2
+    assert Plan.from_dict(plan.to_dict()) == plan
 
 
 def _prepared_rows(M, K, nw_dtype, eps, seed=5):
@@ -642,12 +655,26 @@ def interval_ok(logits_row, token, u, temperature, top_k, top_p, penalty, last):
     return False
 
 
+def test_the_uniform_numbers_of_the_tests_and_of_the_host_side_agree():
+    """The tests state the sampler's hash themselves (kernel_refs.uniform), pinned by the
+    published first outputs of splitmix64; the host side's `uniform`, which the generation loop
+    would use, must be the same function."""
+    from inferllm_amd.sampling.params import request_seed, uniform
+    assert [R.mix64(i * 0x9E3779B97F4A7C15) for i in (1, 2, 3)] == \
+        [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F]
+    for seed in (0, 3, 2**63 + 5, (1 << 64) - 1):
+        for c in (0, 1, 77):
+            assert uniform(seed, c) == R.uniform(seed, c)
+            assert 0.0 <= R.uniform(seed, c) < 1.0
+    assert len({R.uniform(request_seed(9, i), c) for i in range(4) for c in range(64)}) > 250
+
+
 @pytest.mark.parametrize("V,temperature,top_k,top_p,penalty", [
     (256, 0.8, 0, 1.0, 1.0), (320, 0.8, 40, 0.95, 1.1), (411, 0.1, 40, 0.95, 1.3), (1000, 1.5, 5, 1.0, 1.0),
     (32000, 1.0, 0, 0.9, 1.0), (300, 0.7, 1, 1.0, 1.0), (128256, 0.9, 50, 0.8, 1.2),
     (2000, 0.9, 1024, 0.7, 1.1), (2000, 0.9, 1025, 0.7, 1.0), (50, 1.0, 49, 0.5, 1.0), (32000, 0.1, 40, 0.95, 1.1)])
 def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top_p, penalty):
-    from inferllm_amd.sampling.params import uniform
+    uniform = R.uniform                                      # the tests' own statement of the hash
     B = 6
     logits = rnd(B, V, seed=8, std=2.0)
     logits[2] = 0.0                                            # all equal: ties everywhere

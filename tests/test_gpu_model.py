@@ -115,14 +115,14 @@ def test_steps_of_17_to_64_rows(tmp_path_factory, monkeypatch):
 
 @pytest.mark.parametrize("first", [1, 5, 17])
 def test_few_rows_through_the_planes_where_they_pay(tmp_path_factory, monkeypatch, first):
-    """From how few rows the down projection goes through planes is measured per shape; here it
+    """From how few rows the down projection goes through planes is a table entry per shape; here it
     is pinned (1: every step; 5: steps of 5 rows or more; 17: never below 17), and prompts of 3
     and 9 tokens and six sequences decoding together must come out as the plain model's in each."""
     from inferllm_amd import StepEntry
     from inferllm_amd.kernels import ops
     eng, plain, config = setup(tmp_path_factory, "B", "bfloat16", max_batch=8, decode_copies=True)
     shape = (config["hidden_size"], config["intermediate_size"])
-    monkeypatch.setitem(ops._PLANES_FROM, shape, first)
+    eng.plan.planes_from[shape] = first
     calls = []
     real = ops.linear_planes
     monkeypatch.setattr(ops, "linear_planes", lambda x, w, *a: calls.append(x.shape[0]) or real(x, w, *a))
@@ -148,20 +148,31 @@ def test_few_rows_through_the_planes_where_they_pay(tmp_path_factory, monkeypatc
         assert calls and min(calls) >= first and (first > 1 or 1 in calls or 2 in calls)
 
 
-def test_the_rows_from_which_planes_pay_are_measured_once_per_shape():
+def test_the_rows_from_which_planes_pay(monkeypatch):
+    """By the plan's table; a shape the table lacks follows the rule (from 17 rows) and is timed
+    only by a plan that measures, once."""
     from inferllm_amd.kernels import ops
+    from inferllm_amd.kernels.plan import Plan
     for shape, measured in (((128, 512), False), ((1024, 4096), True)):
         m = torch.randn(*shape, device="cuda", dtype=torch.bfloat16)
         w = ops.Weight(m, ops.tile_weight(m, ops.tile_rows(shape[0], "plain")), "plain")
-        ops._PLANES_FROM.pop(shape, None)
         x = torch.zeros(8, shape[1], device="cuda", dtype=torch.bfloat16)
+        x17 = torch.zeros(17, shape[1], device="cuda", dtype=torch.bfloat16)
         assert ops.linear_planes_fits(x, w)
+        fixed = Plan()
+        monkeypatch.setattr(ops, "_plan", fixed)
+        assert not ops.linear_planes_pays(x, w) and ops.linear_planes_pays(x17, w)
+        assert not fixed.planes_from                       # nothing was timed or remembered
+        fixed.planes_from[shape] = 5
+        assert ops.linear_planes_pays(x, w) and not ops.linear_planes_pays(x[:4], w)
+        tuned = Plan(measure=True)
+        monkeypatch.setattr(ops, "_plan", tuned)
         a = ops.linear_planes_pays(x, w)
-        first = ops._PLANES_FROM[shape]
+        first = tuned.planes_from[shape]
         assert first in (1, 5, 9, 13, 17) and (measured or first == 17)    # small ones: never
         assert a == (8 >= first)
-        assert ops.linear_planes_pays(torch.zeros(17, shape[1], device="cuda", dtype=torch.bfloat16), w)
-        ops._PLANES_FROM.pop(shape, None)
+        assert ops.linear_planes_pays(x17, w)
+        assert Plan.from_dict(tuned.to_dict()) == tuned and not Plan.from_dict(tuned.to_dict()).measure
 
 
 @pytest.mark.parametrize("copies", [True, False])

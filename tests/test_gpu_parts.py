@@ -183,7 +183,17 @@ def test_decode_graph_replays_equal_eager_steps(tmp_path, n_reqs):
 
 
 # ---------------------------------------------------------------- a toy mixer with state
+_toy = []
+
+
 def register_toy():
+    """Registers the toy parts and architecture once a process; returns the config class."""
+    if not _toy:
+        _toy.append(_register_toy())
+    return _toy[0]
+
+
+def _register_toy():
     from inferllm_amd.cache import StateSpec
     from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
     from inferllm_amd.parts import Mixer, register_part
@@ -220,22 +230,41 @@ def register_toy():
                 state[s, self.E] = counts[-1]
             return (out @ self.w.t()).to(h.dtype)
 
+    @register_part("mixer", "toy_running_mean_on_device")
+    class RunningMeanOnDevice(RunningMean):
+        """The same with steps of single tokens done on the device alone (no host read), so that
+        they may be captured into a graph; and it goes on from its state by any number of tokens."""
+        graph_safe = True
+        takes_continuations = True
+
+        def forward(self, h, ctx, line, writes_cache, position):
+            if ctx.prefill:
+                return super().forward(h, ctx, line, writes_cache, position)
+            state = ctx.cache.state_line(line)
+            slots = ctx.seq_slot.long()
+            now = state.index_select(0, slots)
+            now[:, :self.E] += h.float()
+            now[:, self.E] += 1
+            state.index_copy_(0, slots, now)
+            return ((now[:, :self.E] / now[:, self.E:]) @ self.w.t()).to(h.dtype)
+
     @register_architecture("ToyRunningMeanForTests")
     class ToyConfig:
-        def __init__(self, hidden_size, vocab_size, layers, eps):
-            self.E, self.V, self.L, self.eps = hidden_size, vocab_size, layers, eps
+        def __init__(self, hidden_size, vocab_size, layers, eps, mixer="toy_running_mean"):
+            self.E, self.V, self.L, self.eps, self.mixer = hidden_size, vocab_size, layers, eps, mixer
 
         @classmethod
         def from_dict(cls, d):
-            return cls(d["hidden_size"], d["vocab_size"], d["layers"], d["eps"])
+            return cls(d["hidden_size"], d["vocab_size"], d["layers"], d["eps"],
+                       d.get("mixer", "toy_running_mean"))
 
         def to_dict(self):
             return {"architectures": ["ToyRunningMeanForTests"], "hidden_size": self.E,
-                    "vocab_size": self.V, "layers": self.L, "eps": self.eps}
+                    "vocab_size": self.V, "layers": self.L, "eps": self.eps, "mixer": self.mixer}
 
         def to_spec(self):
             norm = lambda n: PartSpec("rms_norm", {"size": self.E, "eps": self.eps}, {"weight": n})
-            layers = [LayerSpec("pre_norm", PartSpec("toy_running_mean", {"hidden_size": self.E}, {"w": f"l{i}.mix"}),
+            layers = [LayerSpec("pre_norm", PartSpec(self.mixer, {"hidden_size": self.E}, {"w": f"l{i}.mix"}),
                                 PartSpec("swiglu", {"hidden_size": self.E, "intermediate_size": 2 * self.E},
                                          {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
                                 norm(f"l{i}.n1"), norm(f"l{i}.n2"), None) for i in range(self.L)]
@@ -284,6 +313,70 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     for _ in range(3):
         seq.append(int(torch.argmax(toy_plain(w, cfg, seq)[-1])))
     assert got == [seq[len(reqs[1]):]]
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_a_mixer_with_state_under_decode_graphs(tmp_path, graphs):
+    """State is not idempotent as a store of keys is: a decode step that ran twice (once to warm
+    up before the capture of its graph, once as the replay) would count a token twice.  Steps of
+    1, 2 and 3 sequences (three graphs, each captured at its first use, in the middle of the
+    sequences) must leave the running means as one pass over the tokens does."""
+    import inferllm_amd as I
+    from tiny import random_ids, read_weights
+    register_toy()
+    cfg = {"architectures": ["ToyRunningMeanForTests"], "hidden_size": 48, "vocab_size": 100, "layers": 2,
+           "eps": 1e-5, "mixer": "toy_running_mean_on_device"}
+    d = I.write_random_model(str(tmp_path / "toy"), I.config_from_dict(cfg), seed=4)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="float32", max_batch=4, max_seq_len=256, use_graphs=graphs)
+    assert eng.runner.use_graphs == graphs
+    reqs = [random_ids(n, 100, 40 + n) for n in (12, 9, 15)]
+    want = [toy_plain(w, cfg, r) for r in reqs]
+    slots = [eng.alloc_slot() for _ in reqs]
+    heads = [3, 2, 4]
+    eng.step([I.StepEntry(s, r[:h], []) for s, r, h in zip(slots, reqs, heads)])
+    at = list(heads)
+    live = [0, 1, 2]
+    while live:
+        out = eng.step([I.StepEntry(slots[i], [reqs[i][at[i]]], [0]) for i in live])
+        for j, i in enumerate(live):
+            assert rel(out[j], want[i][at[i]]) < 2e-5, (i, at[i], len(live))
+            at[i] += 1
+        live = [i for i in live if at[i] < len(reqs[i])]
+    if graphs:
+        assert {k[0] for k in eng.runner._graphs} == {1, 2, 4}
+
+
+def test_a_mixer_says_whether_it_goes_on_by_several_tokens(tmp_path):
+    """The rule "all start, or all go on by one" belongs to the mixers: attention reads a prompt's
+    keys from the step's own rows and refuses a continuation by several tokens; a mixer with
+    state of fixed size takes one, and a prompt can be cut into steps of any lengths, also mixed
+    with sequences that start."""
+    import inferllm_amd as I
+    from inferllm_amd.engine.step import StepError
+    from tiny import TINY_A, make_model_dir, random_ids, read_weights
+    register_toy()
+    cfg = {"architectures": ["ToyRunningMeanForTests"], "hidden_size": 48, "vocab_size": 100, "layers": 2,
+           "eps": 1e-5, "mixer": "toy_running_mean_on_device"}
+    d = I.write_random_model(str(tmp_path / "toy"), I.config_from_dict(cfg), seed=6)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="float32", max_batch=4, max_seq_len=256)
+    a, b = random_ids(30, 100, 1), random_ids(11, 100, 2)
+    wa, wb = toy_plain(w, cfg, a), toy_plain(w, cfg, b)
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    out = eng.step([I.StepEntry(sa, a[:7], [6])])
+    assert rel(out[0], wa[6]) < 2e-5
+    out = eng.step([I.StepEntry(sa, a[7:20], [0, 12]), I.StepEntry(sb, b[:5], [4])])   # one goes on, one starts
+    assert rel(out[0], wa[7]) < 2e-5 and rel(out[1], wa[19]) < 2e-5 and rel(out[2], wb[4]) < 2e-5
+    out = eng.step([I.StepEntry(sa, a[20:], [9]), I.StepEntry(sb, b[5:6], [0])])       # ten tokens and one
+    assert rel(out[0], wa[29]) < 2e-5 and rel(out[1], wb[5]) < 2e-5
+    # attention does not: the step function refuses and says which part is the reason
+    la = I.Engine.from_pretrained(make_model_dir(tmp_path, TINY_A, seed=1), dtype="float32", max_batch=2)
+    s = la.alloc_slot()
+    la.step([I.StepEntry(s, [1, 2, 3], [])])
+    with pytest.raises(StepError, match="Attention cannot go on by several"):
+        la.step([I.StepEntry(s, [4, 5], [1])])
+    assert la.cache.length(s) == 3                       # refused before anything was reserved
 
 
 def test_embedding_and_head_parts():

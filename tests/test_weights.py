@@ -81,16 +81,22 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert s in msg
 
 
-def test_stored_precision_is_kept():
+def test_precision_in_memory():
+    """Matrices take the engine's dtype as the reference gives every tensor the runtime type of
+    its file code (src/core/graph.cpp:216-231); tensors marked keep_stored keep the file's."""
     bf, f32, f16 = torch.bfloat16, torch.float32, torch.float16
     assert kept_dtype(bf, "float", bf) == bf
-    assert kept_dtype(f32, "float", bf) == f32          # stored in 32-bit stays so
-    assert kept_dtype(f16, "float", bf) == f32          # widened exactly
+    assert kept_dtype(f32, "float", bf) == bf           # a matrix is rounded to the engine's dtype
+    assert kept_dtype(f16, "float", bf) == bf
+    assert kept_dtype(f32, "float", bf, keep_stored=True) == f32   # stored in 32-bit stays so
+    assert kept_dtype(f16, "float", bf, keep_stored=True) == f32   # widened exactly
+    assert kept_dtype(bf, "float", bf, keep_stored=True) == bf
     assert kept_dtype(bf, "float", f32) == f32          # a float32 engine widens everything
+    assert kept_dtype(f16, "float", f32, keep_stored=True) == f32
     assert kept_dtype(torch.int64, "int", bf) == torch.int32
 
 
-def test_mixed_precision_folder_loads_as_stored(tmp_path):
+def test_mixed_precision_folder(tmp_path):
     cfg = I.config_from_dict(TINY_A)
     d = make_model_dir(tmp_path, TINY_A, seed=2, dtype=torch.bfloat16)
     w = read_weights(d)
@@ -98,12 +104,34 @@ def test_mixed_precision_folder_loads_as_stored(tmp_path):
     write_safetensors(os.path.join(d, "model.safetensors"), w.items())
     model = DecoderModel(cfg.to_spec())
     t = load_named_tensors(d, model.wants(), torch.bfloat16, "cpu")
-    assert t["model.norm.weight"].dtype == torch.float32
+    assert t["model.norm.weight"].dtype == torch.float32     # a norm weight keeps its 32 bits
     assert t["model.layers.0.input_layernorm.weight"].dtype == torch.bfloat16
     assert t["lm_head.weight"].dtype == torch.bfloat16
     t32 = load_named_tensors(d, model.wants(), torch.float32, "cpu")
     assert all(v.dtype == torch.float32 for v in t32.values())
     assert torch.equal(t32["lm_head.weight"], t["lm_head.weight"].float())
+
+
+@pytest.mark.parametrize("stored", [torch.float16, torch.float32])
+def test_float16_and_float32_folders_in_a_bfloat16_engine(tmp_path, stored):
+    """Every matrix is rounded to bfloat16 to nearest even; norm weights stay 32-bit; with
+    keep_stored nothing is rounded."""
+    cfg = I.config_from_dict(TINY_A)
+    d = make_model_dir(tmp_path, TINY_A, seed=5, dtype=stored)
+    w = read_weights(d)
+    model = DecoderModel(cfg.to_spec())
+    t = load_named_tensors(d, model.wants(), torch.bfloat16, "cpu")
+    for n, v in t.items():
+        if v.dim() == 2:
+            assert v.dtype == torch.bfloat16, n
+            assert torch.equal(v, w[n].float().to(torch.bfloat16)), n
+        else:
+            assert v.dtype == torch.float32 and torch.equal(v, w[n].float()), n
+    # ties go to the even neighbour: 1 + 2^-8 lies midway between 1 and 1 + 2^-7
+    x = torch.tensor([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8], dtype=torch.float32)
+    assert x.to(torch.bfloat16).float().tolist() == [1.0, 1.0 + 2.0 ** -6]
+    kept = load_named_tensors(d, model.wants(), torch.bfloat16, "cpu", keep_stored=True)
+    assert all(v.dtype == torch.float32 and torch.equal(v, w[n].float()) for n, v in kept.items())
 
 
 def test_sharded_folder(tmp_path):
