@@ -1,6 +1,6 @@
 // C entry points of the kernel library.  Every function launches on `stream`
 // and returns ILLM_OK, ILLM_ERR_ARG (sizes or dtypes it does not take; nothing
-// was launched) or ILLM_ERR_LAUNCH.  Pointers are device pointers.  dtype codes:
+// was launched), ILLM_ERR_LAUNCH or, where said, ILLM_ERR_SCRATCH.  Pointers are device pointers.  dtype codes:
 // 0 = float32, 1 = bfloat16.
 #pragma once
 #include <stdint.h>
@@ -74,6 +74,22 @@ int illm_attn_decode_bf16(const void* qkv, void* out, const void* kcache, const 
                           const int32_t* seq_slot, const int32_t* seq_len, float* partial,
                           int nsplit, int waves, int B, int nh, int nkv, int hd, float scale,
                           int window, void* stream);
+
+// illm_attn_decode_bf16 for callers that cannot allocate device memory (code under HIP graph
+// capture, tight serving loops, harnesses that forbid it): it has no counterpart in the
+// reference.  The split results go through an array that the library holds on every GPU it runs
+// on (ILLM_DECODE_SCRATCH_BYTES, until the process ends) instead of a `partial` argument; the call
+// allocates and frees nothing.  B * nh * nsplit * (hd + 2) * 4 bytes must fit the array, else
+// ILLM_ERR_SCRATCH (3) and nothing is launched; nsplit == 1 uses no scratch.  All calls on one GPU
+// share the array, so calls that overlap on one GPU (two streams) race: run them one after the
+// other.  Nothing needs clearing between calls: every entry that is read was written by the same
+// call before.
+#define ILLM_DECODE_SCRATCH_BYTES (4u << 20)
+int illm_attn_decode_bf16_static(const void* qkv, void* out, const void* kcache,
+                                 const void* vcache, const int32_t* page_table, int table_stride,
+                                 int page_size, int ring, const int32_t* seq_slot,
+                                 const int32_t* seq_len, int nsplit, int waves, int B, int nh,
+                                 int nkv, int hd, float scale, int window, void* stream);
 
 // Y[M, N] = X[M, K] . W[N, K]^T for bfloat16 X and W, 1 <= M <= 64, K % 8 == 0, on the
 // matrix cores with float32 accumulation; Y float32 or bfloat16.

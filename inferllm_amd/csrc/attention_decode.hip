@@ -15,6 +15,8 @@
 // src/kern/naive/naive.cpp:576-604.
 #include <math.h>
 
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -908,4 +910,50 @@ extern "C" int illm_attn_decode_bf16(const void* qkv, void* out, const void* kca
         default: GO(32);
     }
 #undef GO
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same decode attention for callers that cannot allocate device memory: the split results go
+// through a file-scope array instead of a workspace argument.  Each GPU holds its own copy of the
+// array at its own address, which the host learns once per device from the runtime; host code
+// never passes the array's name to a kernel.
+static __device__ __align__(256) float scratch[ILLM_DECODE_SCRATCH_BYTES / sizeof(float)];
+
+#define ILLM_MAX_DEVICES 64
+static float* scratch_of_device[ILLM_MAX_DEVICES];     // null until the device's first call
+static std::mutex scratch_lock;
+
+// The address of `scratch` on the current device, looked up at the device's first call.
+static int scratch_here(float** p) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ILLM_MAX_DEVICES) return ILLM_ERR_LAUNCH;
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_of_device[dev]) {
+        void* q = nullptr;
+        if (hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)) != hipSuccess || !q) return ILLM_ERR_LAUNCH;
+        scratch_of_device[dev] = (float*)q;
+    }
+    *p = scratch_of_device[dev];
+    return ILLM_OK;
+}
+
+extern "C" int illm_attn_decode_bf16_static(const void* qkv, void* out, const void* kcache,
+                                            const void* vcache, const int32_t* page_table,
+                                            int table_stride, int page_size, int ring,
+                                            const int32_t* seq_slot, const int32_t* seq_len,
+                                            int nsplit, int waves, int B, int nh, int nkv, int hd,
+                                            float scale, int window, void* stream) {
+    if (B < 0 || nh <= 0 || nsplit <= 0 || hd <= 0) return ILLM_ERR_ARG;
+    float* partial = nullptr;
+    if (nsplit > 1) {
+        const size_t need = (size_t)B * nh * nsplit * (size_t)(hd + 2) * sizeof(float);
+        if (need > ILLM_DECODE_SCRATCH_BYTES) return ILLM_ERR_SCRATCH;
+        const int rc = scratch_here(&partial);
+        if (rc != ILLM_OK) return rc;
+    }
+    // every (sequence, head, split) entry that the merge reads is written by the first kernel of
+    // this call (a split without keys leaves max = -inf, sum = 0), so nothing has to be cleared
+    return illm_attn_decode_bf16(qkv, out, kcache, vcache, page_table, table_stride, page_size, ring,
+                                 seq_slot, seq_len, partial, nsplit, waves, B, nh, nkv, hd, scale,
+                                 window, stream);
 }

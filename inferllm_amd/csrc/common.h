@@ -10,6 +10,7 @@
 #define ILLM_OK 0
 #define ILLM_ERR_ARG 1      // a size or dtype the kernel does not take
 #define ILLM_ERR_LAUNCH 2   // the runtime refused the launch
+#define ILLM_ERR_SCRATCH 3  // the call needs more of the library's own scratch memory than it has
 
 #define ILLM_WAVE 64
 

@@ -34,7 +34,8 @@ from .plan import NEVER_BELOW, Plan
 
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
-_ERRORS = {1: "sizes or dtypes the kernel does not take", 2: "the HIP runtime refused the launch"}
+_ERRORS = {1: "sizes or dtypes the kernel does not take", 2: "the HIP runtime refused the launch",
+           3: "the call needs more of the library's own scratch memory than it holds"}
 
 
 class KernelError(RuntimeError):
