@@ -8,9 +8,10 @@ stopwatch, or the same request could give other bfloat16 logits in another proce
 the choice is a table by shape:
 
 * `Plan.fixed()` (what an engine uses unless told otherwise): the tables below, measured once
-  on an MI355X for the matrix shapes of LLaMA-2-7B, LLaMA-3-8B and LLaMA-2-70B
-  (`python -m inferllm_amd.kernels.tune`), and for every other shape one rule: planes from 17
-  rows on, products of many rows whole.  Nothing is ever timed.
+  on an MI355X for the matrix shapes of LLaMA-2-7B, LLaMA-2-13B, LLaMA-3-8B and LLaMA-2-70B
+  (`python -m inferllm_amd.kernels.tune`: the majority of three measurements, and a way other
+  than the rule's must win by 7 %), and for every other shape one rule: planes from 17 rows on,
+  products of many rows whole.  Nothing is ever timed.
 * `Plan(measure=True)` (`Engine(tune=True)`): a shape that the tables lack is timed the first
   time it is used outside graph capture and the winner is kept; `to_dict()` gives the result,
   which `Engine(plan=...)` pins in another process.
@@ -26,12 +27,97 @@ NEVER_BELOW = 17          # planes are not taken below 17 rows (the rule for unl
 # (N, K) of a matrix with K >= 2 N -> fewest rows (1, 5, 9, 13 or 17) from which the planes and
 # the norm that adds them take less time than the residual-adding few-rows product.
 FIXED_PLANES_FROM: Dict[Tuple[int, int], int] = {
+    (4096, 11008): 13,
+    (4096, 14336): 9,
+    (5120, 13824): 1,
+    (8192, 28672): 5,
 }
 
 # (rows / 256 rounded up, N, K) -> plan of a product of at least 1024 rows and 8192 columns:
 # () whole, (c,) cut of the output columns at c, ("rows", n) the rows in n equal parts.
 # ("pad", rows / 32 rounded up, N, K) -> () or ("pad", 256) for products of 65 to 255 rows.
 FIXED_CUTS: Dict[tuple, tuple] = {
+    ('pad', 4, 4096, 11008): ('pad', 256),
+    ('pad', 4, 4096, 14336): ('pad', 256),
+    ('pad', 5, 4096, 11008): ('pad', 256),
+    ('pad', 5, 4096, 14336): ('pad', 256),
+    ('pad', 6, 4096, 11008): ('pad', 256),
+    ('pad', 6, 4096, 14336): ('pad', 256),
+    (10, 27648, 5120): (12288,),
+    (11, 22016, 4096): (12288,),
+    (11, 27648, 5120): (12288,),
+    (11, 8192, 8192): (4096,),
+    (12, 22016, 4096): (8192,),
+    (12, 27648, 5120): (8192,),
+    (12, 57344, 8192): (8192,),
+    (13, 15360, 5120): (7680,),
+    (13, 22016, 4096): (8192,),
+    (13, 28672, 4096): (12288,),
+    (13, 8192, 28672): (4096,),
+    (14, 10240, 8192): (4096,),
+    (14, 15360, 5120): (7680,),
+    (14, 22016, 4096): (8192,),
+    (14, 28672, 4096): (8192,),
+    (15, 10240, 8192): (4096,),
+    (15, 22016, 4096): (11008,),
+    (15, 27648, 5120): (24576,),
+    (15, 8192, 28672): (4096,),
+    (16, 10240, 8192): (4096,),
+    (16, 22016, 4096): (8192,),
+    (16, 27648, 5120): (12288,),
+    (17, 10240, 8192): (4096,),
+    (17, 12288, 4096): (6144,),
+    (17, 22016, 4096): (16384,),
+    (17, 8192, 8192): (4096,),
+    (18, 15360, 5120): (7680,),
+    (18, 22016, 4096): (8192,),
+    (19, 10240, 8192): (4096,),
+    (19, 8192, 8192): (4096,),
+    (20, 10240, 8192): (4096,),
+    (20, 22016, 4096): (11008,),
+    (20, 28672, 4096): (12288,),
+    (20, 8192, 28672): (4096,),
+    (20, 8192, 8192): (4096,),
+    (21, 10240, 8192): (4096,),
+    (21, 22016, 4096): (20480,),
+    (21, 27648, 5120): (12288,),
+    (21, 28672, 4096): (8192,),
+    (22, 15360, 5120): (7680,),
+    (23, 8192, 8192): (4096,),
+    (24, 12288, 4096): (6144,),
+    (24, 22016, 4096): (20480,),
+    (24, 28672, 4096): (8192,),
+    (25, 22016, 4096): (20480,),
+    (25, 27648, 5120): (12288,),
+    (25, 28672, 4096): (8192,),
+    (26, 10240, 8192): (4096,),
+    (26, 27648, 5120): (8192,),
+    (27, 10240, 8192): (4096,),
+    (27, 12288, 4096): (6144,),
+    (27, 15360, 5120): (8192,),
+    (27, 22016, 4096): (8192,),
+    (28, 10240, 8192): (4096,),
+    (28, 22016, 4096): (8192,),
+    (28, 8192, 28672): ('rows', 2),
+    (29, 15360, 5120): (12288,),
+    (29, 28672, 4096): (12288,),
+    (30, 15360, 5120): (7680,),
+    (30, 22016, 4096): (12288,),
+    (31, 15360, 5120): (8192,),
+    (31, 22016, 4096): (20480,),
+    (32, 22016, 4096): (20480,),
+    (32, 27648, 5120): (12288,),
+    (4, 27648, 5120): (12288,),
+    (5, 28672, 4096): (24576,),
+    (6, 22016, 4096): (20480,),
+    (6, 27648, 5120): (8192,),
+    (7, 10240, 8192): (8192,),
+    (7, 22016, 4096): (8192,),
+    (7, 28672, 4096): (12288,),
+    (8, 10240, 8192): (8192,),
+    (8, 22016, 4096): (8192,),
+    (8, 27648, 5120): (12288,),
+    (9, 22016, 4096): (8192,),
 }
 
 
