@@ -8,9 +8,16 @@ feed-forward 11008, vocabulary 32000) with seeded random bfloat16 weights, a bat
 of 8 sequences with 512-token prompts that decode 256 tokens (8 more to warm up),
 cache context 4096.  A step is one decode step of the whole batch: step function, greedy choice on the device, the tokens
 back on the host.  One JSON line is printed: decoded tokens per second, the
-prefill of 2,048 tokens, the decode step against the HBM roofline, and decoding
-at batch 1 and 64.  Peaks are the published ones of MI355X (HBM 8 TB/s, dense
-bf16 MFMA 2.5 PFLOP/s, float32 157.3 TFLOP/s).
+prefill of 2,048 tokens, the decode step against the HBM roofline, and under
+`points` decoding at batch 1 and 64, decoding from 3,800-token contexts at batch
+8 and 64, and the LLaMA-3-8B shape with 16 prompts of 64 to 4,096 tokens through the
+generation loop (`--with-70b` adds the LLaMA-2-70B shape: prefill of 2,048 tokens,
+decode at batch 1 and 32 from 1,024-token prompts).  Every decode point has a
+`..._hbm_frac` beside it: the bytes its step has to read (every weight once, the
+cache of its live sequences) / its time / the HBM peak.  Peaks are the published ones
+of MI355X (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, float32 157.3 TFLOP/s).
+The run fails (non-zero) if any timed run produced a non-finite logit or the same
+greedy token everywhere.
 """
 import argparse
 import json
@@ -49,68 +56,66 @@ def kv_bytes_per_token(cfg, layers, esz):
     return layers * 2 * nkv * hd * esz
 
 
-def prefill_flops(cfg, layers, T, out_rows=1):
+def prefill_flops(cfg, layers, T, out_rows=1, lens=None):
+    """Flops of a prefill of T tokens (`lens`: the prompts' lengths if more than one)."""
     E, F, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nh, nkv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
     hd = cfg.get("head_dim", E // nh)
     linear = 2.0 * T * ((nh + 2 * nkv) * hd * E + E * nh * hd + 3 * E * F)
-    attn = 2.0 * 2.0 * nh * hd * (T * (T + 1) / 2)
+    attn = sum(2.0 * 2.0 * nh * hd * (n * (n + 1) / 2) for n in (lens or [T]))
     return layers * (linear + attn) + 2.0 * out_rows * V * E
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
-    ap.add_argument("--prompt", type=int, default=512)
-    ap.add_argument("--shape", default="llama2-7b", choices=sorted(SHAPES),
-                    help="layer sizes (default: the headline configuration)")
-    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
-    ap.add_argument("--prefill-only", action="store_true",
-                    help="run only the 2,048-token prefill (for profiles); prints its own line")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
-        return 2
+class Bench:
+    """One engine of one shape and the runs on it."""
 
-    import torch
-    from inferllm_amd import Engine, StepEntry
-    from inferllm_amd.kernels import ops
-    from inferllm_amd.sampling import Sampler, SamplingParams
+    def __init__(self, cfg, layers, dtype, max_batch, max_tokens, seed=1234):
+        import torch
+        from inferllm_amd import Engine
+        self.torch = torch
+        self.cfg = dict(cfg)
+        self.full_layers = cfg["num_hidden_layers"]
+        self.layers = layers or self.full_layers
+        self.cfg["num_hidden_layers"] = self.layers
+        self.esz = 2 if dtype == "bfloat16" else 4
+        self.dkey = "bf16" if dtype == "bfloat16" else "fp32"
+        t0 = time.time()
+        self.eng = Engine.from_random(self.cfg, seed=0, dtype=dtype, device="cuda:0",
+                                      max_batch=max_batch, max_seq_len=cfg["max_position_embeddings"],
+                                      max_tokens=max_tokens)
+        torch.cuda.synchronize()
+        print(f"[bench] engine ready in {time.time() - t0:.1f} s "
+              f"({self.layers} layers, room for {max_tokens} tokens)", file=sys.stderr, flush=True)
+        self.g = torch.Generator().manual_seed(seed)
 
-    shape_name, shape_cfg = SHAPES[args.shape]
-    cfg = dict(shape_cfg)
-    full_layers = cfg["num_hidden_layers"]
-    layers = args.layers or full_layers
-    cfg["num_hidden_layers"] = layers
-    ctx_len = cfg["max_position_embeddings"]
-    esz = 2 if args.dtype == "bfloat16" else 4
-    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
-    dev = "cuda:0"
-    max_b = max(args.batch, 1 if args.no_points else 64)
-    per_seq = -(-(args.prompt + args.steps + args.warmup + 2) // 64) * 64     # whole cache pages
-    room = max(max_b * max(per_seq, 1024), 4096)
-    t0 = time.time()
-    eng = Engine.from_random(cfg, seed=0, dtype=args.dtype, device=dev, max_batch=max_b,
-                             max_seq_len=ctx_len, max_tokens=room)
-    torch.cuda.synchronize()
-    print(f"[bench] engine ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
-    g = torch.Generator().manual_seed(1234)
+    def close(self):
+        self.eng = None
+        import gc
+        gc.collect()
+        self.torch.cuda.empty_cache()
 
-    def decode_run(batch, steps, warmup):
-        """tokens/s, ms/step, mean context of `steps` timed decode steps of `batch` sequences."""
-        prompts = [torch.randint(0, cfg["vocab_size"], (args.prompt,), generator=g).tolist()
-                   for _ in range(batch)]
+    def ids(self, n):
+        return self.torch.randint(0, self.cfg["vocab_size"], (n,), generator=self.g).tolist()
+
+    def step_bytes(self, batch, mean_ctx):
+        return (weight_bytes_per_step(self.cfg, self.layers, self.esz)
+                + batch * mean_ctx * kv_bytes_per_token(self.cfg, self.layers, self.esz))
+
+    def decode_run(self, batch, steps, warmup, prompt):
+        """(tokens/s, ms/step, fraction of the HBM peak) of `steps` timed decode steps of `batch`
+        sequences that start from prompts of `prompt` tokens."""
+        from inferllm_amd import StepEntry
+        from inferllm_amd.kernels import ops
+        from inferllm_amd.sampling import Sampler, SamplingParams
+        torch, eng = self.torch, self.eng
+        prompts = [self.ids(prompt) for _ in range(batch)]
         slots = [eng.alloc_slot() for _ in range(batch)]
-        # prompts go in pieces of at most 8 sequences to bound the prefill's activations
+        # prompts go in pieces of at most 16,384 tokens to bound the prefill's activations
+        per = max(1, 16384 // prompt)
         toks = [0] * batch
-        for i in range(0, batch, 8):
-            part = list(range(i, min(batch, i + 8)))
-            logits = eng.step([StepEntry(slots[j], prompts[j], [args.prompt - 1]) for j in part])
+        for i in range(0, batch, per):
+            part = list(range(i, min(batch, i + per)))
+            logits = eng.step([StepEntry(slots[j], prompts[j], [prompt - 1]) for j in part])
             for j, t in zip(part, ops.argmax(logits.contiguous()).tolist()):
                 toks[j] = t
 
@@ -119,7 +124,6 @@ def main() -> int:
         sampler = Sampler(SamplingParams(), eng.device)             # greedy
         draw = sampler.draw(eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)]),
                             [0] * batch, [0] * batch)
-
         seen = []
 
         def one():
@@ -139,22 +143,27 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         # what was timed must have computed something: finite logits, and greedy tokens that
-        # change from step to step (a run on NaN or constant logits would be as fast)
+        # are not one and the same everywhere (a run on NaN or constant logits would be as fast)
         if not bool(torch.isfinite(logits).all()):
             raise SystemExit(f"bench: non-finite logits in the decode run at batch {batch}")
         distinct = {int(t) for row in seen for t in row}
-        print(f"[bench] batch {batch}: {len(distinct)} distinct greedy tokens in {len(seen)} steps",
-              file=sys.stderr, flush=True)
+        print(f"[bench] batch {batch}, prompts of {prompt}: {dt / steps * 1e3:.3f} ms a step, "
+              f"{len(distinct)} distinct greedy tokens in {len(seen)} steps", file=sys.stderr, flush=True)
         if len(seen) >= 16 and len(distinct) < 2:
             raise SystemExit(f"bench: the greedy token is {sorted(distinct)} in every step of every "
                              f"sequence at batch {batch}: the logits are degenerate")
-        mean_ctx = args.prompt + 1 + warmup + (steps + 1) / 2.0
+        mean_ctx = prompt + 1 + warmup + (steps + 1) / 2.0
         for s in slots:
             eng.free_slot(s)
-        return batch * steps / dt, dt / steps * 1e3, mean_ctx
+        ms = dt / steps * 1e3
+        frac = self.step_bytes(batch, mean_ctx) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        return batch * steps / dt, ms, frac
 
-    def prefill_run(T=2048, reps=3):
-        ids = torch.randint(0, cfg["vocab_size"], (T,), generator=g).tolist()
+    def prefill_run(self, T=2048, reps=3):
+        from inferllm_amd import StepEntry
+        from inferllm_amd.kernels import ops
+        torch, eng = self.torch, self.eng
+        ids = self.ids(T)
         times = []
         for i in range(reps):
             s = eng.alloc_slot()
@@ -168,24 +177,77 @@ def main() -> int:
                 raise SystemExit("bench: non-finite logits in the prefill")
             eng.free_slot(s)
         pt = min(times[1:])
-        fl = prefill_flops(cfg, layers, T)
+        fl = prefill_flops(self.cfg, self.layers, T)
         return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
+                "frac": round(fl / pt / (PEAK_TFLOPS[self.dkey] * 1e12), 4)}
+
+    def generate_run(self, lens, new_tokens):
+        """Prompts of the given lengths through `Engine.generate` (all in one batch), twice; the
+        second run's figures: (prefill tokens/s, its fraction of the matrix peak, decode tokens/s,
+        its fraction of the HBM peak)."""
+        prompts = [self.ids(n) for n in lens]
+        for _ in range(2):
+            out = self.eng.generate(prompts, max_new_tokens=new_tokens, stop_token_ids=[])
+            st = self.eng.last_stats
+        assert all(len(o) == new_tokens for o in out)
+        if len({t for o in out for t in o}) < 2:
+            raise SystemExit("bench: the generation loop produced one and the same token everywhere")
+        B, T = len(lens), sum(lens)
+        pf = T / st.prefill_seconds
+        pf_frac = (prefill_flops(self.cfg, self.layers, T, B, lens) / st.prefill_seconds
+                   / (PEAK_TFLOPS[self.dkey] * 1e12))
+        steps = st.decode_steps
+        ms = st.decode_seconds / steps * 1e3
+        mean_ctx = T / B + 1 + (steps + 1) / 2.0
+        frac = self.step_bytes(B, mean_ctx) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        return pf, pf_frac, B * steps / st.decode_seconds, frac
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--shape", default="llama2-7b", choices=sorted(SHAPES),
+                    help="layer sizes (default: the headline configuration)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip everything under `points` and the prefill")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill (for profiles); prints its own line")
+    ap.add_argument("--with-70b", action="store_true",
+                    help="add the LLaMA-2-70B shape to `points` (138 GB of weights: minutes)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
+        return 2
+
+    shape_name, shape_cfg = SHAPES[args.shape]
+    ctx_len = shape_cfg["max_position_embeddings"]
+    headline = args.shape == "llama2-7b" and args.dtype == "bfloat16" and not args.no_points
+    long_ctx = 3800
+    max_b = max(args.batch, 1 if args.no_points else 64)
+    per_seq = -(-(args.prompt + args.steps + args.warmup + 2) // 64) * 64     # whole cache pages
+    room = max(max_b * max(per_seq, 1024), 4096)
+    if headline:
+        room = max(room, 64 * (-(-(long_ctx + 64 + 8) // 64) * 64))
+    b = Bench(shape_cfg, args.layers, args.dtype, max_b, room)
+    cfg, layers = b.cfg, b.layers
 
     if args.prefill_only:
-        print(json.dumps({"prefill": prefill_run(reps=max(3, args.steps))}), flush=True)
+        print(json.dumps({"prefill": b.prefill_run(reps=max(3, args.steps))}), flush=True)
         return 0
 
-    tps, ms, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
-    step_bytes = weight_bytes_per_step(cfg, layers, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, layers, esz)
-    achieved = step_bytes / (ms * 1e-3) / 1e9
+    tps, ms, frac = b.decode_run(args.batch, args.steps, args.warmup, args.prompt)
     out = {
         "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2,048 tokens (LLaMA-2-7B)",
         "value_is": f"decode tokens/s at batch {args.batch}", "value": round(tps, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": dkey, "data": "synthetic: seeded random weights N(0, 0.02), uniform random token ids",
-        "config": {"model": shape_name, "layers": layers, "layers_full": full_layers,
+        "vs_baseline": None, "dtype": b.dkey, "data": "synthetic: seeded random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": shape_name, "layers": layers, "layers_full": b.full_layers,
                    "hidden_size": cfg["hidden_size"], "intermediate_size": cfg["intermediate_size"],
                    "num_attention_heads": cfg["num_attention_heads"],
                    "num_key_value_heads": cfg["num_key_value_heads"],
@@ -193,14 +255,44 @@ def main() -> int:
                    "vocab_size": cfg["vocab_size"], "global_batch": args.batch,
                    "seq_len": ctx_len, "prompt_len": args.prompt, "rope_theta": cfg["rope_theta"],
                    "rms_norm_eps": cfg["rms_norm_eps"], "parallelism": "single GPU"},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(frac * HBM_PEAK_GBS, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(frac, 4)},
     }
     if not args.no_points:
-        out["prefill"] = prefill_run()
-        b1, _, _ = decode_run(1, min(args.steps, 256), 4)
-        b64, _, _ = decode_run(64, min(args.steps, 256), 4)
-        out["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
+        out["prefill"] = b.prefill_run()
+        points = {}
+        few = min(args.steps, 256)
+        for name, batch in (("decode_b1", 1), ("decode_b64", 64)):
+            v, _, f = b.decode_run(batch, few, 4, args.prompt)
+            points[name], points[name + "_hbm_frac"] = round(v, 2), round(f, 4)
+        if headline:
+            # long contexts: the cache's share of a step's bytes grows from a seventh to nine tenths
+            for name, batch in (("decode_b8_ctx3800", 8), ("decode_b64_ctx3800", 64)):
+                v, _, f = b.decode_run(batch, 64, 4, long_ctx)
+                points[name], points[name + "_hbm_frac"] = round(v, 2), round(f, 4)
+            b.close()
+            # LLaMA-3-8B shape (grouped heads, vocabulary 128,256): 16 prompts of 64 to 4,096
+            # tokens, lengths seeded, one batch through the generation loop, 128 new tokens each
+            import torch
+            lens = torch.randint(64, 4097, (16,), generator=torch.Generator().manual_seed(16)).tolist()
+            total = sum(-(-(n + 130) // 64) * 64 for n in lens)
+            b8 = Bench(LLAMA3_8B, 0, args.dtype, 16, total)
+            pf, pf_frac, dc, dc_frac = b8.generate_run(lens, 128)
+            points.update({"llama3_8b_ragged16_prompt_tokens": sum(lens),
+                           "llama3_8b_ragged16_prefill": round(pf, 1),
+                           "llama3_8b_ragged16_prefill_frac": round(pf_frac, 4),
+                           "llama3_8b_ragged16_decode": round(dc, 2),
+                           "llama3_8b_ragged16_decode_hbm_frac": round(dc_frac, 4)})
+            b8.close()
+            if args.with_70b:
+                b70 = Bench(LLAMA2_70B, 0, args.dtype, 32, 32 * 1280)
+                p70 = b70.prefill_run()
+                points.update({"llama2_70b_prefill": p70["value"], "llama2_70b_prefill_frac": p70["frac"]})
+                for name, batch in (("llama2_70b_decode_b1", 1), ("llama2_70b_decode_b32", 32)):
+                    v, _, f = b70.decode_run(batch, 128, 4, 1024)
+                    points[name], points[name + "_hbm_frac"] = round(v, 2), round(f, 4)
+                b70.close()
+        out["points"] = points
     print(json.dumps(out), flush=True)
     return 0
 
