@@ -130,6 +130,26 @@ void illm_set_skinny_one_shot(int on);
 // products on the matrix cores (default 1).
 void illm_set_gqa_pv_on_matrix_cores(int on);
 
+// Products of 1 to 128 bfloat16 rows (meant for 9 and more; 64 rows a launch) from the tiled copy
+// Wt of W, K a multiple of 64, X shared by a block's waves through LDS, K cut inside the block
+// (csrc/gemm_rows.hip).  illm_gemm_rows_bf16: Y[M, N] = X . W^T (plain tiles), float32 or bfloat16.
+// illm_gemm_rows_gateup_silu: Y[M, F] = silu(X . Wg^T) * (X . Wu^T) from the gate|up tiles.
+// illm_qkv_rope_store_rows: as illm_qkv_rope_store_skinny, from the q|k|v tiles.  ssq (M <= 16
+// only): as for illm_gemm_skinny_bf16.
+int illm_gemm_rows_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M, int N, int K,
+                        const float* ssq, int parts, float eps, void* stream);
+int illm_gemm_rows_gateup_silu(const void* X, const void* Wt, void* Y, int y_dt, int M, int F,
+                               int K, const float* ssq, int parts, float eps, void* stream);
+int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int K,
+                             const float* cos_sin, int max_pos, const int32_t* row_pos,
+                             const int32_t* row_slot, void* kcache, void* vcache,
+                             const int32_t* page_table, int table_stride, int page_size, int ring,
+                             int nh, int nkv, int hd, const float* ssq, int parts, float eps,
+                             void* stream);
+// Tuning and tests: tiles a block of these products takes (2, 3, 4), parts of K (1, 2, 4) and
+// k-steps of 32 in a piece (2, 4); 0: the library's own choice.
+void illm_set_rows_shape(int tb, int kp, int piece);
+
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
 // product, `ssq` included.  waves_wanted: waves per block (0: the default choice).
 int illm_gemm_skinny_gateup_silu(const void* X, const void* W, const void* Wt, void* Y, int y_dt,

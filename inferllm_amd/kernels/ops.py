@@ -474,6 +474,9 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
             return gemm_skinny_bf16(x, w, out_dtype or x.dtype)
         x = x.rows()
     out_dtype = out_dtype or x.dtype
+    if (isinstance(w, Weight) and out_dtype == torch.float32 and x.shape[0] >= ROWS_FROM
+            and rows_fits(x, w, "plain")):
+        return linear_rows(x, w, out_dtype)              # logits of 17 to 128 rows
     if isinstance(w, Weight) and not (x.dtype == torch.bfloat16 and 1 <= x.shape[0] <= SKINNY_BEST_ROWS):
         w = w.plain                                      # only the few-rows kernel reads the copy
     if x.dtype == torch.float32 or w.dtype == torch.float32:
@@ -589,6 +592,35 @@ def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return _run_plan(x, w, plan)
 
 
+ROWS_MAX = 128           # rows the products of csrc/gemm_rows.hip take (64 a launch)
+ROWS_FROM = 17           # from this many rows they are taken (up to 16: the few-rows kernels)
+
+
+def rows_fits(x, w, mode: str) -> bool:
+    """Whether the products of csrc/gemm_rows.hip take these operands: bfloat16 rows (or
+    `NormedRows`, up to 16) and a weight with a decode copy in `mode`'s tile order."""
+    xt = x.xb if isinstance(x, NormedRows) else x
+    return (isinstance(w, Weight) and w.tiled is not None and w.mode == mode
+            and isinstance(xt, torch.Tensor) and xt.dtype == torch.bfloat16 and xt.dim() == 2
+            and 1 <= xt.shape[0] <= (16 if isinstance(x, NormedRows) else ROWS_MAX)
+            and xt.shape[1] == w.plain.shape[1] and xt.shape[1] % 64 == 0)
+
+
+def linear_rows(x, w: "Weight", out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M <= 128, K] . w^T from the plain decode copy, X shared by a block's waves through LDS
+    and K cut inside the block: the product of 17 to 128 rows with a wide matrix."""
+    _need(rows_fits(x, w, "plain"), "linear_rows: operands not taken")
+    xt, ssq, parts, eps = _operand(x)
+    xt = xt.contiguous()
+    _gpu(xt, w.tiled)
+    M, K = xt.shape
+    N = w.plain.shape[0]
+    y = torch.empty((M, N), dtype=out_dtype, device=xt.device)
+    _check(_lib().illm_gemm_rows_bf16(_p(xt), _p(w.tiled), _p(y), _code(y), M, N, K, ssq, parts,
+                                      eps, _stream()), "linear_rows")
+    return y
+
+
 SKINNY_MAX_ROWS = 64     # rows the few-rows kernel takes
 SKINNY_BEST_ROWS = 16    # up to here it beats the vendor GEMM (measured at the 7B shapes)
 
@@ -622,9 +654,13 @@ PLAIN_WAVES = 0          # and for the plain few-rows product
 
 
 def qkv_rope_store_fits(x, w_qkv, hd: int) -> bool:
-    """Whether the one-kernel q|k|v product + rotation + cache store takes these operands."""
-    return (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and
-            1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0 and hd % 16 == 0)
+    """Whether the one-kernel q|k|v product + rotation + cache store takes these operands: up to
+    16 rows always, up to 128 with a decode copy of the matrix in q|k|v tile order."""
+    if not (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and hd % 16 == 0):
+        return False
+    if 1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0:
+        return True
+    return rows_fits(x, w_qkv, "qkv")
 
 
 def qkv_rope_store(x, w_qkv, cos_sin: torch.Tensor,
@@ -648,6 +684,12 @@ def qkv_rope_store(x, w_qkv, cos_sin: torch.Tensor,
           vcache.shape == kcache.shape and vcache.dtype == torch.bfloat16 and page_table.dim() == 2,
           "qkv_rope_store: cache shape or dtype")
     y = torch.empty((M, N), dtype=torch.bfloat16, device=xt.device)
+    if M >= ROWS_FROM:
+        _check(_lib().illm_qkv_rope_store_rows(
+            _p(xt), wt, _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
+            _p(kcache), _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, nh, nkv,
+            hd, ssq, parts, eps, _stream()), "qkv_rope_store (rows)")
+        return y
     _check(_lib().illm_qkv_rope_store_skinny(
         _p(xt), _p(w_qkv), wt, _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
         _p(kcache), _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, nh, nkv, hd,
@@ -674,6 +716,14 @@ def gate_up_silu(x, w_gate_up) -> torch.Tensor:
         _check(_lib().illm_gemm_skinny_gateup_silu(_p(xt), _p(wp), wt, _p(y), _code(y), M,
                                                    F2 // 2, K, ssq, parts, eps, GATE_UP_WAVES,
                                                    _stream()), "gate_up_silu")
+        return y
+    if M >= ROWS_FROM and F2 % 2 == 0 and rows_fits(x, w_gate_up, "gate_up"):
+        x = x.contiguous()
+        _gpu(x, w_gate_up.tiled)
+        y = torch.empty((M, F2 // 2), dtype=x.dtype, device=x.device)
+        _check(_lib().illm_gemm_rows_gateup_silu(_p(x), _p(w_gate_up.tiled), _p(y), _code(y), M,
+                                                 F2 // 2, K, None, 0, ctypes.c_float(0.0),
+                                                 _stream()), "gate_up_silu (rows)")
         return y
     if isinstance(x, NormedRows):
         x = x.rows()

@@ -781,3 +781,115 @@ def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed, copy):
     for gotc, wantc in ((kc_g.cpu(), kr), (vc_g.cpu(), vr)):
         assert torch.equal(torch.isnan(gotc), torch.isnan(wantc))        # the same rows, nothing else
         close(torch.nan_to_num(gotc), torch.nan_to_num(wantc), dtype, scale=sc)
+
+
+# ---------------------------------------------------------------- products of 9 to 128 rows
+# (tiles a block, parts of K, k-steps in a piece)
+_ROWS_SHAPES = [(None, None, None), (2, 1, 2), (2, 4, 4), (3, 2, 2), (3, 2, 4), (4, 1, 4), (4, 4, 2)]
+
+
+@pytest.fixture
+def rows_shape():
+    """Forces the block shape of the rows kernels and gives the library's own choice back after."""
+    lib = ops()._lib()
+    yield lambda tb, kp, ps=0: lib.illm_set_rows_shape(tb or 0, kp or 0, ps or 0)
+    lib.illm_set_rows_shape(0, 0, 0)
+
+
+@pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
+@pytest.mark.parametrize("M,N,K", [(17, 40, 128), (33, 100, 192), (64, 12288, 4096), (9, 320, 64), (1, 64, 64),
+                                   (65, 411, 320), (128, 1000, 1088), (48, 32000, 256), (100, 8, 4096)])
+def test_linear_rows(M, N, K, tb, kp, ps, rows_shape):
+    """The product with X shared through LDS and K cut inside the block, in every block shape,
+    float32 and bfloat16 results; row counts around the tile and launch edges (16, 64)."""
+    o = ops()
+    rows_shape(tb, kp, ps)
+    x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2, std=0.2)
+    wc = _decode_copy(w.to(DEV))
+    want = R.linear(x, w, torch.float64)
+    for ydt in DTYPES:
+        got = o.linear_rows(x.to(DEV), wc, ydt)
+        assert got.dtype == ydt
+        close(got, want, ydt, scale=0.2 * math.sqrt(K))
+    # a row's result does not depend on the other rows of the step: the same bits, unless the
+    # forced shape does not fit the LDS with many rows and K is cut into fewer parts for them
+    alone = o.linear_rows(x[M - 1:].to(DEV), wc, torch.float32)
+    among = o.linear_rows(x.to(DEV), wc, torch.float32)[M - 1]
+    if (kp, ps) == (4, 4):
+        close(alone[0], among, torch.float32, scale=0.2 * math.sqrt(K))
+    else:
+        assert torch.equal(alone[0], among)
+
+
+def test_linear_rows_takes_the_norm_and_refuses_what_it_does_not_take(rows_shape):
+    o = ops()
+    M, N, K = 12, 200, 4096
+    x_dev, x = _prepared_rows(M, K, torch.bfloat16, 1e-5)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=2, std=0.2)
+    wc = _decode_copy(w.to(DEV))
+    for tb, kp, ps in ((None, None, None), (2, 4, 2), (4, 1, 4)):
+        rows_shape(tb, kp, ps)
+        close(o.linear_rows(x_dev, wc, torch.float32), R.linear(x, w, torch.float64), torch.bfloat16,
+              scale=0.2 * math.sqrt(K))
+    assert not o.rows_fits(rnd(129, K, dtype=torch.bfloat16).to(DEV), wc, "plain")
+    assert not o.rows_fits(rnd(20, K, dtype=torch.bfloat16).to(DEV), wc, "gate_up")     # another kernel's tiles
+    assert not o.rows_fits(rnd(20, K, dtype=torch.bfloat16).to(DEV), w.to(DEV), "plain")  # no copy
+    assert not o.rows_fits(rnd(20, K).to(DEV), wc, "plain")                             # float32 rows
+    w96 = _decode_copy(rnd(N, 96, dtype=torch.bfloat16, seed=3).to(DEV))
+    assert not o.rows_fits(rnd(20, 96, dtype=torch.bfloat16).to(DEV), w96, "plain")     # K must be a multiple of 64
+    with pytest.raises(o.KernelError):
+        o.linear_rows(rnd(20, K).to(DEV), wc, torch.float32)
+
+
+@pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
+@pytest.mark.parametrize("M,F,K", [(17, 172, 64), (64, 11008, 4096), (40, 50, 192), (128, 203, 320), (33, 8, 1024)])
+def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, ps, rows_shape):
+    """17 to 128 rows: the product and the SiLU-multiply in one kernel, from the gate|up tiles."""
+    o = ops()
+    rows_shape(tb, kp, ps)
+    x = rnd(M, K, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * F, K, dtype=torch.bfloat16, seed=2, std=0.2)
+    got = o.gate_up_silu(x.to(DEV), _decode_copy(w.to(DEV), "gate_up"))
+    g, u = R.linear(x, w[:F], torch.float64), R.linear(x, w[F:], torch.float64)
+    want = g / (1 + torch.exp(-g)) * u
+    top = max(1.0, float(want.abs().max()))
+    close(got, want, torch.bfloat16, scale=top)
+    swapped = u / (1 + torch.exp(-u)) * g
+    assert not torch.allclose(got.double().cpu(), swapped, atol=0.1 * top)
+    # the product alone keeps float32 sums where the unfused path rounds gate and up to bfloat16
+    # first: the fused result is the closer one
+    loose = o.gate_up_silu(x.to(DEV), w.to(DEV))            # no copy: vendor GEMM, then SiLU-multiply
+    close(loose, want, torch.bfloat16, scale=top)
+    assert float((got.double().cpu() - want).abs().mean()) <= float((loose.double().cpu() - want).abs().mean()) * 1.05
+
+
+@pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
+@pytest.mark.parametrize("M,nh,nkv,hd,K", [(17, 4, 2, 32, 64), (64, 32, 32, 128, 4096), (40, 6, 3, 64, 256),
+                                           (128, 8, 1, 96, 128), (33, 3, 3, 48, 192), (70, 2, 1, 16, 1024)])
+def test_qkv_rope_store_of_many_rows(M, nh, nkv, hd, K, tb, kp, ps, rows_shape):
+    """17 to 128 sequences decoding together: the q|k|v product, the rotation and the cache store
+    in one kernel against the three steps."""
+    from inferllm_amd.parts.position import rotary_table
+    o = ops()
+    rows_shape(tb, kp, ps)
+    dtype, page = torch.bfloat16, 64
+    table = rotary_table(777.0, hd, 300, "cpu")
+    x = rnd(M, K, dtype=dtype, seed=1)
+    w = rnd((nh + 2 * nkv) * hd, K, dtype=dtype, seed=2, std=0.1)
+    pos = torch.tensor([(37 * i + 5) % 290 for i in range(M)], dtype=torch.int32)
+    slot = torch.randperm(M + 2, generator=torch.Generator().manual_seed(9))[:M].to(torch.int32)
+    g = torch.Generator().manual_seed(4)
+    pt = torch.randperm((M + 2) * 5, generator=g).reshape(M + 2, 5).to(torch.int32)
+    kc, vc = make_cache((M + 2) * 5, nkv, page, hd, dtype)
+    qkv_ref = R.linear(x, w, torch.float64)
+    kr, vr = kc.clone().double(), vc.clone().double()
+    R.rope_store(qkv_ref, table, hd, 0, pos, slot, None, kr, vr, pt, page, 0, nh, nkv, hd)
+    w_dev = _decode_copy(w.to(DEV), "qkv", nh=nh, nkv=nkv, hd=hd)
+    assert o.qkv_rope_store_fits(x.to(DEV), w_dev, hd) and not o.qkv_rope_store_fits(x.to(DEV), w.to(DEV), hd)
+    got = o.qkv_rope_store(x.to(DEV), w_dev, table.to(DEV), pos.to(DEV), slot.to(DEV), kc_g := kc.to(DEV),
+                           vc_g := vc.to(DEV), pt.to(DEV), page, 0, nh, nkv, hd).cpu()
+    sc = math.sqrt(K) * 0.1
+    close(got[:, :nh * hd], qkv_ref[:, :nh * hd], dtype, scale=sc)
+    for gotc, wantc in ((kc_g.cpu(), kr), (vc_g.cpu(), vr)):
+        assert torch.equal(torch.isnan(gotc), torch.isnan(wantc))        # the same rows, nothing else
+        close(torch.nan_to_num(gotc), torch.nan_to_num(wantc), dtype, scale=sc)
