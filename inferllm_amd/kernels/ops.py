@@ -474,8 +474,8 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
             return gemm_skinny_bf16(x, w, out_dtype or x.dtype)
         x = x.rows()
     out_dtype = out_dtype or x.dtype
-    if (isinstance(w, Weight) and out_dtype == torch.float32 and x.shape[0] >= ROWS_FROM
-            and rows_fits(x, w, "plain")):
+    if (isinstance(w, Weight) and out_dtype == torch.float32 and rows_fits(x, w, "plain")
+            and x.shape[0] >= rows_from("plain", w)):
         return linear_rows(x, w, out_dtype)              # logits of 17 to 128 rows
     if isinstance(w, Weight) and not (x.dtype == torch.bfloat16 and 1 <= x.shape[0] <= SKINNY_BEST_ROWS):
         w = w.plain                                      # only the few-rows kernel reads the copy
@@ -593,7 +593,14 @@ def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 ROWS_MAX = 128           # rows the products of csrc/gemm_rows.hip take (64 a launch)
-ROWS_FROM = 17           # from this many rows they are taken (up to 16: the few-rows kernels)
+ROWS_FROM = 17           # from this many rows they are taken unless the plan says otherwise for
+                         # the shape (up to 16 rows the few-rows kernels are the other way)
+
+
+def rows_from(mode: str, w) -> int:
+    """Fewest rows from which the product with `w` in tile order `mode` goes to
+    csrc/gemm_rows.hip: the plan's entry for the shape, else ROWS_FROM."""
+    return _plan.rows_from.get((mode,) + tuple(w.shape), ROWS_FROM)
 
 
 def rows_fits(x, w, mode: str) -> bool:
@@ -663,6 +670,44 @@ def qkv_rope_store_fits(x, w_qkv, hd: int) -> bool:
     return rows_fits(x, w_qkv, "qkv")
 
 
+def measure_rows_from_qkv(w_qkv: "Weight", nh: int, nkv: int, hd: int) -> int:
+    """Fewest rows (5, 9, 13 or 17) from which the fused q|k|v product of csrc/gemm_rows.hip takes
+    less time than the few-rows one (for the tuner; times both at 16, 12, 8 rows)."""
+    N, K = w_qkv.plain.shape
+    dev = w_qkv.plain.device
+    x = torch.zeros((16, K), dtype=torch.bfloat16, device=dev)
+    table = torch.zeros((16, hd // 2, 2), dtype=torch.float32, device=dev)
+    pos = torch.arange(16, dtype=torch.int32, device=dev)
+    pages = torch.arange(16, dtype=torch.int32, device=dev).view(16, 1).contiguous()
+    kc = torch.zeros((16, nkv, 64, hd), dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    saved, key = dict(_plan.rows_from), ("qkv", N, K)
+
+    def timed(rows: int, threshold: int) -> float:
+        _plan.rows_from[key] = threshold
+        run = lambda: qkv_rope_store(x[:rows], w_qkv, table, pos[:rows], pos[:rows], kc, vc, pages,
+                                     64, 0, nh, nkv, hd)
+        run(); run()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(8):
+            run()
+        end.record()
+        end.synchronize()
+        return start.elapsed_time(end)
+
+    first = ROWS_FROM
+    try:
+        for rows in (16, 12, 8):
+            if timed(rows, 1) >= 0.95 * timed(rows, ROWS_FROM):
+                break
+            first = rows - 3
+    finally:
+        _plan.rows_from.clear()
+        _plan.rows_from.update(saved)
+    return first
+
+
 def qkv_rope_store(x, w_qkv, cos_sin: torch.Tensor,
                    row_pos: torch.Tensor, row_slot: torch.Tensor, kcache: torch.Tensor,
                    vcache: torch.Tensor, page_table: torch.Tensor, page_size: int, ring: int,
@@ -684,7 +729,7 @@ def qkv_rope_store(x, w_qkv, cos_sin: torch.Tensor,
           vcache.shape == kcache.shape and vcache.dtype == torch.bfloat16 and page_table.dim() == 2,
           "qkv_rope_store: cache shape or dtype")
     y = torch.empty((M, N), dtype=torch.bfloat16, device=xt.device)
-    if M >= ROWS_FROM:
+    if wt is not None and K % 64 == 0 and M >= rows_from("qkv", w_qkv):
         _check(_lib().illm_qkv_rope_store_rows(
             _p(xt), wt, _p(y), M, K, _p(cos_sin), cos_sin.shape[0], _p(row_pos), _p(row_slot),
             _p(kcache), _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, nh, nkv,
@@ -706,6 +751,15 @@ def gate_up_silu(x, w_gate_up) -> torch.Tensor:
         x = x.rows()
     M, K = x.shape
     F2 = w_gate_up.shape[0]
+    if F2 % 2 == 0 and rows_fits(x, w_gate_up, "gate_up") and M >= rows_from("gate_up", w_gate_up):
+        xt, ssq, parts, eps = _operand(x)
+        xt = xt.contiguous()
+        _gpu(xt, w_gate_up.tiled)
+        y = torch.empty((M, F2 // 2), dtype=x.dtype, device=xt.device)
+        _check(_lib().illm_gemm_rows_gateup_silu(_p(xt), _p(w_gate_up.tiled), _p(y), _code(y), M,
+                                                 F2 // 2, K, ssq, parts, eps, _stream()),
+               "gate_up_silu (rows)")
+        return y
     if (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and F2 % 2 == 0
             and 1 <= M <= SKINNY_BEST_ROWS and K % 8 == 0):
         xt, ssq, parts, eps = _operand(x)
@@ -716,14 +770,6 @@ def gate_up_silu(x, w_gate_up) -> torch.Tensor:
         _check(_lib().illm_gemm_skinny_gateup_silu(_p(xt), _p(wp), wt, _p(y), _code(y), M,
                                                    F2 // 2, K, ssq, parts, eps, GATE_UP_WAVES,
                                                    _stream()), "gate_up_silu")
-        return y
-    if M >= ROWS_FROM and F2 % 2 == 0 and rows_fits(x, w_gate_up, "gate_up"):
-        x = x.contiguous()
-        _gpu(x, w_gate_up.tiled)
-        y = torch.empty((M, F2 // 2), dtype=x.dtype, device=x.device)
-        _check(_lib().illm_gemm_rows_gateup_silu(_p(x), _p(w_gate_up.tiled), _p(y), _code(y), M,
-                                                 F2 // 2, K, None, 0, ctypes.c_float(0.0),
-                                                 _stream()), "gate_up_silu (rows)")
         return y
     if isinstance(x, NormedRows):
         x = x.rows()

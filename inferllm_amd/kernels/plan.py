@@ -12,6 +12,9 @@ the choice is a table by shape:
   (`python -m inferllm_amd.kernels.tune`: the majority of three measurements, and a way other
   than the rule's must win by 7 %), and for every other shape one rule: planes from 17 rows on,
   products of many rows whole.  Nothing is ever timed.
+  The third table says from how few rows (below 17) the q|k|v product goes to the kernel that
+  shares X through LDS (csrc/gemm_rows.hip) rather than to the few-rows kernel; gate|up and the
+  head measured equal or worse there below 17 rows and have no entries.
 * `Plan(measure=True)` (`Engine(tune=True)`): a shape that the tables lack is timed the first
   time it is used outside graph capture and the winner is kept; `to_dict()` gives the result,
   which `Engine(plan=...)` pins in another process.
@@ -121,31 +124,45 @@ FIXED_CUTS: Dict[tuple, tuple] = {
 }
 
 
+# (tile order "plain" / "gate_up" / "qkv", N, K) of a matrix with a decode copy -> fewest rows
+# (below 17) from which its product goes to the kernels that share X through LDS
+# (csrc/gemm_rows.hip) instead of the few-rows kernels, whose waves each read X for themselves.
+# Unlisted shapes: from 17 rows.
+FIXED_ROWS_FROM: Dict[tuple, int] = {
+    ("qkv", 6144, 4096): 5,        # 16 rows: 18.2 -> 14.7 us
+    ("qkv", 10240, 8192): 5,       # 16 rows: 45.9 -> 33.9 us
+    ("qkv", 12288, 4096): 13,      # 16 rows: 25.0 -> 21.5 us
+}
+
+
 class Plan:
     """The tables one engine's products are dispatched by (see the module text)."""
 
     def __init__(self, planes_from: Optional[dict] = None, cuts: Optional[dict] = None,
-                 measure: bool = False):
+                 measure: bool = False, rows_from: Optional[dict] = None):
         self.planes_from: Dict[Tuple[int, int], int] = dict(planes_from or {})
         self.cuts: Dict[tuple, tuple] = dict(cuts or {})
+        self.rows_from: Dict[tuple, int] = dict(rows_from or {})
         self.measure = bool(measure)
 
     @classmethod
     def fixed(cls, measure: bool = False) -> "Plan":
-        return cls(FIXED_PLANES_FROM, FIXED_CUTS, measure)
+        return cls(FIXED_PLANES_FROM, FIXED_CUTS, measure, FIXED_ROWS_FROM)
 
     # ------------------------------------------------------------ as plain data
     def to_dict(self) -> dict:
         """JSON-able: {"planes_from": [[N, K, rows], ...], "cuts": [[key, plan], ...]}."""
         return {"planes_from": [[n, k, r] for (n, k), r in sorted(self.planes_from.items())],
-                "cuts": [[list(k), list(p)] for k, p in sorted(self.cuts.items(), key=repr)]}
+                "cuts": [[list(k), list(p)] for k, p in sorted(self.cuts.items(), key=repr)],
+                "rows_from": [[m, n, k, r] for (m, n, k), r in sorted(self.rows_from.items())]}
 
     @classmethod
     def from_dict(cls, d: dict) -> "Plan":
         """A pinned plan: what `to_dict` gave, nothing measured."""
         return cls({(int(n), int(k)): int(r) for n, k, r in d.get("planes_from", [])},
-                   {tuple(k): tuple(p) for k, p in d.get("cuts", [])}, measure=False)
+                   {tuple(k): tuple(p) for k, p in d.get("cuts", [])}, measure=False,
+                   rows_from={(str(m), int(n), int(k)): int(r) for m, n, k, r in d.get("rows_from", [])})
 
     def __eq__(self, other) -> bool:
         return (isinstance(other, Plan) and self.planes_from == other.planes_from
-                and self.cuts == other.cuts)
+                and self.cuts == other.cuts and self.rows_from == other.rows_from)

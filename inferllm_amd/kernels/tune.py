@@ -6,8 +6,9 @@ For every config.json it builds one layer of the model with random weights, take
 the parts really multiply by (fused q|k|v and gate|up included) and times, per shape: from how
 few rows the thin matrices go through planes, and for products of many rows the whole product
 against its cuts, per class of 256 rows up to --max-rows, and whole against filled up to 256
-rows for 65 to 255 rows.  It prints the two tables as Python literals, ready for
-`FIXED_PLANES_FROM` and `FIXED_CUTS`.  Entries that say "whole" are left out: that is the rule
+rows for 65 to 255 rows.  It prints the tables as Python literals, ready for
+`FIXED_PLANES_FROM`, `FIXED_CUTS` and `FIXED_ROWS_FROM` (from how few rows the fused q|k|v
+product takes the kernel that shares X through LDS).  Entries that say "whole" are left out: that is the rule
 for unlisted shapes anyway.
 """
 from __future__ import annotations
@@ -47,7 +48,18 @@ def tune_config(cfg: dict, max_rows: int, repeats: int, say) -> tuple:
     eng = Engine.from_random(one, seed=0, dtype="bfloat16", max_batch=1, max_seq_len=64,
                              decode_copies=True, plan=Plan())
     ops.use_plan(Plan())
-    planes, cuts = {}, {}
+    planes, cuts, rows = {}, {}, {}
+    for part in eng.model.every_part():
+        # a mixer that keeps a fused q|k|v matrix with its head geometry (the attention part)
+        w = getattr(part, "w_qkv", None)
+        if isinstance(w, ops.Weight) and w.mode == "qkv" and w.tiled is not None and w.shape[1] % 64 == 0:
+            key = ("qkv",) + tuple(w.shape)
+            if key not in rows:
+                votes = sorted(ops.measure_rows_from_qkv(w, part.nh, part.nkv, part.hd)
+                               for _ in range(repeats))
+                rows[key] = votes[len(votes) // 2]
+                say(f"  q|k|v {w.shape[0]} x {w.shape[1]}: shared-X kernel from {rows[key]} rows (runs: {votes})")
+    rows = {k: v for k, v in rows.items() if v != ops.ROWS_FROM}
     for (N, K), w in sorted(matrices(eng).items()):
         plain = ops.plain_weight(w)
         if (isinstance(w, ops.Weight) and w.mode == "plain" and w.tiled is not None and K >= 2 * N
@@ -74,7 +86,7 @@ def tune_config(cfg: dict, max_rows: int, repeats: int, say) -> tuple:
             if best:
                 cuts[(rows256, N, K)] = best
         say(f"  products {N} x {K}: {sum(1 for k in cuts if k[-2:] == (N, K))} classes are not whole")
-    return planes, cuts
+    return planes, cuts, rows
 
 
 def main(argv=None) -> int:
@@ -85,14 +97,15 @@ def main(argv=None) -> int:
     ap.add_argument("--repeats", type=int, default=3, help="measurements per entry; the majority wins")
     args = ap.parse_args(argv)
     say = lambda m: print(m, file=sys.stderr, flush=True)
-    planes, cuts = {}, {}
+    planes, cuts, rows = {}, {}, {}
     for path in args.configs:
         with open(path, "r", encoding="utf-8") as f:
             cfg = json.load(f)
         say(f"{path}:")
-        p, c = tune_config(cfg, args.max_rows, args.repeats, say)
+        p, c, r = tune_config(cfg, args.max_rows, args.repeats, say)
         planes.update(p)
         cuts.update(c)
+        rows.update(r)
     print("FIXED_PLANES_FROM = {")
     for k in sorted(planes):
         print(f"    {k}: {planes[k]},")
@@ -100,6 +113,10 @@ def main(argv=None) -> int:
     print("FIXED_CUTS = {")
     for k in sorted(cuts, key=repr):
         print(f"    {k}: {cuts[k]},")
+    print("}")
+    print("FIXED_ROWS_FROM = {")
+    for k in sorted(rows):
+        print(f"    {k}: {rows[k]},")
     print("}")
     return 0
 

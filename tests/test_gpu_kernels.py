@@ -529,6 +529,16 @@ def test_gate_up_silu_takes_the_norm(M, F, K):
     g, u = R.linear(h, w[:F], torch.float64), R.linear(h, w[F:], torch.float64)
     want = g / (1 + torch.exp(-g)) * u
     close(got, want, torch.bfloat16, scale=max(1.0, float(want.abs().max())))
+    if K % 64 == 0:
+        # the same through the kernel that shares X through LDS, where the plan sends few rows to it
+        o = ops()
+        plan = o.current_plan()
+        try:
+            plan.rows_from[("gate_up", 2 * F, K)] = 1
+            again = o.gate_up_silu(rows, _decode_copy(w.to(DEV), "gate_up"))
+        finally:
+            del plan.rows_from[("gate_up", 2 * F, K)]
+        close(again, want, torch.bfloat16, scale=max(1.0, float(want.abs().max())))
 
 
 @pytest.mark.parametrize("nw_dtype", [None] + DTYPES)
@@ -746,16 +756,24 @@ def test_window_edge_prefill_and_decode(dtype, hd):
 
 
 _QKV_SHAPES = [(1, 32, 32, 128, 4096), (8, 4, 2, 32, 64), (16, 6, 3, 64, 200), (3, 8, 1, 96, 72),
-               (5, 3, 3, 48, 136), (2, 2, 1, 16, 40), (5, 3, 3, 48, 160), (7, 2, 2, 16, 96)]
+               (5, 3, 3, 48, 136), (2, 2, 1, 16, 40), (5, 3, 3, 48, 160), (7, 2, 2, 16, 96),
+               (13, 3, 3, 48, 192), (16, 8, 2, 128, 1024)]
 
 
 # with the decode copy only where one can be made (K a multiple of 32)
 @pytest.mark.parametrize("M,nh,nkv,hd,K,copy", [s + (c,) for s in _QKV_SHAPES for c in (False, True)
                                                 if not (c and s[4] % 32)])
 @pytest.mark.parametrize("normed", [False, True])
-def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed, copy):
-    """The fused decode kernel against (norm,) product, then rotation and cache store."""
+@pytest.mark.parametrize("shared_x", [False, True])
+def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed, copy, shared_x, monkeypatch):
+    """The fused decode kernel against (norm,) product, then rotation and cache store.
+    `shared_x`: the plan sends these few rows to the kernel that shares X through LDS
+    (csrc/gemm_rows.hip), which needs the decode copy and K a multiple of 64."""
     from inferllm_amd.parts.position import rotary_table
+    if shared_x:
+        if not copy or K % 64:
+            pytest.skip("the shared-X kernel needs the decode copy and K % 64 == 0")
+        monkeypatch.setitem(ops().current_plan().rows_from, ("qkv", (nh + 2 * nkv) * hd, K), 1)
     dtype, page = torch.bfloat16, 64
     table = rotary_table(777.0, hd, 300, "cpu")
     x = rnd(M, K, dtype=dtype, seed=1)
