@@ -58,6 +58,12 @@ int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens
                            int max_len, int nh, int nkv, int hd, float scale, int window,
                            void* stream);
 
+// Tuning and tests: which prefill attention kernel head sizes up to 128 take: 0 the one with one
+// LDS buffer (which larger head sizes use), 2 the one with two buffers and one barrier a tile
+// (needs a positive scale), 1 (default) the second for head sizes 96 and 128 and sequences of
+// 1,024 keys or more.
+void illm_set_prefill_two_buffers(int on);
+
 // One query row per sequence over the paged cache.  partial: float32
 // [B][nh][nsplit][hd + 2] scratch.  seq_len[b] = keys of sequence b, the new one included.
 int illm_attn_decode_generic(const void* qkv, void* out, int dt, const void* kcache,

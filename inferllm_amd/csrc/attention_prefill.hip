@@ -222,6 +222,246 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     }
 }
 
+// The same for head sizes up to 128 with two LDS buffers and one barrier a tile: while a tile is
+// multiplied the next one, already in registers, is written to the other buffer and the one
+// after it is asked for.  K and V^T rows are not padded but swizzled (16-byte units XORed with
+// the row's low bits), so two buffers of both are 512 * HD bytes (64 KB at head size 128, two
+// blocks a compute unit).  V is transposed in registers, 4 keys x 8 dims a thread, and written
+// as 8-byte runs of 4 keys; within a tile of 64 keys the runs are placed in the order in which
+// the first product leaves the scores of a lane (keys 16 m + 4 h + {0..3} and + 8 + {0..3} for
+// half-wave h), so that the A operand of the second product is one 16-byte read.
+template <int HD>
+__global__ void __launch_bounds__(256, 2)
+attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
+                          const int32_t* __restrict__ cu, int n_qblk, int nh, int nkv,
+                          float scale_log2, int window, int hb_per_xcd, int n_hb, int zigzag) {
+    constexpr int KS = HD / 16;        // k-steps of the first product
+    constexpr int DB = HD / 32;        // 32-row blocks of O^T
+    constexpr int UK = HD / 8;         // 16-byte units in a K row
+    constexpr int KMASK = (UK % 8 == 0) ? 7 : 3;
+    constexpr int K_TILE = PF_BN * HD;             // elements of a K buffer
+    constexpr int V_TILE = HD * PF_BN;             // elements of a V^T buffer (rows of 64 keys)
+    extern __shared__ __attribute__((aligned(16))) bf16_t pf_lds[];
+    bf16_t* ks = pf_lds;                           // [2][64][HD]
+    bf16_t* vts = pf_lds + 2 * K_TILE;             // [2][HD][64]
+
+    const int xcd = blockIdx.x % 8, slot_id = blockIdx.x / 8;
+    const int hb = xcd * hb_per_xcd + slot_id % hb_per_xcd;
+    if (hb >= n_hb) return;
+    const int qi = slot_id / hb_per_xcd, top = zigzag ? (n_qblk + 1) / 2 : n_qblk;
+    const int qb = qi < top ? n_qblk - 1 - qi : qi - top;
+    const int h = hb % nh, b = hb / nh;
+    const int start = cu[b], len = cu[b + 1] - start;
+    const int q0 = qb * PF_BM;
+    if (q0 >= len) return;
+    const int kvh = h / (nh / nkv);
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
+    const int tid = threadIdx.x, wave = wave_index(), lane = tid & 63;
+    const int lq = lane & 31, half = lane >> 5;
+    const int q_row0 = q0 + wave * 32;
+    const int q = q_row0 + lq;
+    const int qc = q < len ? q : len - 1;
+
+    uint4 qf[KS];
+    {
+        const bf16_t* qp = qkv + (size_t)(start + qc) * rowlen + (size_t)h * HD + half * 8;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) qf[s] = *(const uint4*)(qp + s * 16);
+    }
+    f32x16_t o[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[d][i] = 0.f;
+    float m = NEG_INF, l = 0.f;
+
+    const int k_end = min(len, q0 + PF_BM);
+    int k_begin = window > 0 ? max(0, q0 - window + 1) : 0;
+    k_begin = (k_begin / PF_BN) * PF_BN;
+    const int wk_end = min(len, q_row0 + 32);                       // this wave's last key + 1
+    const int wk_begin = window > 0 ? max(0, q_row0 - window + 1) : 0;
+
+    // staging.  K: unit u = (key, chunk) as in the kernel above.  V: unit u = (chunk c = u / 16,
+    // key group g = u % 16): keys 4 g .. 4 g + 3, dims 8 c .. 8 c + 7.
+    constexpr int NLD = (PF_BN * HD / 8) / 256;          // K units a thread
+    constexpr int NVU = (2 * HD + 255) / 256;            // V units a thread
+    // (native vector types: arrays of the runtime's uint4 struct are not always kept in registers)
+    illm_u32x4_t kpre[NLD], vpre0[NVU], vpre1[NVU], vpre2[NVU], vpre3[NVU];
+    auto fetch = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < NLD; ++it) {
+            const int u = tid + it * 256;
+            const int key = ((u >> 6) & 3) * 16 + (u & 15);
+            const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
+            const int krow = min(k0 + key, len - 1);
+            kpre[it] = *(const illm_u32x4_t*)(qkv + (size_t)(start + krow) * rowlen +
+                                              (size_t)(nh + kvh) * HD + ch * 8);
+        }
+#pragma unroll
+        for (int it = 0; it < NVU; ++it) {
+            const int u = tid + it * 256;
+            const int c = (u >> 4) < UK ? (u >> 4) : UK - 1, g = u & 15;
+            const bf16_t* vsrc = qkv + (size_t)(nh + nkv + kvh) * HD + c * 8;
+            vpre0[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 0, len - 1)) * rowlen);
+            vpre1[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 1, len - 1)) * rowlen);
+            vpre2[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 2, len - 1)) * rowlen);
+            vpre3[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 3, len - 1)) * rowlen);
+        }
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+        bf16_t* kd = ks + buf * K_TILE;
+        bf16_t* vd = vts + buf * V_TILE;
+#pragma unroll
+        for (int it = 0; it < NLD; ++it) {
+            const int u = tid + it * 256;
+            const int key = ((u >> 6) & 3) * 16 + (u & 15);
+            const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
+            *(illm_u32x4_t*)(kd + key * HD + ((ch ^ (key & KMASK)) * 8)) = kpre[it];
+        }
+#pragma unroll
+        for (int it = 0; it < NVU; ++it) {
+            const int u = tid + it * 256;
+            if (NVU * 256 != 2 * HD && u >= 2 * HD) continue;
+            const int c = u >> 4, g = u & 15;
+            // where the group's 4 keys go in the row of 64: bits (sub, sub, m, a, h) -> (.., h, a)
+            const int pg = (g & 12) | ((g & 1) << 1) | ((g >> 1) & 1);
+#pragma unroll
+            for (int dp = 0; dp < 4; ++dp) {                 // dims 2 dp and 2 dp + 1
+                const uint32_t a0 = vpre0[it][dp], a1 = vpre1[it][dp], a2 = vpre2[it][dp], a3 = vpre3[it][dp];
+                const uint2 even = make_uint2((a0 & 0xffffu) | (a1 << 16), (a2 & 0xffffu) | (a3 << 16));
+                const uint2 odd = make_uint2((a0 >> 16) | (a1 & 0xffff0000u), (a2 >> 16) | (a3 & 0xffff0000u));
+                const int d0 = 8 * c + 2 * dp;
+                *(uint2*)(vd + d0 * PF_BN + ((((pg >> 1) ^ (d0 & 7)) * 2 + (pg & 1)) * 4)) = even;
+                *(uint2*)(vd + (d0 + 1) * PF_BN + ((((pg >> 1) ^ ((d0 + 1) & 7)) * 2 + (pg & 1)) * 4)) = odd;
+            }
+        }
+    };
+
+    if (k_begin < k_end) {
+        fetch(k_begin);
+        stage(0);
+        if (k_begin + PF_BN < k_end) fetch(k_begin + PF_BN);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = k_begin; k0 < k_end; k0 += PF_BN, buf ^= 1) {
+        if (k0 < wk_end && k0 + PF_BN > wk_begin) {                 // something visible to this wave
+            const bf16_t* kb = ks + buf * K_TILE;
+            const bf16_t* vb = vts + buf * V_TILE;
+            // S^T[key][q] for two sub-tiles of 32 keys
+            // (the two sub-tiles' sums alternate, so that no product waits for the one before it)
+            f32x16_t s[2];
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[sub][i] = 0.f;
+#pragma unroll
+            for (int st = 0; st < KS; ++st)
+#pragma unroll
+                for (int sub = 0; sub < 2; ++sub) {
+                    const int krow = sub * 32 + lq;
+                    const uint4 a = *(const uint4*)(kb + krow * HD + (((st * 2 + half) ^ (krow & KMASK)) * 8));
+                    s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&a,
+                                                                     *(const bf16x8_t*)&qf[st],
+                                                                     s[sub], 0, 0, 0);
+                }
+            const bool need_mask = (k0 + PF_BN > q_row0 + 1) || (k0 + PF_BN > len) || (window > 0);
+            float mx = NEG_INF;
+            if (need_mask) {                 // the same for the whole wave: one branch, two bodies
+#pragma unroll
+                for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int key = k0 + sub * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
+                        const bool ok = key <= q && key < len && (window <= 0 || key > q - window);
+                        const float v = ok ? s[sub][i] : NEG_INF;
+                        s[sub][i] = v;
+                        mx = fmaxf(mx, v);
+                    }
+            } else {
+#pragma unroll
+                for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[sub][i]);
+            }
+            // the running max is kept in scaled units (scale > 0, so the order is the same);
+            // the scale is applied inside the exponential's argument: one multiply-add a score
+            mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE)) * scale_log2;
+            const float m_new = fmaxf(m, mx);
+            const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m - m_use);
+            float rs = 0.f;
+            uint4 pb[2][2];
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub) {
+                float p[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    p[i] = __builtin_amdgcn_exp2f(fmaf(s[sub][i], scale_log2, -m_use));
+                    rs += p[i];
+                }
+#pragma unroll
+                for (int mf = 0; mf < 2; ++mf) {
+                    pb[sub][mf].x = pack_bf16x2(p[8 * mf + 0], p[8 * mf + 1]);
+                    pb[sub][mf].y = pack_bf16x2(p[8 * mf + 2], p[8 * mf + 3]);
+                    pb[sub][mf].z = pack_bf16x2(p[8 * mf + 4], p[8 * mf + 5]);
+                    pb[sub][mf].w = pack_bf16x2(p[8 * mf + 6], p[8 * mf + 7]);
+                }
+            }
+            l = l * alpha + rs;
+            m = m_new;
+            if (__any(alpha != 1.f)) {          // the running max moved for some query of the wave
+#pragma unroll
+                for (int d = 0; d < DB; ++d)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o[d][i] *= alpha;
+            }
+            // O^T[d][q] += V^T[d][keys] . P^T[keys][q]: 8 keys of a lane are one 16-byte unit
+            // (the blocks of dims innermost: consecutive products add to different sums)
+#pragma unroll
+            for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                for (int mf = 0; mf < 2; ++mf)
+#pragma unroll
+                    for (int d = 0; d < DB; ++d) {
+                        const int drow = d * 32 + lq;
+                        const uint4 a = *(const uint4*)(vb + drow * PF_BN +
+                                                        (((sub * 4 + mf * 2 + half) ^ (drow & 7)) * 8));
+                        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&a,
+                                                                       *(const bf16x8_t*)&pb[sub][mf],
+                                                                       o[d], 0, 0, 0);
+                    }
+        }
+        // the next tile into the other buffer (last read before the barrier that ended the
+        // previous round), the one after it on its way
+        if (k0 + PF_BN < k_end) {
+            stage(buf ^ 1);
+            if (k0 + 2 * PF_BN < k_end) fetch(k0 + 2 * PF_BN);
+        }
+        __syncthreads();
+    }
+    l += __shfl_xor(l, 32, ILLM_WAVE);
+    if (q < len) {
+        const float inv = 1.0f / l;
+        bf16_t* op = out + (size_t)(start + q) * nh * HD + (size_t)h * HD + 4 * half;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; ++b4) {
+                uint2 v;
+                v.x = pack_bf16x2(o[d][4 * b4 + 0] * inv, o[d][4 * b4 + 1] * inv);
+                v.y = pack_bf16x2(o[d][4 * b4 + 2] * inv, o[d][4 * b4 + 3] * inv);
+                *(uint2*)(op + d * 32 + 8 * b4) = v;
+            }
+    }
+}
+
+// Tuning and tests: 0 sends head sizes up to 128 to the kernel with one LDS buffer always, 2 to the
+// one with two buffers always (the scale must be positive); 1 (default): two buffers for head
+// sizes 96 and 128 and sequences of 1,024 keys or more.
+static int PF_TWO_BUFFERS = 1;
+extern "C" void illm_set_prefill_two_buffers(int on) { PF_TWO_BUFFERS = on; }
+
 template <int HD>
 static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_seqs, int max_len,
                           int nh, int nkv, float scale, int window, hipStream_t st) {
@@ -230,6 +470,17 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
     const long long hb_per_xcd = (n_hb + 7) / 8;
     const long long blocks = 8 * hb_per_xcd * n_qblk;
     if (blocks > 0x7fffffffLL) return ILLM_ERR_ARG;
+    if constexpr (HD <= 128) {
+        // measured at 32 heads: head size 128, 2,048 keys 81 -> 76 us, 4,096 keys 236 -> 214; head
+        // size 64 and sequences of 512 lose a tenth (a tile more of set-up before the first product)
+        if (PF_TWO_BUFFERS == 2 || (PF_TWO_BUFFERS == 1 && HD >= 96 && max_len >= 1024 && scale > 0.f)) {
+            hipLaunchKernelGGL(attn_prefill_mfma2_kernel<HD>, dim3((unsigned)blocks), dim3(256),
+                               (size_t)512 * HD, st, (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh,
+                               nkv, scale * 1.44269504088896340736f, window, (int)hb_per_xcd,
+                               (int)n_hb, hb_per_xcd * n_qblk <= 64 ? 1 : 0);
+            return illm_launch_status();
+        }
+    }
     hipLaunchKernelGGL(attn_prefill_mfma_kernel<HD>, dim3((unsigned)blocks), dim3(256), 0, st,
                        (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
                        scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,

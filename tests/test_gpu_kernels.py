@@ -209,15 +209,22 @@ def test_attn_prefill(dtype, nh, nkv, hd, lens, window):
     # more blocks than the chip holds at once (heaviest first, not paired), and a long sequence
     (32, 8, 128, [600, 130, 577, 64], 0), (2, 1, 128, [2500, 40], 0)])
 def test_attn_prefill_mfma(nh, nkv, hd, lens, window):
-    """The matrix-core kernel over several blocks of 128 query rows and tiles of 64 keys."""
+    """The matrix-core kernels over several blocks of 128 query rows and tiles of 64 keys: the one
+    with one LDS buffer, the one with two (head sizes up to 128), and the library's own choice."""
     dtype = torch.bfloat16
     T = sum(lens)
     qkv = rnd(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=17)
     cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
     scale = 1.0 / math.sqrt(hd)
-    got = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), len(lens), max(lens), nh, nkv, hd, scale, window)
     want = R.attn_prefill(qkv, cu, len(lens), max(lens), nh, nkv, hd, scale, window)
-    close(got, want, dtype, scale=2)
+    lib = ops()._lib()
+    try:
+        for which in (0, 2, 1):
+            lib.illm_set_prefill_two_buffers(which)
+            got = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), len(lens), max(lens), nh, nkv, hd, scale, window)
+            close(got, want, dtype, scale=2)
+    finally:
+        lib.illm_set_prefill_two_buffers(1)
 
 
 def test_attn_prefill_finds_one_far_key():
