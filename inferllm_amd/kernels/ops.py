@@ -12,12 +12,15 @@ MFMA kernels of this library when the shape fits them (few rows: decoding), and
 to the vendor GEMM through `torch.matmul` otherwise, which is where the reference
 uses a vendor GEMM too (cublasSgemm, src/kern/gpu/kernel_gpu.cu:420-435).
 
-Four things ride on the products.  `Weight`: a matrix with a second copy in the
+Five things ride on the products.  `Weight`: a matrix with a second copy in the
 kernels' own tile order (`decode_weight`).  `linear_add` / `NormedRows`: the
 residual add in the product's epilogue and the RMS norm that follows it taken by
 the next product (up to 16 rows).  `linear_planes`: the product of up to 128 rows (from
 17, or from fewer where the plan says that pays) with a long thin matrix, K cut into
-ranges whose float32 planes `add_rmsnorm` adds.
+ranges whose float32 planes `add_rmsnorm` adds.  `linear_rows`, and `qkv_rope_store` and
+`gate_up_silu` from 17 rows on (from fewer where the plan says): products of up to 64 (128)
+rows with the wide matrices, X shared by a block's waves through LDS, with the rotation and
+cache store or the SiLU-multiply in the same kernel (csrc/gemm_rows.hip).
 `_planned_matmul`: products of many rows whole or cut along the output columns, as the
 current plan's table says for the shape (`kernels.plan`: fixed tables by default, so that
 nothing depends on a stopwatch).
@@ -593,6 +596,10 @@ def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 ROWS_MAX = 128           # rows the products of csrc/gemm_rows.hip take (64 a launch)
+ROWS_FUSED_MAX = 64      # rows up to which the fused q|k|v and gate|up products are taken: beyond
+                         # a launch's 64 rows W is read twice and the vendor GEMM with the
+                         # elementwise kernels behind it wins (measured at 128 rows of the 7B
+                         # shapes: q|k|v 47 against 33 + 5 us, gate|up 84 against 46 + 4)
 ROWS_FROM = 17           # from this many rows they are taken unless the plan says otherwise for
                          # the shape (up to 16 rows the few-rows kernels are the other way)
 
@@ -607,9 +614,10 @@ def rows_fits(x, w, mode: str) -> bool:
     """Whether the products of csrc/gemm_rows.hip take these operands: bfloat16 rows (or
     `NormedRows`, up to 16) and a weight with a decode copy in `mode`'s tile order."""
     xt = x.xb if isinstance(x, NormedRows) else x
+    most = 16 if isinstance(x, NormedRows) else (ROWS_MAX if mode == "plain" else ROWS_FUSED_MAX)
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == mode
             and isinstance(xt, torch.Tensor) and xt.dtype == torch.bfloat16 and xt.dim() == 2
-            and 1 <= xt.shape[0] <= (16 if isinstance(x, NormedRows) else ROWS_MAX)
+            and 1 <= xt.shape[0] <= most
             and xt.shape[1] == w.plain.shape[1] and xt.shape[1] % 64 == 0)
 
 
@@ -662,7 +670,7 @@ PLAIN_WAVES = 0          # and for the plain few-rows product
 
 def qkv_rope_store_fits(x, w_qkv, hd: int) -> bool:
     """Whether the one-kernel q|k|v product + rotation + cache store takes these operands: up to
-    16 rows always, up to 128 with a decode copy of the matrix in q|k|v tile order."""
+    16 rows always, up to 64 with a decode copy of the matrix in q|k|v tile order."""
     if not (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and hd % 16 == 0):
         return False
     if 1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0:

@@ -867,9 +867,9 @@ def test_linear_rows_takes_the_norm_and_refuses_what_it_does_not_take(rows_shape
 
 
 @pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
-@pytest.mark.parametrize("M,F,K", [(17, 172, 64), (64, 11008, 4096), (40, 50, 192), (128, 203, 320), (33, 8, 1024)])
+@pytest.mark.parametrize("M,F,K", [(17, 172, 64), (64, 11008, 4096), (40, 50, 192), (64, 203, 320), (33, 8, 1024)])
 def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, ps, rows_shape):
-    """17 to 128 rows: the product and the SiLU-multiply in one kernel, from the gate|up tiles."""
+    """17 to 64 rows: the product and the SiLU-multiply in one kernel, from the gate|up tiles."""
     o = ops()
     rows_shape(tb, kp, ps)
     x = rnd(M, K, dtype=torch.bfloat16, seed=1)
@@ -890,9 +890,9 @@ def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, ps, rows_shape):
 
 @pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
 @pytest.mark.parametrize("M,nh,nkv,hd,K", [(17, 4, 2, 32, 64), (64, 32, 32, 128, 4096), (40, 6, 3, 64, 256),
-                                           (128, 8, 1, 96, 128), (33, 3, 3, 48, 192), (70, 2, 1, 16, 1024)])
+                                           (64, 8, 1, 96, 128), (33, 3, 3, 48, 192), (50, 2, 1, 16, 1024)])
 def test_qkv_rope_store_of_many_rows(M, nh, nkv, hd, K, tb, kp, ps, rows_shape):
-    """17 to 128 sequences decoding together: the q|k|v product, the rotation and the cache store
+    """17 to 64 sequences decoding together: the q|k|v product, the rotation and the cache store
     in one kernel against the three steps."""
     from inferllm_amd.parts.position import rotary_table
     o = ops()
