@@ -49,9 +49,10 @@ struct GrScale {
     float eps;
 };
 
-// GR_PIECE: k-steps of 32 in a piece (2 or 4)
+// GR_PIECE: k-steps of 32 in a piece.  A block of four tiles has at most two parts of K (eight
+// waves), one of two or three tiles up to four.
 template <int MT, int TB, int MODE, int GR_PIECE>
-__global__ void __launch_bounds__(64 * TB * 4)
+__global__ void __launch_bounds__(64 * TB * (TB == 4 ? 2 : 4))
 gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, void* __restrict__ Y,
                  int y_dt, int M, int N, int K, int tiles, int kp, GrRope rope, GrScale scale) {
     constexpr int UNITS = MT * 16 * GR_PIECE * 4;            // 16-byte units of a part's X piece
@@ -118,6 +119,26 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
             A[u] = __builtin_nontemporal_load((const illm_u32x4_t*)(wtile + (size_t)(pc_ * GR_PIECE + u) * 512));                       \
     }
 
+    // GR_QKV_ROPE: what the waves of part 0 need to finish their tile (positions, angles, cache
+    // pages) is asked for around the first pieces of W, two dependent loads deep, and has long
+    // arrived when the sums are complete.  Indices are clamped, so every lane loads something.
+    int rot_head = -1, rot_j = 0, e_pos[MT], e_slot[MT], e_page[MT];
+    float cs[MT][8];
+    const bool finishes = MODE == GR_QKV_ROPE && part == 0;
+    if (finishes) {
+        const int tph = rope.hd / 16, n_rot = (rope.nh + rope.nkv) * tph;
+        if (tile_ok && tile < n_rot) {
+            rot_head = tile / tph;
+            rot_j = tile % tph;
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r < M ? mt * 16 + r : M - 1;
+            e_pos[mt] = rope.row_pos[m];
+            e_slot[mt] = rope.row_slot[m];
+        }
+    }
+
     f32x4_t acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -128,6 +149,19 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
     GR_LOAD_X(p_begin + 1, xr1)
     GR_LOAD_W(p_begin + 1, wr1)
     GR_LOAD_W(p_begin + 2, wr2)
+    if (finishes) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const float4* c4 = (const float4*)(rope.cos_sin + (size_t)e_pos[mt] * rope.hd +
+                                               2 * (8 * rot_j + 4 * (q & 1)));
+            const float4 c0 = c4[0], c1 = c4[1];
+            cs[mt][0] = c0.x; cs[mt][1] = c0.y; cs[mt][2] = c0.z; cs[mt][3] = c0.w;
+            cs[mt][4] = c1.x; cs[mt][5] = c1.y; cs[mt][6] = c1.z; cs[mt][7] = c1.w;
+            int lp = e_pos[mt] / rope.page_size;
+            if (rope.ring > 0) lp %= rope.ring;
+            e_page[mt] = rope.page_table[(size_t)e_slot[mt] * rope.table_stride + lp];
+        }
+    }
     // A stage of a round of four: piece p = p_begin + I.  One barrier a piece is enough with two
     // buffers: whoever writes buffer BUF again, two pieces on, has passed the next piece's
     // barrier, which every wave reaches only after it has finished reading this one.
@@ -160,44 +194,6 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
 #undef GR_LOAD_X
 #undef GR_LOAD_W
     __syncthreads();                                         // the X pieces are no longer read
-
-    // what the waves of part 0 need to finish their tile, asked for before the parts are added:
-    // positions, angles and cache rows (GR_QKV_ROPE)
-    int rot_head = -1, rot_j = 0;
-    float cs[MT][8];
-    size_t c_off[MT];
-    if (MODE == GR_QKV_ROPE && part == 0 && tile_ok) {
-        const int tph = rope.hd / 16, n_rot = (rope.nh + rope.nkv) * tph;
-        if (tile < n_rot) {
-            rot_head = tile / tph;
-            rot_j = tile % tph;
-        }
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 16 + r;
-            c_off[mt] = 0;
-            if (m >= M) continue;
-            const int pos = rope.row_pos[m], slot = rope.row_slot[m];
-            if (rot_head >= 0) {
-                if (q < 2) {
-                    const float4* c4 = (const float4*)(rope.cos_sin + (size_t)pos * rope.hd +
-                                                       2 * (8 * rot_j + 4 * q));
-                    const float4 c0 = c4[0], c1 = c4[1];
-                    cs[mt][0] = c0.x; cs[mt][1] = c0.y; cs[mt][2] = c0.z; cs[mt][3] = c0.w;
-                    cs[mt][4] = c1.x; cs[mt][5] = c1.y; cs[mt][6] = c1.z; cs[mt][7] = c1.w;
-                    if (rot_head >= rope.nh)
-                        c_off[mt] = cache_row_offset(rope.page_table, rope.table_stride, slot, pos,
-                                                     rope.page_size, rope.ring, rope.nkv,
-                                                     rot_head - rope.nh, rope.hd) + 8 * rot_j + 4 * q;
-                }
-            } else {
-                const int vrow = (tile - n_rot) * 16 + 4 * q;
-                c_off[mt] = cache_row_offset(rope.page_table, rope.table_stride, slot, pos,
-                                             rope.page_size, rope.ring, rope.nkv, vrow / rope.hd,
-                                             rope.hd) + vrow % rope.hd;
-            }
-        }
-    }
 
     // the parts' sums, added in part order by the waves of part 0
     if (kp > 1) {
@@ -274,14 +270,22 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
                         y0[i] = v[i] * c - o[i] * sn;
                         y1[i] = v[i] * sn + o[i] * c;
                     }
+                    // the row of the cache: [page][kv head][row in page][head_dim]
+                    const size_t c_off = (((size_t)e_page[mt] * rope.nkv + (rot_head - rope.nh)) *
+                                              rope.page_size + e_pos[mt] % rope.page_size) * rope.hd +
+                                         8 * rot_j + 4 * q;
                     bf16_t* dst = rot_head < rope.nh
                                       ? (bf16_t*)Y + (size_t)m * N + rot_head * rope.hd + 8 * rot_j + 4 * q
-                                      : rope.kcache + c_off[mt];
+                                      : rope.kcache + c_off;
                     *(uint2*)dst = make_uint2(pack_bf16x2(y0[0], y0[1]), pack_bf16x2(y0[2], y0[3]));
                     *(uint2*)(dst + rope.hd / 2) =
                         make_uint2(pack_bf16x2(y1[0], y1[1]), pack_bf16x2(y1[2], y1[3]));
                 } else {
-                    *(uint2*)(rope.vcache + c_off[mt]) =
+                    const int vrow = (tile - (rope.nh + rope.nkv) * (rope.hd / 16)) * 16 + 4 * q;
+                    const size_t c_off = (((size_t)e_page[mt] * rope.nkv + vrow / rope.hd) *
+                                              rope.page_size + e_pos[mt] % rope.page_size) * rope.hd +
+                                         vrow % rope.hd;
+                    *(uint2*)(rope.vcache + c_off) =
                         make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
                 }
             }
@@ -295,12 +299,11 @@ static int GR_TB = 0, GR_KP = 0, GR_PS = 0;   // tuning and tests: forced values
 extern "C" void illm_set_rows_shape(int tb, int kp, int piece) {
     GR_TB = (tb >= 2 && tb <= 4) ? tb : 0;
     GR_KP = (kp == 1 || kp == 2 || kp == 4) ? kp : 0;
-    GR_PS = (piece == 2 || piece == 4) ? piece : 0;
+    GR_PS = piece;            // (one piece size is built)
 }
 
 static void rows_shape(int tiles, int K, int mt, int* tb, int* kp, int* ps) {
-    *ps = GR_PS ? GR_PS : 2;
-    if (K % (*ps * 32)) *ps = 2;
+    *ps = 2;                  // pieces of 128 k measured no better at any shape, worse at 64 rows
     const int GR_PIECE = *ps;
     const int cus = 256;
     int best_tb = 4;
@@ -334,6 +337,7 @@ static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int
                        int tiles, const GrRope& rope, const GrScale& scale, hipStream_t st) {
     int tb, kp, ps;
     rows_shape(tiles, K, MT, &tb, &kp, &ps);
+    if (tb == 4 && kp > 2) kp = 2;                          // the kernel's launch bounds
     while (kp > 1 && (size_t)kp * 2 * MT * 16 * ps * 4 * 16 > 64 * 1024) kp /= 2;
     const size_t x_bytes = (size_t)kp * 2 * MT * 16 * ps * 4 * 16 + (MT == 1 ? 64 : 0);
     const size_t red_bytes = (size_t)(kp - 1) * tb * MT * 64 * 16;
@@ -342,15 +346,10 @@ static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int
 #define GO(TB_, PS_)                                                                              \
     hipLaunchKernelGGL((gemm_rows_kernel<MT, TB_, MODE, PS_>), grid, block, smem, st, x, wt, y,   \
                        y_dt, rows, N, K, tiles, kp, rope, scale)
-    if (ps == 2) {
-        if (tb == 2) GO(2, 2);
-        else if (tb == 3) GO(3, 2);
-        else GO(4, 2);
-    } else {
-        if (tb == 2) GO(2, 4);
-        else if (tb == 3) GO(3, 4);
-        else GO(4, 4);
-    }
+    (void)ps;
+    if (tb == 2) GO(2, 2);
+    else if (tb == 3) GO(3, 2);
+    else GO(4, 2);
 #undef GO
     return illm_launch_status();
 }
