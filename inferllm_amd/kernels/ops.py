@@ -396,6 +396,24 @@ def linear_planes_fits(x, w) -> bool:
             and w.plain.shape[1] >= 2 * w.plain.shape[0])
 
 
+def _cold_time(fn, reps: int = 5) -> float:
+    """Median milliseconds of `fn` with the last-level cache flushed before every run: a decode
+    step streams gigabytes between two uses of a matrix, so its products always run cold, and a
+    matrix of tens of megabytes timed back to back would be served from the cache."""
+    flush = torch.empty(1 << 28, dtype=torch.int16, device=torch.cuda.current_device())   # 512 MB
+    fn()
+    times = []
+    for _ in range(reps):
+        flush.zero_()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        end.record()
+        end.synchronize()
+        times.append(start.elapsed_time(end))
+    return sorted(times)[len(times) // 2]
+
+
 def measure_planes_from(w: "Weight") -> int:
     """Fewest rows from which `linear_planes` and the norm that adds its planes take less time
     than `linear_add` (whose norm the next product takes), measured at 16, 12, 8 and 4 rows."""
@@ -407,16 +425,7 @@ def measure_planes_from(w: "Weight") -> int:
     into = torch.zeros((SKINNY_BEST_ROWS, N), dtype=torch.float32, device=dev)
     nw = torch.ones(N, dtype=torch.bfloat16, device=dev)
 
-    def timed(fn) -> float:
-        fn()
-        fn()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(8):
-            fn()
-        end.record()
-        end.synchronize()
-        return start.elapsed_time(end)
+    timed = _cold_time
 
     first = NEVER_BELOW
     for rows in (16, 12, 8, 4):
@@ -693,16 +702,8 @@ def measure_rows_from_qkv(w_qkv: "Weight", nh: int, nkv: int, hd: int) -> int:
 
     def timed(rows: int, threshold: int) -> float:
         _plan.rows_from[key] = threshold
-        run = lambda: qkv_rope_store(x[:rows], w_qkv, table, pos[:rows], pos[:rows], kc, vc, pages,
-                                     64, 0, nh, nkv, hd)
-        run(); run()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(8):
-            run()
-        end.record()
-        end.synchronize()
-        return start.elapsed_time(end)
+        return _cold_time(lambda: qkv_rope_store(x[:rows], w_qkv, table, pos[:rows], pos[:rows], kc,
+                                                 vc, pages, 64, 0, nh, nkv, hd))
 
     first = ROWS_FROM
     try:

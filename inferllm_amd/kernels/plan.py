@@ -129,9 +129,10 @@ FIXED_CUTS: Dict[tuple, tuple] = {
 # (csrc/gemm_rows.hip) instead of the few-rows kernels, whose waves each read X for themselves.
 # Unlisted shapes: from 17 rows.
 FIXED_ROWS_FROM: Dict[tuple, int] = {
-    ("qkv", 6144, 4096): 5,        # 16 rows: 18.2 -> 14.7 us
-    ("qkv", 10240, 8192): 5,       # 16 rows: 45.9 -> 33.9 us
-    ("qkv", 12288, 4096): 13,      # 16 rows: 25.0 -> 21.5 us
+    ("qkv", 6144, 4096): 5,        # 16 rows: 18.2 -> 13.0 us
+    ("qkv", 10240, 8192): 5,       # 16 rows: 45.9 -> 30.9 us
+    ("qkv", 12288, 4096): 13,      # 16 rows: 25.0 -> 19.9 us
+    ("qkv", 15360, 5120): 5,
 }
 
 
