@@ -72,13 +72,26 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
     p_end = p_end < pieces ? p_end : pieces;
 
     if (MT == 1 && scale.ssq && wave == TB * kp - 1) {
-        // the scale of every X row, by the last wave while the others already stream W
-        for (int m = 0; m < M; ++m) {
-            float t = 0.f;
-            for (int p = lane; p < scale.parts; p += 64) t += scale.ssq[(size_t)m * scale.parts + p];
-            t = wave_sum(t);
-            if (lane == 0) row_rs[m] = 1.0f / sqrtf(t / (float)K + scale.eps);
+        // the scale of every X row, by the last wave while the others already stream W: all
+        // rows' loads are asked for at once, then one sum over the wave a row
+        float t[16];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) t[m] = 0.f;
+        for (int p = lane; p < scale.parts; p += 64) {
+            float v[16];
+#pragma unroll
+            for (int m = 0; m < 16; ++m)
+                v[m] = m < M ? scale.ssq[(size_t)m * scale.parts + p] : 0.f;
+#pragma unroll
+            for (int m = 0; m < 16; ++m) t[m] += v[m];
         }
+        float mine = 0.f;
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            const float sum = wave_sum(t[m]);
+            if (lane == m) mine = sum;
+        }
+        if (lane < 16) row_rs[lane] = 1.0f / sqrtf(mine / (float)K + scale.eps);
     }
 
     // staging of the part's X piece: unit u = row u / 8, 8 k at (u % 8) * 8; rows >= M read row
