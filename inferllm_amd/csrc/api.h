@@ -29,7 +29,7 @@ int illm_silu_mul(const void* gate_up, void* out, int dt, int T, int F, void* st
 
 // Rotate q and k of packed rows [q (nh*hd) | k (nkv*hd) | v (nkv*hd)] in place by the
 // angles of `cos_sin` ([max_pos][rot/2][2] float32; null: no rotation) at row_pos[t],
-// pairing 0 = (i, i + rot/2), 1 = (2i, 2i+1); then store k and v of each row in the
+// pairing 0 = (i, i + hd/2), 1 = (2i, 2i+1), i < rot/2; then store k and v of each row in the
 // paged cache of row_slot[t] (skipped when kcache is null).  With a ring of pages, slot_len
 // (length of every slot after the step) lets rows that a later row of the same step would
 // overwrite be skipped; it may be null when no sequence brings more than one row.

@@ -57,9 +57,12 @@ class Attention(Mixer):
         return KVSpec("window" if self.window else "full", self.nkv, self.hd, self.window)
 
     def load(self, tensors) -> None:
+        # the decode copy of q|k|v follows the tiles of the position encoding's fused kernel, if it
+        # has one; else plain tiles, which the few-rows product reads
+        mode = self.position.qkv_tile_mode(self.hd) if self.position is not None else "plain"
+        geometry = dict(nh=self.nh, nkv=self.nkv, hd=self.hd) if mode == "qkv" else {}
         self.w_qkv = ops.decode_weight(_fuse([self._take(tensors, n) for n in ("q", "k", "v")]),
-                                       "qkv", self.decode_copies, nh=self.nh, nkv=self.nkv,
-                                       hd=self.hd)
+                                       mode, self.decode_copies, **geometry)
         self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous(), "plain",
                                      self.decode_copies)
 

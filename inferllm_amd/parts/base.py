@@ -87,6 +87,8 @@ class Part:
 
 
 class Mixer(Part):
+    # The position encoding of the mixer's block, set by the block before `load` (None: none).
+    position = None
     # True: in a step of several tokens per sequence (`ctx.prefill`) the mixer also serves
     # sequences that already hold tokens, reading what it kept of them (rows then start at
     # `ctx.row_pos`, not at 0).  False: such a step must start every sequence at its first
@@ -139,6 +141,11 @@ class PositionEncoding(Part):
         """Encode q and k of packed rows in place and store k, v in the cache (if given)."""
         raise NotImplementedError
 
+    def qkv_tile_mode(self, head_dim: int) -> str:
+        """The tile order in which `project_qkv` wants the decode copy of the fused q|k|v matrix
+        (`ops.tile_rows`): "plain" unless the encoding has a fused kernel with tiles of its own."""
+        return "plain"
+
     def project_qkv(self, h: torch.Tensor, w_qkv: torch.Tensor, ctx: StepContext, nh: int,
                     nkv: int, hd: int, kcache, vcache, group) -> torch.Tensor:
         """Packed rows [q | k | v] = h . w_qkv^T, encoded, k and v stored.  An encoding may
@@ -169,6 +176,7 @@ class Block(Part):
         return out
 
     def load(self, tensors) -> None:
+        self.mixer.position = self.position      # a mixer may lay its matrices out for the encoding
         for p in self.parts():
             p.load(tensors)
 

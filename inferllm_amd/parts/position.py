@@ -62,6 +62,11 @@ class Rotary(PositionEncoding):
                        group.ring if group is not None else 0, nh, nkv, hd)
 
 
+    def qkv_tile_mode(self, head_dim: int) -> str:
+        # the fused product + rotation + store kernels pair a row with its partner head_dim / 2 on
+        fused = self.pairing == "half" and self.rotary_dim == head_dim and head_dim % 16 == 0
+        return "qkv" if fused else "plain"
+
     def project_qkv(self, h, w_qkv, ctx: StepContext, nh, nkv, hd, kcache, vcache, group):
         if (not ctx.prefill and kcache is not None and self.pairing == "half"
                 and self.rotary_dim == hd and ops.qkv_rope_store_fits(h, w_qkv, hd)

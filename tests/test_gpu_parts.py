@@ -92,6 +92,58 @@ def test_attention_part_whole_then_token_by_token(dtype, nh, nkv, hd, E, theta, 
             assert rel(out[b], want[b][head[b] + j]) < TOL[dtype], (b, j)
 
 
+@pytest.mark.parametrize("pairing,rot_frac", [("half", 1), ("interleaved", 1), ("half", 2)])
+def test_the_decode_copy_of_qkv_follows_the_position_part(pairing, rot_frac):
+    """The block tells its mixer which position encoding it has; the attention part lays the decode
+    copy of q|k|v out for that encoding's fused kernel if it has one (rotate-half over the whole
+    head) and in plain tiles otherwise, where the few-rows product reads it.  Either way prompt
+    and single tokens equal the plain computation."""
+    from inferllm_amd.config import PartSpec
+    from inferllm_amd.kernels import ops
+    from inferllm_amd.parts import build_part, part_class
+    dtype, nh, nkv, hd, E, theta = torch.bfloat16, 4, 2, 32, 64, 10000.0
+    rot_dim = hd // rot_frac
+    att = build_part("mixer", PartSpec("attention", {"hidden_size": E, "num_heads": nh, "num_kv_heads": nkv,
+                                                       "head_dim": hd}, {k: k for k in "qkvo"}))
+    rot = build_part("position", PartSpec("rotary", {"head_dim": hd, "rotary_dim": rot_dim, "theta": theta,
+                                                       "pairing": pairing, "max_positions": 512}))
+    norm = lambda n: build_part("norm", PartSpec("rms_norm", {"size": E, "eps": 1e-5}, {"weight": n}))
+    ffn = build_part("feed_forward", PartSpec("swiglu", {"hidden_size": E, "intermediate_size": 128},
+                                              {"gate": "g", "up": "u", "down": "d"}))
+    block = part_class("block", "pre_norm")(mixer=att, feed_forward=ffn, mixer_norm=norm("n1"),
+                                            feed_forward_norm=norm("n2"), position=rot)
+    w = {"q": rnd(nh * hd, E, seed=1, std=0.2), "k": rnd(nkv * hd, E, seed=2, std=0.2),
+         "v": rnd(nkv * hd, E, seed=3, std=0.2), "o": rnd(E, nh * hd, seed=4, std=0.2),
+         "g": rnd(128, E, seed=5, std=0.2), "u": rnd(128, E, seed=6, std=0.2), "d": rnd(E, 128, seed=7, std=0.2),
+         "n1": 1 + rnd(E, seed=8, std=0.1), "n2": 1 + rnd(E, seed=9, std=0.1)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    for part in [block] + block.parts():
+        part.decode_copies = True
+    block.load({k: v.to(DEV) for k, v in w.items()})
+    fused = pairing == "half" and rot_frac == 1
+    assert isinstance(att.w_qkv, ops.Weight) and att.w_qkv.mode == ("qkv" if fused else "plain")
+    S = 9
+    h = rnd(S, E, seed=20).to(dtype)
+
+    def plain(hh):
+        n = hh.shape[0]
+        q = P.linear(hh, w["q"]).reshape(n, nh, hd); k = P.linear(hh, w["k"]).reshape(n, nkv, hd)
+        v = P.linear(hh, w["v"]).reshape(n, nkv, hd)
+        # rot_dim / 2 pairs are rotated: (i, i + head_dim / 2) or (2 i, 2 i + 1), angles by rot_dim
+        rope = P.rope_rotate_half if pairing == "half" else P.rope_interleaved
+        q, k = rope(q, range(n), theta, rot_dim), rope(k, range(n), theta, rot_dim)
+        return P.linear(P.causal_attention(q, k, v), w["o"])
+    want = plain(h)
+    cache, slots = make_ctx([0], None, {0: att.kv_spec()}, dtype)
+    ctx = step_ctx(cache, slots, [0], [S - 2], dtype, True)
+    out = att.forward(h[:S - 2].to(DEV), ctx, 0, True, rot)
+    assert rel(out, want[:S - 2]) < TOL[dtype]
+    for j in (S - 2, S - 1):
+        ctx = step_ctx(cache, slots, [j], [1], dtype, False)
+        out = att.forward(h[j:j + 1].to(DEV), ctx, 0, True, rot)
+        assert rel(out[0], want[j]) < TOL[dtype], j
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norm_feed_forward_and_block_parts(dtype):
     from inferllm_amd.parts import build_part, part_class
