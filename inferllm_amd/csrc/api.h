@@ -58,6 +58,23 @@ int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens
                            int max_len, int nh, int nkv, int hd, float scale, int window,
                            void* stream);
 
+// The two above for steps whose rows go on from tokens the cache already holds (a prompt cut into
+// several steps): keys and values are read from the paged cache, which must hold the step's own
+// rows too by then; row r of sequence b stands at position seq_start[b] + r and sees the keys
+// 0 .. its position of the sequence in seq_slot[b].  The bfloat16 kernel needs pages of a multiple
+// of 64 rows.
+int illm_attn_prefill_paged_generic(const void* qkv, void* out, int dt, const int32_t* cu_seqlens,
+                                    const int32_t* seq_slot, const int32_t* seq_start,
+                                    const void* kcache, const void* vcache,
+                                    const int32_t* page_table, int table_stride, int page_size,
+                                    int ring, int n_seqs, int max_len, int nh, int nkv, int hd,
+                                    float scale, int window, void* stream);
+int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
+                                 const int32_t* seq_slot, const int32_t* seq_start,
+                                 const void* kcache, const void* vcache, const int32_t* page_table,
+                                 int table_stride, int page_size, int ring, int n_seqs, int max_len,
+                                 int nh, int nkv, int hd, float scale, int window, void* stream);
+
 // Tuning and tests: which prefill attention kernel head sizes up to 128 take: 0 the one with one
 // LDS buffer (which larger head sizes use), 2 the one with two buffers and one barrier a tile
 // (needs a positive scale), 1 (default) the second for head sizes 96 and 128 and sequences of

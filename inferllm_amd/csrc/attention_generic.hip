@@ -18,11 +18,24 @@
 #define AK 32  // keys of a tile
 #define NEG_INF (-INFINITY)
 
+// Where a step's rows go on from tokens the cache already holds (PAGED): keys and values are
+// read from the paged cache, which holds the step's own rows too by then, at absolute positions;
+// row r of sequence b stands at position seq_start[b] + r.
+struct AttnPages {
+    const void* kcache;
+    const void* vcache;
+    const int32_t* page_table;
+    const int32_t* seq_slot;
+    const int32_t* seq_start;
+    int table_stride, page_size, ring;
+};
+
 // grid (query tiles, heads, sequences); 256 threads: 8 per query row.
+template <bool PAGED>
 __global__ void __launch_bounds__(256)
 attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out, int dt,
                             const int32_t* __restrict__ cu, int nh, int nkv, int hd, float scale,
-                            int window) {
+                            int window, AttnPages pg) {
     extern __shared__ float smem[];
     const int hp = hd + 1;
     float* qs = smem;            // [AQ][hp]
@@ -33,6 +46,9 @@ attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out
     const int start = cu[b], len = cu[b + 1] - start;
     const int q0 = blockIdx.x * AQ;
     if (q0 >= len) return;
+    const int pos0 = PAGED ? pg.seq_start[b] : 0;       // position of the sequence's first row
+    const int slot = PAGED ? pg.seq_slot[b] : 0;
+    const int total = pos0 + len;                       // keys of the sequence after this step
     const int kvh = h / (nh / nkv);
     const size_t rowlen = (size_t)(nh + 2 * nkv) * hd;
     const int tid = threadIdx.x, i = tid >> 3, g = tid & 7;
@@ -47,9 +63,10 @@ attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out
     float acc[32];
 #pragma unroll
     for (int k = 0; k < 32; ++k) acc[k] = 0.f;
-    const int qpos = q0 + i;
-    const int k_hi = min(len, q0 + AQ);
-    int k_lo = window > 0 ? max(0, q0 - window + 1) : 0;
+    const int qrow = q0 + i;                            // row within the sequence's rows of the step
+    const int qpos = pos0 + qrow;                       // its position
+    const int k_hi = min(total, pos0 + q0 + AQ);
+    int k_lo = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
     k_lo = (k_lo / AK) * AK;
 
     for (int k0 = k_lo; k0 < k_hi; k0 += AK) {
@@ -57,10 +74,17 @@ attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out
         for (int e = tid; e < AK * hd; e += 256) {
             const int r = e / hd, d = e - r * hd;
             float kv = 0.f, vv = 0.f;
-            if (k0 + r < len) {
-                const size_t base = (size_t)(start + k0 + r) * rowlen;
-                kv = ld_f(qkv, dt, base + (size_t)(nh + kvh) * hd + d);
-                vv = ld_f(qkv, dt, base + (size_t)(nh + nkv + kvh) * hd + d);
+            if (k0 + r < total) {
+                if (PAGED) {
+                    const size_t at = cache_row_offset(pg.page_table, pg.table_stride, slot, k0 + r,
+                                                       pg.page_size, pg.ring, nkv, kvh, hd) + d;
+                    kv = ld_f(pg.kcache, dt, at);
+                    vv = ld_f(pg.vcache, dt, at);
+                } else {
+                    const size_t base = (size_t)(start + k0 + r) * rowlen;
+                    kv = ld_f(qkv, dt, base + (size_t)(nh + kvh) * hd + d);
+                    vv = ld_f(qkv, dt, base + (size_t)(nh + nkv + kvh) * hd + d);
+                }
             }
             ks[r * hp + d] = kv;
             vs[r * hp + d] = vv;
@@ -73,7 +97,7 @@ attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out
             const int j = g + 8 * c, kj = k0 + j;
             float a = 0.f;
             for (int d = 0; d < hd; ++d) a = fmaf(qs[i * hp + d], ks[j * hp + d], a);
-            const bool ok = qpos < len && kj <= qpos && (window <= 0 || kj > qpos - window);
+            const bool ok = qrow < len && kj <= qpos && (window <= 0 || kj > qpos - window);
             s[c] = ok ? a * scale : NEG_INF;
             tm = fmaxf(tm, s[c]);
         }
@@ -105,9 +129,9 @@ attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out
             }
         }
     }
-    if (qpos < len) {
+    if (qrow < len) {
         const float inv = 1.0f / l_i;
-        const size_t ob = (size_t)(start + qpos) * nh * hd + (size_t)h * hd;
+        const size_t ob = (size_t)(start + qrow) * nh * hd + (size_t)h * hd;
 #pragma unroll
         for (int k = 0; k < 32; ++k) {
             const int d = g + 8 * k;
@@ -116,27 +140,50 @@ attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out
     }
 }
 
-extern "C" int illm_attn_prefill_generic(const void* qkv, void* out, int dt,
-                                         const int32_t* cu_seqlens, int n_seqs, int max_len,
-                                         int nh, int nkv, int hd, float scale, int window,
-                                         void* stream) {
+template <bool PAGED>
+static int launch_prefill_generic(const void* qkv, void* out, int dt, const int32_t* cu_seqlens,
+                                  int n_seqs, int max_len, int nh, int nkv, int hd, float scale,
+                                  int window, const AttnPages& pg, hipStream_t stream) {
     if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
         !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535)
         return ILLM_ERR_ARG;
     if (n_seqs == 0 || max_len == 0) return ILLM_OK;
     const size_t smem = ((size_t)(AQ + 2 * AK) * (hd + 1) + AQ * (AK + 1)) * sizeof(float);
     if (smem > 48 * 1024) {
-        if (hipFuncSetAttribute((const void*)attn_prefill_generic_kernel,
+        if (hipFuncSetAttribute((const void*)attn_prefill_generic_kernel<PAGED>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)smem) != hipSuccess) {
             (void)hipGetLastError();
             return ILLM_ERR_ARG;
         }
     }
-    hipLaunchKernelGGL(attn_prefill_generic_kernel, dim3((max_len + AQ - 1) / AQ, nh, n_seqs),
-                       dim3(256), smem, (hipStream_t)stream, qkv, out, dt, cu_seqlens, nh, nkv, hd,
-                       scale, window);
+    hipLaunchKernelGGL(attn_prefill_generic_kernel<PAGED>, dim3((max_len + AQ - 1) / AQ, nh, n_seqs),
+                       dim3(256), smem, stream, qkv, out, dt, cu_seqlens, nh, nkv, hd, scale, window,
+                       pg);
     return illm_launch_status();
+}
+
+extern "C" int illm_attn_prefill_generic(const void* qkv, void* out, int dt,
+                                         const int32_t* cu_seqlens, int n_seqs, int max_len,
+                                         int nh, int nkv, int hd, float scale, int window,
+                                         void* stream) {
+    return launch_prefill_generic<false>(qkv, out, dt, cu_seqlens, n_seqs, max_len, nh, nkv, hd,
+                                         scale, window, AttnPages(), (hipStream_t)stream);
+}
+
+extern "C" int illm_attn_prefill_paged_generic(const void* qkv, void* out, int dt,
+                                               const int32_t* cu_seqlens, const int32_t* seq_slot,
+                                               const int32_t* seq_start, const void* kcache,
+                                               const void* vcache, const int32_t* page_table,
+                                               int table_stride, int page_size, int ring, int n_seqs,
+                                               int max_len, int nh, int nkv, int hd, float scale,
+                                               int window, void* stream) {
+    if (!seq_slot || !seq_start || !kcache || !vcache || !page_table || table_stride <= 0 ||
+        page_size <= 0)
+        return ILLM_ERR_ARG;
+    const AttnPages pg = {kcache, vcache, page_table, seq_slot, seq_start, table_stride, page_size, ring};
+    return launch_prefill_generic<true>(qkv, out, dt, cu_seqlens, n_seqs, max_len, nh, nkv, hd,
+                                        scale, window, pg, (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------- decode

@@ -33,11 +33,25 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 #define PF_BM 128     // query rows per block
 #define NEG_INF (-INFINITY)
 
-template <int HD>
+// PAGED: the step's rows go on from tokens the cache already holds.  Keys and values are read
+// from the paged cache (which holds the step's own rows too by then) at absolute positions, a
+// tile of 64 keys being one page or an aligned part of one; row r of sequence b stands at
+// position seq_start[b] + r.
+struct PfPages {
+    const bf16_t* kcache;
+    const bf16_t* vcache;
+    const int32_t* page_table;
+    const int32_t* seq_slot;
+    const int32_t* seq_start;
+    int table_stride, page_size, ring;
+};
+
+template <int HD, bool PAGED>
 __global__ void __launch_bounds__(256, (HD <= 128 ? 2 : 1))
 attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
                          const int32_t* __restrict__ cu, int n_qblk, int nh, int nkv,
-                         float scale_log2, int window, int hb_per_xcd, int n_hb, int zigzag) {
+                         float scale_log2, int window, int hb_per_xcd, int n_hb, int zigzag,
+                         PfPages pg) {
     constexpr int KLD = HD + 8;        // K tile row stride: 16 bytes of padding
     constexpr int VLD = PF_BN + 4;     // V^T row stride
     constexpr int KS = HD / 16;        // k-steps of the first product
@@ -59,13 +73,17 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     const int start = cu[b], len = cu[b + 1] - start;
     const int q0 = qb * PF_BM;
     if (q0 >= len) return;
+    const int pos0 = PAGED ? pg.seq_start[b] : 0;       // position of the sequence's first row
+    const int slot = PAGED ? pg.seq_slot[b] : 0;
+    const int total = pos0 + len;                       // keys of the sequence after this step
     const int kvh = h / (nh / nkv);
     const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
     const int tid = threadIdx.x, wave = wave_index(), lane = tid & 63;
     const int lq = lane & 31, half = lane >> 5;
     const int q_row0 = q0 + wave * 32;
-    const int q = q_row0 + lq;
+    const int q = q_row0 + lq;                          // row within the sequence's rows
     const int qc = q < len ? q : len - 1;
+    const int qp = pos0 + q;                            // its position
 
     uint4 qf[KS];
     {
@@ -80,24 +98,37 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
         for (int i = 0; i < 16; ++i) o[d][i] = 0.f;
     float m = NEG_INF, l = 0.f;
 
-    const int k_end = min(len, q0 + PF_BM);
-    int k_begin = window > 0 ? max(0, q0 - window + 1) : 0;
+    const int k_end = min(total, pos0 + q0 + PF_BM);
+    int k_begin = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
     k_begin = (k_begin / PF_BN) * PF_BN;
-    const int wk_end = min(len, q_row0 + 32);                       // this wave's last key + 1
-    const int wk_begin = window > 0 ? max(0, q_row0 - window + 1) : 0;
+    const int wk_end = min(total, pos0 + q_row0 + 32);              // this wave's last key + 1
+    const int wk_begin = window > 0 ? max(0, pos0 + q_row0 - window + 1) : 0;
 
     constexpr int NLD = (PF_BN * HD / 8) / 256;     // 16-byte pieces of K (and of V) per thread
     uint4 kpre[NLD], vpre[NLD];
     auto fetch = [&](int k0) {
+        size_t page_base = 0;                           // PAGED: the tile's page, this kv head
+        if (PAGED) {
+            int lp = k0 / pg.page_size;
+            if (pg.ring > 0) lp %= pg.ring;
+            const int phys = pg.page_table[(size_t)slot * pg.table_stride + lp];
+            page_base = ((size_t)phys * nkv + kvh) * pg.page_size;
+        }
 #pragma unroll
         for (int it = 0; it < NLD; ++it) {
             const int u = tid + it * 256;
             const int key = ((u >> 6) & 3) * 16 + (u & 15);
             const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
-            const int krow = min(k0 + key, len - 1);
-            const bf16_t* src = qkv + (size_t)(start + krow) * rowlen;
-            kpre[it] = *(const uint4*)(src + (size_t)(nh + kvh) * HD + ch * 8);
-            vpre[it] = *(const uint4*)(src + (size_t)(nh + nkv + kvh) * HD + ch * 8);
+            const int krow = min(k0 + key, total - 1);
+            if (PAGED) {
+                const size_t at = (page_base + krow % pg.page_size) * HD + ch * 8;
+                kpre[it] = *(const uint4*)(pg.kcache + at);
+                vpre[it] = *(const uint4*)(pg.vcache + at);
+            } else {
+                const bf16_t* src = qkv + (size_t)(start + krow) * rowlen;
+                kpre[it] = *(const uint4*)(src + (size_t)(nh + kvh) * HD + ch * 8);
+                vpre[it] = *(const uint4*)(src + (size_t)(nh + nkv + kvh) * HD + ch * 8);
+            }
         }
     };
     if (k_begin < k_end) fetch(k_begin);
@@ -136,7 +167,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
                                                                  0, 0, 0);
             }
         }
-        const bool need_mask = (k0 + PF_BN > q_row0 + 1) || (k0 + PF_BN > len) || (window > 0);
+        const bool need_mask = (k0 + PF_BN > pos0 + q_row0 + 1) || (k0 + PF_BN > total) || (window > 0);
         float mx = NEG_INF;
         if (need_mask) {                 // the same for the whole wave: one branch, two bodies
 #pragma unroll
@@ -144,7 +175,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int key = k0 + sub * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
-                    const bool ok = key <= q && key < len && (window <= 0 || key > q - window);
+                    const bool ok = key <= qp && key < total && (window <= 0 || key > qp - window);
                     const float v = ok ? s[sub][i] * scale_log2 : NEG_INF;
                     s[sub][i] = v;
                     mx = fmaxf(mx, v);
@@ -464,13 +495,14 @@ extern "C" void illm_set_prefill_two_buffers(int on) { PF_TWO_BUFFERS = on; }
 
 template <int HD>
 static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_seqs, int max_len,
-                          int nh, int nkv, float scale, int window, hipStream_t st) {
+                          int nh, int nkv, float scale, int window, hipStream_t st,
+                          const PfPages* pg = nullptr) {
     const int n_qblk = (max_len + PF_BM - 1) / PF_BM;
     const long long n_hb = (long long)nh * n_seqs;
     const long long hb_per_xcd = (n_hb + 7) / 8;
     const long long blocks = 8 * hb_per_xcd * n_qblk;
     if (blocks > 0x7fffffffLL) return ILLM_ERR_ARG;
-    if constexpr (HD <= 128) {
+    if constexpr (HD <= 128) if (!pg) {
         // measured at 32 heads: head size 128, 2,048 keys 81 -> 76 us, 4,096 keys 236 -> 214; head
         // size 64 and sequences of 512 lose a tenth (a tile more of set-up before the first product)
         if (PF_TWO_BUFFERS == 2 || (PF_TWO_BUFFERS == 1 && HD >= 96 && max_len >= 1024 && scale > 0.f)) {
@@ -481,10 +513,17 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
             return illm_launch_status();
         }
     }
-    hipLaunchKernelGGL(attn_prefill_mfma_kernel<HD>, dim3((unsigned)blocks), dim3(256), 0, st,
+    if (pg) {
+        hipLaunchKernelGGL((attn_prefill_mfma_kernel<HD, true>), dim3((unsigned)blocks), dim3(256), 0,
+                           st, (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
+                           scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
+                           hb_per_xcd * n_qblk <= 64 ? 1 : 0, *pg);
+        return illm_launch_status();
+    }
+    hipLaunchKernelGGL((attn_prefill_mfma_kernel<HD, false>), dim3((unsigned)blocks), dim3(256), 0, st,
                        (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
                        scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
-                       hb_per_xcd * n_qblk <= 64 ? 1 : 0);   // 32 CUs of an XCD, two blocks each
+                       hb_per_xcd * n_qblk <= 64 ? 1 : 0, PfPages());   // 32 CUs of an XCD, two blocks each
     return illm_launch_status();
 }
 
@@ -506,5 +545,34 @@ extern "C" int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t*
         case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
         case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
         default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+    }
+}
+
+// The same where the step's rows go on from tokens the cache already holds: keys and values from
+// the paged cache (bfloat16, pages of a multiple of 64 rows), row r of sequence b at position
+// seq_start[b] + r.  The step's own keys and values must be in the cache already.
+extern "C" int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
+                                            const int32_t* seq_slot, const int32_t* seq_start,
+                                            const void* kcache, const void* vcache,
+                                            const int32_t* page_table, int table_stride,
+                                            int page_size, int ring, int n_seqs, int max_len, int nh,
+                                            int nkv, int hd, float scale, int window, void* stream) {
+    if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
+        hd % 32 || !seq_slot || !seq_start || !kcache || !vcache || !page_table ||
+        table_stride <= 0 || page_size <= 0 || page_size % PF_BN)
+        return ILLM_ERR_ARG;
+    if (n_seqs == 0 || max_len == 0) return ILLM_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const PfPages pg = {(const bf16_t*)kcache, (const bf16_t*)vcache, page_table, seq_slot, seq_start,
+                        table_stride, page_size, ring};
+    switch (hd) {
+        case 32: return launch_prefill<32>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 64: return launch_prefill<64>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 96: return launch_prefill<96>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 128: return launch_prefill<128>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
     }
 }

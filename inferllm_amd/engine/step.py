@@ -1,5 +1,8 @@
 """The step function: one batch of sequences, either all at their first token
-(whole prompts of unequal lengths) or all going on by one token.
+(whole prompts of unequal lengths) or all going on by one token; if every mixer of
+the model says it can go on from what it kept by several tokens (attention without a
+window does: its rows then attend over the paged cache), also any mix of starting
+sequences and sequences that go on by any number of tokens (a prompt cut into steps).
 
 It runs only the tokens it is given, packed as one batch, against the cache that
 earlier steps left, and returns float32 logits at the places asked for.  Steps
@@ -168,12 +171,12 @@ class StepRunner:
             cu.append(cu[-1] + n)
         T, B = len(tokens), len(entries)
         host = torch.tensor(tokens + pos + slot + cu + [e.slot for e in entries]
-                            + [s + len(e.tokens) for e, s in zip(entries, starts)] + want,
-                            dtype=torch.int32)
+                            + [s + len(e.tokens) for e, s in zip(entries, starts)]
+                            + [int(s) for s in starts] + want, dtype=torch.int32)
         meta = host.to(self.device)
         o = 0
         parts = []
-        for n in (T, T, T, B + 1, B, B, len(want)):
+        for n in (T, T, T, B + 1, B, B, B, len(want)):
             parts.append(meta[o:o + n])
             o += n
         ctx = StepContext(
@@ -181,8 +184,9 @@ class StepRunner:
             tokens=parts[0], row_pos=parts[1], row_slot=parts[2], cu_seqlens=parts[3],
             seq_slot=parts[4], seq_len=parts[5],
             max_len=max(s + len(e.tokens) for e, s in zip(entries, starts)),
-            cache=self.cache)
-        return self.model.forward(ctx, parts[6] if want else None)
+            cache=self.cache, seq_start=parts[6], max_rows=max(len(e.tokens) for e in entries),
+            continues=any(int(s) > 0 for s in starts))
+        return self.model.forward(ctx, parts[7] if want else None)
 
     def _decode(self, entries: Sequence[StepEntry], starts: Sequence[int],
                 device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:

@@ -806,6 +806,38 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
     return out
 
 
+def attn_prefill_paged(qkv: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: torch.Tensor,
+                       seq_start: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                       page_table: torch.Tensor, page_size: int, ring: int, n_seqs: int,
+                       max_len: int, nh: int, nkv: int, hd: int, scale: float,
+                       window: int) -> torch.Tensor:
+    """Causal attention of a step's packed rows that go on from tokens the cache already holds:
+    row r of sequence b stands at position seq_start[b] + r and attends over the keys 0 .. its
+    position of the paged cache, which must hold the step's own keys and values too by now.
+    `max_len`: the most rows a sequence brings.  Returns [T, nh * hd]."""
+    _gpu(qkv, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table)
+    _i32(cu_seqlens, n_seqs + 1); _i32(seq_slot, n_seqs); _i32(seq_start, n_seqs); _i32(page_table)
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] >= nh * hd, "attn_prefill_paged: packed rows [q | ...]")
+    _need(nh % nkv == 0, "attn_prefill_paged: heads must be a multiple of kv heads")
+    _need(kcache.dtype == qkv.dtype and vcache.shape == kcache.shape and
+          kcache.shape[1:] == (nkv, page_size, hd) and page_table.dim() == 2,
+          "attn_prefill_paged: cache shape or dtype")
+    _need(qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_prefill_paged: packed qkv rows")
+    out = torch.empty((T, nh * hd), dtype=qkv.dtype, device=qkv.device)
+    if qkv.dtype == torch.bfloat16 and hd % 32 == 0 and page_size % 64 == 0:
+        _check(_lib().illm_attn_prefill_paged_bf16(
+            _p(qkv), _p(out), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache), _p(vcache),
+            _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_len, nh, nkv, hd,
+            ctypes.c_float(scale), window, _stream()), f"attn_prefill_paged_bf16 (head_dim {hd})")
+        return out
+    _check(_lib().illm_attn_prefill_paged_generic(
+        _p(qkv), _p(out), _code(qkv), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache),
+        _p(vcache), _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_len, nh, nkv,
+        hd, ctypes.c_float(scale), window, _stream()), f"attn_prefill_paged (head_dim {hd})")
+    return out
+
+
 def decode_splits(B: int, nkv: int, max_len: int, nh: int = 0, hd: int = 0):
     """(nsplit, waves): how to cut the keys of a decode step among blocks (`nsplit` ranges per
     sequence, combined by a merge kernel) and among the waves of a block (combined in LDS).

@@ -28,11 +28,19 @@ class Attention(Mixer):
     1/sqrt(head_dim) after the dot product (op.cpp:488).  Query head h reads kv head
     h / (num_heads / num_kv_heads) (src/kern/naive/naive.cpp:576-604).  `window`
     keeps only the last `window` keys visible; `softmax_scale` replaces the default.
-    Whole prompts attend over the step's own rows; single tokens over the cache.
+    Whole prompts attend over the step's own rows; single tokens, and rows that go on from
+    tokens of earlier steps, over the cache.
     """
 
     adds_residual = True
     takes_normed_rows = True
+
+    @property
+    def takes_continuations(self) -> bool:
+        """A step of several tokens may go on from keys the cache holds (a prompt cut into
+        steps): its rows then attend over the paged cache.  Not with a window, whose ring of
+        pages a long step overwrites while it is still read."""
+        return self.window is None
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: Optional[int] = None, softmax_scale: Optional[float] = None, tensors=None):
@@ -87,12 +95,18 @@ class Attention(Mixer):
             q = ops.linear(h, ops.plain_weight(self.w_qkv)[: nh * hd])
             if position is not None:
                 position.on_qkv(q, ctx, nh, 0, hd, None, None, None)
-            if ctx.prefill:
+            if ctx.prefill and not ctx.continues:
                 kv = ctx.exchange[("kv_rows", line)][:, nh * hd:]
             else:
-                kv = q.new_zeros((q.shape[0], 2 * nkv * hd))   # single tokens read the cache
+                kv = q.new_zeros((q.shape[0], 2 * nkv * hd))   # read from the cache
             qkv = torch.cat([q, kv], dim=1)
-        if ctx.prefill:
+        if ctx.prefill and ctx.continues:
+            # some sequence goes on from tokens of earlier steps: over the cache, which holds
+            # this step's keys and values too by now
+            o = ops.attn_prefill_paged(qkv, ctx.cu_seqlens, ctx.seq_slot, ctx.seq_start, kc, vc,
+                                       group.table, group.page_size, group.ring, ctx.n_seqs,
+                                       ctx.max_rows, nh, nkv, hd, self.scale, window)
+        elif ctx.prefill:
             o = ops.attn_prefill(qkv, ctx.cu_seqlens, ctx.n_seqs, ctx.max_len, nh, nkv, hd,
                                  self.scale, window)
         else:

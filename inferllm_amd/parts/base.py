@@ -45,6 +45,11 @@ class StepContext:
     seq_len: torch.Tensor             # [seqs] length of each sequence after this step
     max_len: int                      # longest sequence after this step (host number)
     cache: CacheManager
+    # steps of several tokens a sequence (`prefill`): where each sequence's rows begin, and whether
+    # any begins beyond position 0 (the step goes on from what the cache and the states hold)
+    seq_start: Optional[torch.Tensor] = None     # [seqs] position of the sequence's first row
+    max_rows: int = 0                 # most rows a sequence brings (host number)
+    continues: bool = False
     exchange: Dict[Any, Any] = field(default_factory=dict)   # between runs of layers in one step
 
 

@@ -130,6 +130,35 @@ def attn_prefill(qkv, cu_seqlens, n_seqs, max_len, nh, nkv, hd, scale, window):
     return out
 
 
+def attn_prefill_paged(qkv, cu_seqlens, seq_slot, seq_start, kcache, vcache, page_table, page_size,
+                       ring, n_seqs, max_len, nh, nkv, hd, scale, window):
+    """Rows that go on from tokens the cache holds: row r of sequence b stands at position
+    seq_start[b] + r and sees the keys 0 .. its position, all read from the paged cache."""
+    T = qkv.shape[0]
+    view = qkv.view(T, nh + 2 * nkv, hd)
+    out = torch.zeros(T, nh * hd, dtype=qkv.dtype, device=qkv.device)
+    for b in range(n_seqs):
+        s0, s1 = int(cu_seqlens[b]), int(cu_seqlens[b + 1])
+        if s1 == s0:
+            continue
+        slot, p0 = int(seq_slot[b]), int(seq_start[b])
+        total = p0 + (s1 - s0)
+        first = max(0, p0 - window + 1) if window and window > 0 else 0
+        ks, vs = [], []
+        for pos in range(first, total):
+            page, r = cache_offsets(page_table, slot, pos, page_size, ring)
+            ks.append(kcache[page, :, r, :])
+            vs.append(vcache[page, :, r, :])
+        k, v = torch.stack(ks), torch.stack(vs)
+        idx = torch.arange(first, total)
+        for a in range(s1 - s0):
+            vis = idx <= p0 + a
+            if window and window > 0:
+                vis = vis & (idx > p0 + a - window)
+            out[s0 + a] = _attend(view[s0 + a, :nh], k, v, scale, vis).reshape(-1).to(qkv.dtype)
+    return out
+
+
 def decode_splits(B, nkv, max_len, nh=0, hd=0):
     return 2, 1
 
@@ -223,5 +252,5 @@ def patch(monkeypatch):
     from inferllm_amd.kernels import ops
     for name in ("embed", "add_rmsnorm", "silu_mul", "rope_store", "linear", "gemm_generic", "gate_up_silu", "qkv_rope_store_fits",
                  "linear_add_fits",
-                 "attn_prefill", "decode_splits", "attn_decode", "argmax", "sample"):
+                 "attn_prefill", "attn_prefill_paged", "decode_splits", "attn_decode", "argmax", "sample"):
         monkeypatch.setattr(ops, name, globals()[name])

@@ -227,6 +227,35 @@ def test_attn_prefill_mfma(nh, nkv, hd, lens, window):
         lib.illm_set_prefill_two_buffers(1)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,starts,rows,page", [
+    (4, 2, 32, [0, 70, 5], [40, 30, 1], 64), (8, 8, 128, [200, 0], [130, 64], 64), (3, 1, 48, [17, 64], [9, 200], 64),
+    (6, 2, 24, [3], [5], 16), (2, 2, 256, [63], [66], 64), (32, 8, 128, [1000, 37, 0], [300, 27, 129], 64)])
+def test_attn_prefill_paged(dtype, nh, nkv, hd, starts, rows, page):
+    """A step's rows that go on from tokens the cache holds (a prompt cut into steps): attention
+    over the paged cache at absolute positions, several sequences with different starts (0
+    among them: a sequence that begins while others go on).  Stale rows of the pages are NaN."""
+    lens = [s + r for s, r in zip(starts, rows)]
+    pt, kc, vc, slots, _ = paged_case(dtype, nkv, hd, lens, page)
+    for b, sl in enumerate(slots.tolist()):                    # rows beyond a sequence's end: NaN
+        lp, r = divmod(lens[b], page)
+        if r:
+            kc[int(pt[sl, lp]), :, r:] = float("nan"); vc[int(pt[sl, lp]), :, r:] = float("nan")
+    kc[-1] = float("nan"); vc[-1] = float("nan")
+    T = sum(rows)
+    qkv = rnd(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=11)
+    qkv[:, nh * hd:] = float("nan")                            # k and v come from the cache alone
+    cu = torch.tensor([0] + list(torch.tensor(rows).cumsum(0)), dtype=torch.int32)
+    st = torch.tensor(starts, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(hd)
+    got = ops().attn_prefill_paged(qkv.to(DEV), cu.to(DEV), slots.to(DEV), st.to(DEV), kc.to(DEV), vc.to(DEV),
+                                   pt.to(DEV), page, 0, len(rows), max(rows), nh, nkv, hd, scale, 0)
+    want = R.attn_prefill_paged(qkv, cu, slots, st, kc, vc, pt, page, 0, len(rows), max(rows), nh, nkv, hd,
+                                scale, 0)
+    assert torch.isfinite(got.float()).all()
+    close(got, want, dtype, scale=2)
+
+
 def test_attn_prefill_finds_one_far_key():
     """One early key is made to stand out for a late query: the output is that key's value."""
     nh, nkv, hd, n = 2, 1, 128, 700

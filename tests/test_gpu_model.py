@@ -236,6 +236,36 @@ def test_unequal_batches_with_slot_reuse(tmp_path_factory, name, dtype, graphs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
+def test_a_prompt_cut_into_steps(tmp_path_factory, name, dtype):
+    """Attention goes on from the cache by any number of tokens a step: a prompt cut at odd
+    places (also across cache pages), a second sequence that starts while the first goes on, a
+    step in which one brings many tokens and the other one; every position's logits equal the
+    plain model's, whole."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, name, dtype, max_batch=2)
+    assert eng.model.one_token_mixers == []
+    a, b = requests_for(config, [120, 75], seed=12)
+    wa, wb = plain(a), plain(b)
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    got_a, got_b = [], []
+    got_a.append(eng.step([StepEntry(sa, a[:30], list(range(30)))]).clone())
+    got_a.append(eng.step([StepEntry(sa, a[30:31], [0])]).clone())                 # one token: a decode step
+    out = eng.step([StepEntry(sa, a[31:100], list(range(69))), StepEntry(sb, b[:70], list(range(70)))])
+    got_a.append(out[:69].clone()); got_b.append(out[69:].clone())
+    out = eng.step([StepEntry(sb, b[70:71], [0]), StepEntry(sa, a[100:], list(range(20)))])
+    got_b.append(out[:1].clone()); got_a.append(out[1:].clone())
+    for t in b[71:]:
+        got_b.append(eng.step([StepEntry(sb, [t], [0])]).clone())
+    for got, want, who in ((got_a, wa, "a"), (got_b, wb, "b")):
+        per_pos = (torch.cat(got).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+        assert float(per_pos.max()) < BUDGET[dtype], \
+            f"request {who}: first bad position {int((per_pos >= BUDGET[dtype]).nonzero()[0])}"
+    eng.free_slot(sa); eng.free_slot(sb)
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(tmp_path_factory, dtype):
     """Decode 250 tokens one by one after a 3-token prompt (crossing several pages)."""
     from inferllm_amd import StepEntry

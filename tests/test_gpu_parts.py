@@ -400,10 +400,10 @@ def test_a_mixer_with_state_under_decode_graphs(tmp_path, graphs):
 
 
 def test_a_mixer_says_whether_it_goes_on_by_several_tokens(tmp_path):
-    """The rule "all start, or all go on by one" belongs to the mixers: attention reads a prompt's
-    keys from the step's own rows and refuses a continuation by several tokens; a mixer with
-    state of fixed size takes one, and a prompt can be cut into steps of any lengths, also mixed
-    with sequences that start."""
+    """The rule "all start, or all go on by one" belongs to the mixers: a mixer that says it takes
+    continuations (one with state of fixed size here; attention without a window too) lets a
+    prompt be cut into steps of any lengths, also mixed with sequences that start; a model with
+    a mixer that does not is refused such steps."""
     import inferllm_amd as I
     from inferllm_amd.engine.step import StepError
     from tiny import TINY_A, make_model_dir, random_ids, read_weights
@@ -422,13 +422,18 @@ def test_a_mixer_says_whether_it_goes_on_by_several_tokens(tmp_path):
     assert rel(out[0], wa[7]) < 2e-5 and rel(out[1], wa[19]) < 2e-5 and rel(out[2], wb[4]) < 2e-5
     out = eng.step([I.StepEntry(sa, a[20:], [9]), I.StepEntry(sb, b[5:6], [0])])       # ten tokens and one
     assert rel(out[0], wa[29]) < 2e-5 and rel(out[1], wb[5]) < 2e-5
-    # attention does not: the step function refuses and says which part is the reason
+    # the host-reading form of the mixer does not say it can: the step function refuses and says
+    # which part is the reason; attention without a window can (tests/test_gpu_model.py)
+    cfg2 = dict(cfg, mixer="toy_running_mean")
+    d2 = I.write_random_model(str(tmp_path / "toy2"), I.config_from_dict(cfg2), seed=6)
+    e2 = I.Engine.from_pretrained(d2, dtype="float32", max_batch=2, max_seq_len=256)
+    s = e2.alloc_slot()
+    e2.step([I.StepEntry(s, [1, 2, 3], [])])
+    with pytest.raises(StepError, match="RunningMean cannot go on by several"):
+        e2.step([I.StepEntry(s, [4, 5], [1])])
+    assert e2.cache.length(s) == 3                       # refused before anything was reserved
     la = I.Engine.from_pretrained(make_model_dir(tmp_path, TINY_A, seed=1), dtype="float32", max_batch=2)
-    s = la.alloc_slot()
-    la.step([I.StepEntry(s, [1, 2, 3], [])])
-    with pytest.raises(StepError, match="Attention cannot go on by several"):
-        la.step([I.StepEntry(s, [4, 5], [1])])
-    assert la.cache.length(s) == 3                       # refused before anything was reserved
+    assert la.model.one_token_mixers == []
 
 
 def test_embedding_and_head_parts():

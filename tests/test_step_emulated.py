@@ -101,10 +101,16 @@ def test_step_refuses_mixed_phases_and_bad_ids(tmp_path, emulated):
     r = build_runner(config, w)
     a, b = r.cache.alloc_slot(), r.cache.alloc_slot()
     r.step([StepEntry(a, [1, 2, 3], [])])
-    with pytest.raises(StepError, match="all start"):
+    # a model with a mixer that cannot go on by several tokens (attention with a window, a mixer
+    # that does not say it can) takes steps that all start or all go on by one token only
+    assert r.model.one_token_mixers == []
+    r.model.one_token_mixers = ["SomeMixer"]
+    with pytest.raises(StepError, match="all start.*SomeMixer"):
         r.step([StepEntry(a, [4], [0]), StepEntry(b, [1, 2], [1])])
     with pytest.raises(StepError, match="all start"):
         r.step([StepEntry(a, [4, 5], [0])])
+    assert r.cache.length(a) == 3 and r.cache.length(b) == 0          # refused before anything was reserved
+    r.model.one_token_mixers = []
     with pytest.raises(StepError, match="vocabulary"):
         r.step([StepEntry(a, [256], [0])])
     with pytest.raises(StepError, match="wanted place"):
@@ -112,3 +118,31 @@ def test_step_refuses_mixed_phases_and_bad_ids(tmp_path, emulated):
     with pytest.raises(StepError, match="twice"):
         r.step([StepEntry(a, [5], [0]), StepEntry(a, [6], [0])])
     assert r.step([StepEntry(a, [5], [])]) is None
+
+
+
+def test_a_prompt_cut_into_steps_equals_the_whole_prompt(tmp_path, emulated):
+    """Attention goes on from the cache by any number of tokens: a prompt in pieces of 30, 1 and
+    39 tokens, a second sequence that starts while the first goes on, then single tokens; every
+    position's logits equal the plain model's."""
+    config = CONFIGS["B"]
+    d = make_model_dir(tmp_path, config, seed=6, gain=4.0)
+    w = read_weights(d)
+    V = config["vocab_size"]
+    a, b = random_ids(75, V, 1), random_ids(24, V, 2)
+    wa, wb = plain_llama.forward_logits(config, w, a), plain_llama.forward_logits(config, w, b)
+    r = build_runner(config, w, max_tokens=64 * 4, max_slots=2)
+    sa, sb = r.cache.alloc_slot(), r.cache.alloc_slot()
+    got = r.step([StepEntry(sa, a[:30], list(range(30)))])
+    assert (got.double() - wa[:30]).abs().max() < 1e-5
+    got = r.step([StepEntry(sa, a[30:31], [0])])                              # one token: a decode step
+    assert (got.double() - wa[30:31]).abs().max() < 1e-5
+    got = r.step([StepEntry(sa, a[31:70], list(range(39))), StepEntry(sb, b[:20], [0, 19])])
+    assert (got[:39].double() - wa[31:70]).abs().max() < 1e-5
+    assert (got[39:].double() - wb[[0, 19]]).abs().max() < 1e-5
+    got = r.step([StepEntry(sa, a[70:], [4]), StepEntry(sb, b[20:21], [0])])   # five tokens and one
+    assert (got[0].double() - wa[74]).abs().max() < 1e-5 and (got[1].double() - wb[20]).abs().max() < 1e-5
+    got = r.step([StepEntry(sb, [b[21]], [0])])
+    assert (got[0].double() - wb[21]).abs().max() < 1e-5
+    r.cache.free_slot(sa); r.cache.free_slot(sb)
+    r.cache.check()
