@@ -170,8 +170,8 @@ int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int 
                              int nh, int nkv, int hd, const float* ssq, int parts, float eps,
                              void* stream);
 // Tuning and tests: tiles a block of these products takes (2, 3, 4) and parts of K (1, 2, 4;
-// four tiles: 1, 2); 0: the library's own choice.  `piece` is ignored (one piece size is built).
-void illm_set_rows_shape(int tb, int kp, int piece);
+// four tiles: 1, 2); 0: the library's own choice.
+void illm_set_rows_shape(int tb, int kp);
 
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
 // product, `ssq` included.  waves_wanted: waves per block (0: the default choice).

@@ -308,16 +308,17 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
 
 // Tiles a block takes (2, 3 or 4) and parts of K (1, 2 or 4; a part has at least 4 pieces): a
 // block or two per compute unit, as even as can be, and at least eight waves a compute unit.
-static int GR_TB = 0, GR_KP = 0, GR_PS = 0;   // tuning and tests: forced values (0: the choice below)
-extern "C" void illm_set_rows_shape(int tb, int kp, int piece) {
+static int GR_TB = 0, GR_KP = 0;          // tuning and tests: forced values (0: the choice below)
+extern "C" void illm_set_rows_shape(int tb, int kp) {
     GR_TB = (tb >= 2 && tb <= 4) ? tb : 0;
     GR_KP = (kp == 1 || kp == 2 || kp == 4) ? kp : 0;
-    GR_PS = piece;            // (one piece size is built)
 }
 
-static void rows_shape(int tiles, int K, int mt, int* tb, int* kp, int* ps) {
-    *ps = 2;                  // pieces of 128 k measured no better at any shape, worse at 64 rows
-    const int GR_PIECE = *ps;
+#define GR_PIECE_STEPS 2      // k-steps of 32 in a piece (pieces of 128 k measured no better at 16
+                              // rows and worse at 64)
+
+static void rows_shape(int tiles, int K, int* tb, int* kp) {
+    const int GR_PIECE = GR_PIECE_STEPS;
     const int cus = 256;
     int best_tb = 4;
     double best = -1.0;
@@ -348,10 +349,10 @@ static void rows_shape(int tiles, int K, int mt, int* tb, int* kp, int* ps) {
 template <int MT, int MODE>
 static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int rows, int N, int K,
                        int tiles, const GrRope& rope, const GrScale& scale, hipStream_t st) {
-    int tb, kp, ps;
-    rows_shape(tiles, K, MT, &tb, &kp, &ps);
+    int tb, kp;
+    rows_shape(tiles, K, &tb, &kp);
     if (tb == 4 && kp > 2) kp = 2;                          // the kernel's launch bounds
-    while (kp > 1 && (size_t)kp * 2 * MT * 16 * ps * 4 * 16 > 64 * 1024) kp /= 2;
+    constexpr int ps = GR_PIECE_STEPS;
     const size_t x_bytes = (size_t)kp * 2 * MT * 16 * ps * 4 * 16 + (MT == 1 ? 64 : 0);
     const size_t red_bytes = (size_t)(kp - 1) * tb * MT * 64 * 16;
     const size_t smem = x_bytes > red_bytes ? x_bytes : red_bytes;
@@ -359,10 +360,9 @@ static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int
 #define GO(TB_, PS_)                                                                              \
     hipLaunchKernelGGL((gemm_rows_kernel<MT, TB_, MODE, PS_>), grid, block, smem, st, x, wt, y,   \
                        y_dt, rows, N, K, tiles, kp, rope, scale)
-    (void)ps;
-    if (tb == 2) GO(2, 2);
-    else if (tb == 3) GO(3, 2);
-    else GO(4, 2);
+    if (tb == 2) GO(2, GR_PIECE_STEPS);
+    else if (tb == 3) GO(3, GR_PIECE_STEPS);
+    else GO(4, GR_PIECE_STEPS);
 #undef GO
     return illm_launch_status();
 }

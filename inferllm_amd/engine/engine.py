@@ -101,6 +101,13 @@ class Engine:
                             and w.shape[1] >= 2 * w.shape[0] and w.shape[0] <= ops.MID_MAX_COLS
                             and w.shape[0] % 4 == 0):
                         self.plan.planes_from[tuple(w.shape)] = ops.measure_planes_from(w)
+                # a mixer that keeps a fused q|k|v matrix in its fused kernel's tile order
+                w = getattr(part, "w_qkv", None)
+                if (isinstance(w, ops.Weight) and w.mode == "qkv" and w.tiled is not None
+                        and w.shape[1] % 64 == 0
+                        and ("qkv",) + tuple(w.shape) not in self.plan.rows_from):
+                    self.plan.rows_from[("qkv",) + tuple(w.shape)] = ops.measure_rows_from_qkv(
+                        w, part.nh, part.nkv, part.hd)
         limit = self.spec.max_positions
         self.max_seq_len = min(int(max_seq_len), limit) if max_seq_len else limit
         self.max_batch = int(max_batch)

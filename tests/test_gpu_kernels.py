@@ -838,26 +838,26 @@ def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed, copy, 
 
 
 # ---------------------------------------------------------------- products of 9 to 128 rows
-# (tiles a block, parts of K, k-steps in a piece)
-_ROWS_SHAPES = [(None, None, None), (2, 1, 2), (2, 4, 4), (3, 2, 2), (3, 2, 4), (4, 1, 4), (4, 4, 2)]
+# (tiles a block, parts of K)
+_ROWS_SHAPES = [(None, None), (2, 1), (2, 4), (3, 2), (3, 4), (4, 1), (4, 2)]
 
 
 @pytest.fixture
 def rows_shape():
     """Forces the block shape of the rows kernels and gives the library's own choice back after."""
     lib = ops()._lib()
-    yield lambda tb, kp, ps=0: lib.illm_set_rows_shape(tb or 0, kp or 0, ps or 0)
-    lib.illm_set_rows_shape(0, 0, 0)
+    yield lambda tb, kp: lib.illm_set_rows_shape(tb or 0, kp or 0)
+    lib.illm_set_rows_shape(0, 0)
 
 
-@pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
+@pytest.mark.parametrize("tb,kp", _ROWS_SHAPES)
 @pytest.mark.parametrize("M,N,K", [(17, 40, 128), (33, 100, 192), (64, 12288, 4096), (9, 320, 64), (1, 64, 64),
                                    (65, 411, 320), (128, 1000, 1088), (48, 32000, 256), (100, 8, 4096)])
-def test_linear_rows(M, N, K, tb, kp, ps, rows_shape):
+def test_linear_rows(M, N, K, tb, kp, rows_shape):
     """The product with X shared through LDS and K cut inside the block, in every block shape,
     float32 and bfloat16 results; row counts around the tile and launch edges (16, 64)."""
     o = ops()
-    rows_shape(tb, kp, ps)
+    rows_shape(tb, kp)
     x, w = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2, std=0.2)
     wc = _decode_copy(w.to(DEV))
     want = R.linear(x, w, torch.float64)
@@ -878,7 +878,7 @@ def test_linear_rows_takes_the_norm_and_refuses_what_it_does_not_take(rows_shape
     w = rnd(N, K, dtype=torch.bfloat16, seed=2, std=0.2)
     wc = _decode_copy(w.to(DEV))
     for tb, kp, ps in ((None, None, None), (2, 4, 2), (4, 1, 4)):
-        rows_shape(tb, kp, ps)
+        rows_shape(tb, kp)
         close(o.linear_rows(x_dev, wc, torch.float32), R.linear(x, w, torch.float64), torch.bfloat16,
               scale=0.2 * math.sqrt(K))
     assert not o.rows_fits(rnd(129, K, dtype=torch.bfloat16).to(DEV), wc, "plain")
@@ -891,12 +891,12 @@ def test_linear_rows_takes_the_norm_and_refuses_what_it_does_not_take(rows_shape
         o.linear_rows(rnd(20, K).to(DEV), wc, torch.float32)
 
 
-@pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
+@pytest.mark.parametrize("tb,kp", _ROWS_SHAPES)
 @pytest.mark.parametrize("M,F,K", [(17, 172, 64), (64, 11008, 4096), (40, 50, 192), (64, 203, 320), (33, 8, 1024)])
-def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, ps, rows_shape):
+def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, rows_shape):
     """17 to 64 rows: the product and the SiLU-multiply in one kernel, from the gate|up tiles."""
     o = ops()
-    rows_shape(tb, kp, ps)
+    rows_shape(tb, kp)
     x = rnd(M, K, dtype=torch.bfloat16, seed=1)
     w = rnd(2 * F, K, dtype=torch.bfloat16, seed=2, std=0.2)
     got = o.gate_up_silu(x.to(DEV), _decode_copy(w.to(DEV), "gate_up"))
@@ -913,15 +913,15 @@ def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, ps, rows_shape):
     assert float((got.double().cpu() - want).abs().mean()) <= float((loose.double().cpu() - want).abs().mean()) * 1.05
 
 
-@pytest.mark.parametrize("tb,kp,ps", _ROWS_SHAPES)
+@pytest.mark.parametrize("tb,kp", _ROWS_SHAPES)
 @pytest.mark.parametrize("M,nh,nkv,hd,K", [(17, 4, 2, 32, 64), (64, 32, 32, 128, 4096), (40, 6, 3, 64, 256),
                                            (64, 8, 1, 96, 128), (33, 3, 3, 48, 192), (50, 2, 1, 16, 1024)])
-def test_qkv_rope_store_of_many_rows(M, nh, nkv, hd, K, tb, kp, ps, rows_shape):
+def test_qkv_rope_store_of_many_rows(M, nh, nkv, hd, K, tb, kp, rows_shape):
     """17 to 64 sequences decoding together: the q|k|v product, the rotation and the cache store
     in one kernel against the three steps."""
     from inferllm_amd.parts.position import rotary_table
     o = ops()
-    rows_shape(tb, kp, ps)
+    rows_shape(tb, kp)
     dtype, page = torch.bfloat16, 64
     table = rotary_table(777.0, hd, 300, "cpu")
     x = rnd(M, K, dtype=dtype, seed=1)
