@@ -169,8 +169,8 @@ int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int 
                              const int32_t* page_table, int table_stride, int page_size, int ring,
                              int nh, int nkv, int hd, const float* ssq, int parts, float eps,
                              void* stream);
-// Tuning and tests: tiles a block of these products takes (2, 3, 4) and parts of K (1, 2, 4;
-// four tiles: 1, 2); 0: the library's own choice.
+// Tuning and tests: tiles a block of these products takes (2 to 8) and parts of K (1, 2, 4;
+// four tiles and more: 1, 2); 0: the library's own choice.
 void illm_set_rows_shape(int tb, int kp);
 
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny

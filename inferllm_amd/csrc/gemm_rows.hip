@@ -18,8 +18,13 @@
 // swizzled within a row, two buffers, one barrier a piece).  K is cut inside the block, not over
 // blocks: the parts' sums are added through LDS in part order (a fixed order of summation) and
 // the waves of part 0 finish their tile in registers: a rotation pair, or a gate and its up row,
-// lie 32 lanes apart in the accumulator.  TB and KP are chosen by the host so that the chip has
-// a block or two per compute unit and at least eight waves each.
+// lie 32 lanes apart in the accumulator.
+//
+// What bounds these products at 32 to 64 rows is X, not W: every block reads all of X from the
+// L2 cache, and with few tiles a block that is more bytes than the block's share of W (measured
+// at 64 rows of a 22016 x 4096 gate|up: 45 us with blocks of 3 tiles, 33 us when X comes from
+// the L1 cache instead, 33 us with blocks of 6 tiles).  So the host gives a block as many tiles
+// (2 to 8) as still fill the chip's compute units in whole rounds.
 #include <math.h>
 
 #include "api.h"
@@ -49,10 +54,10 @@ struct GrScale {
     float eps;
 };
 
-// GR_PIECE: k-steps of 32 in a piece.  A block of four tiles has at most two parts of K (eight
-// waves), one of two or three tiles up to four.
+// GR_PIECE: k-steps of 32 in a piece.  A block of four or more tiles has at most two parts of K,
+// one of two or three tiles up to four.
 template <int MT, int TB, int MODE, int GR_PIECE>
-__global__ void __launch_bounds__(64 * TB * (TB == 4 ? 2 : 4))
+__global__ void __launch_bounds__(64 * TB * (TB >= 4 ? 2 : 4))
 gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, void* __restrict__ Y,
                  int y_dt, int M, int N, int K, int tiles, int kp, GrRope rope, GrScale scale) {
     constexpr int UNITS = MT * 16 * GR_PIECE * 4;            // 16-byte units of a part's X piece
@@ -116,7 +121,11 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
     // Loads are unconditional (piece indices clamped; K is a multiple of the piece, so nothing
     // lies beyond it), and every stage of the loop below names its registers statically, so that
     // the compiler's wait counts leave the newer loads in flight while the oldest is used: a wave
-    // has three pieces of W and two of X on their way at any time.
+    // has three pieces of W and two of X on their way at any time.  Loads return in the order of
+    // issue, and the wait count the compiler puts before a stage is the fewer of what the
+    // prologue and what the round before leave behind the load it needs: the prologue therefore
+    // issues its loads in the very order the stages would have (scheduling barriers keep the
+    // compiler from sorting them), or the first stage of every round would wait for all loads.
     const int p_last = (p_end > p_begin ? p_end : pieces) - 1;         // a piece that exists
     const bf16_t* wtile = tile_ok ? wsrc : Wt + (r * 4 + q) * 8;       // no tile: tile 0, dropped
 #define GR_LOAD_X(P, XG)                                                                          \
@@ -156,12 +165,18 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     // (native vector types: arrays of the runtime's uint4 struct are not always kept in registers)
-    illm_u32x4_t xr0[XU], xr1[XU], wr0[GR_PIECE], wr1[GR_PIECE], wr2[GR_PIECE], wr3[GR_PIECE];
-    GR_LOAD_X(p_begin, xr0)
+    illm_u32x4_t xr0[XU], xr1[XU], xr2[XU], xr3[XU];
+    illm_u32x4_t wr0[GR_PIECE], wr1[GR_PIECE], wr2[GR_PIECE], wr3[GR_PIECE];
     GR_LOAD_W(p_begin, wr0)
-    GR_LOAD_X(p_begin + 1, xr1)
+    __builtin_amdgcn_sched_barrier(0);
+    GR_LOAD_X(p_begin, xr0)
+    __builtin_amdgcn_sched_barrier(0);
     GR_LOAD_W(p_begin + 1, wr1)
+    __builtin_amdgcn_sched_barrier(0);
+    GR_LOAD_X(p_begin + 1, xr1)
+    __builtin_amdgcn_sched_barrier(0);
     GR_LOAD_W(p_begin + 2, wr2)
+    __builtin_amdgcn_sched_barrier(0);
     if (finishes) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -175,17 +190,18 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
             e_page[mt] = rope.page_table[(size_t)e_slot[mt] * rope.table_stride + lp];
         }
     }
-    // A stage of a round of four: piece p = p_begin + I.  One barrier a piece is enough with two
+    // A stage of a round of four: piece p = p_begin + I.  It first asks for X two pieces and W
+    // three pieces on, then waits for its own piece of X.  One barrier a piece is enough with two
     // buffers: whoever writes buffer BUF again, two pieces on, has passed the next piece's
     // barrier, which every wave reaches only after it has finished reading this one.
-#define GR_STAGE(I, BUF, XR, WCUR, WNEXT)                                                         \
+#define GR_STAGE(I, BUF, XCUR, XNEXT, WCUR, WNEXT)                                                \
     {                                                                                             \
         const int p = p_begin + (I);                                                              \
-        _Pragma("unroll") for (int j = 0; j < XU; ++j)                                            \
-            ((illm_u32x4_t*)lds)[(BUF) * UNITS + x_dst[j]] = XR[j];                            \
-        __syncthreads();                                                                          \
-        GR_LOAD_X(p + 2, XR)                                                                      \
+        GR_LOAD_X(p + 2, XNEXT)                                                                   \
         GR_LOAD_W(p + 3, WNEXT)                                                                   \
+        _Pragma("unroll") for (int j = 0; j < XU; ++j)                                            \
+            ((illm_u32x4_t*)lds)[(BUF) * UNITS + x_dst[j]] = XCUR[j];                             \
+        __syncthreads();                                                                          \
         if (p < p_end) {                                                                          \
             _Pragma("unroll") for (int u = 0; u < GR_PIECE; ++u)                                  \
                 _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                               \
@@ -198,10 +214,10 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
         }                                                                                         \
     }
     for (int i = 0; i < per; i += 4) {                       // every wave runs the same rounds
-        GR_STAGE(i, 0, xr0, wr0, wr3)
-        GR_STAGE(i + 1, 1, xr1, wr1, wr0)
-        GR_STAGE(i + 2, 0, xr0, wr2, wr1)
-        GR_STAGE(i + 3, 1, xr1, wr3, wr2)
+        GR_STAGE(i, 0, xr0, xr2, wr0, wr3)
+        GR_STAGE(i + 1, 1, xr1, xr3, wr1, wr0)
+        GR_STAGE(i + 2, 0, xr2, xr0, wr2, wr1)
+        GR_STAGE(i + 3, 1, xr3, xr1, wr3, wr2)
     }
 #undef GR_STAGE
 #undef GR_LOAD_X
@@ -306,11 +322,15 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
     }
 }
 
-// Tiles a block takes (2, 3 or 4) and parts of K (1, 2 or 4; a part has at least 4 pieces): a
-// block or two per compute unit, as even as can be, and at least eight waves a compute unit.
+// Tiles a block takes (2 to 8) and parts of K (1, 2 or 4; a part has at least 4 pieces).  The
+// blocks run in rounds of one a compute unit and a block's time grows with its tiles, so the tiles
+// are those with the fewest rounds x tiles, the most tiles among equals (the less of X is read);
+// measured at 16 to 64 rows of the q|k|v, gate|up and head matrices of the 7B, 8B and 70B shapes,
+// where this picks the fastest or one within 3 % of it.  Blocks of up to three tiles cut K in two
+// (six waves at least), larger ones do not.
 static int GR_TB = 0, GR_KP = 0;          // tuning and tests: forced values (0: the choice below)
 extern "C" void illm_set_rows_shape(int tb, int kp) {
-    GR_TB = (tb >= 2 && tb <= 4) ? tb : 0;
+    GR_TB = (tb >= 2 && tb <= 8) ? tb : 0;
     GR_KP = (kp == 1 || kp == 2 || kp == 4) ? kp : 0;
 }
 
@@ -318,32 +338,22 @@ extern "C" void illm_set_rows_shape(int tb, int kp) {
                               // rows and worse at 64)
 
 static void rows_shape(int tiles, int K, int* tb, int* kp) {
-    const int GR_PIECE = GR_PIECE_STEPS;
     const int cus = 256;
-    int best_tb = 4;
-    double best = -1.0;
-    for (int t = 4; t >= 2; --t) {
+    int best_tb = 2;
+    long long best = -1;
+    for (int t = 2; t <= 8; ++t) {
         const int blocks = (tiles + t - 1) / t;
-        // share of the compute units' time that is used if every unit takes its blocks in turn
-        const int rounds = (blocks + cus - 1) / cus;
-        double used = (double)blocks / ((double)rounds * cus);
-        if (blocks >= 2 * cus) used = used > 0.9 ? used : 0.9;     // several blocks a unit even out
-        if (used > best + 0.02) {
-            best = used;
+        const long long cost = (long long)((blocks + cus - 1) / cus) * t;
+        if (best < 0 || cost <= best) {
+            best = cost;
             best_tb = t;
         }
     }
-    const int pieces = (K / 32 + GR_PIECE - 1) / GR_PIECE;
-    const int blocks = (tiles + best_tb - 1) / best_tb;
-    int k = 1;
-    // eight waves a compute unit (blocks * tb * kp >= 8 * cus), within 16 waves a block
-    while (k < 4 && (long long)blocks * best_tb * k < 8LL * cus && best_tb * k * 2 <= 16 &&
-           pieces / (k * 2) >= 4)
-        k *= 2;
     *tb = GR_TB ? GR_TB : best_tb;
-    *kp = GR_KP ? GR_KP : k;
-    if (*tb * *kp > 16) *kp = 16 / *tb >= 4 ? 4 : (16 / *tb >= 2 ? 2 : 1);
-    while (*kp > 1 && pieces < *kp) *kp /= 2;
+    *kp = GR_KP ? GR_KP : (*tb <= 3 ? 2 : 1);
+    if (*tb >= 4 && *kp > 2) *kp = 2;                       // the kernel's launch bounds
+    const int pieces = (K / 32 + GR_PIECE_STEPS - 1) / GR_PIECE_STEPS;
+    while (*kp > 1 && pieces / *kp < 4) *kp /= 2;
 }
 
 template <int MT, int MODE>
@@ -351,7 +361,6 @@ static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int
                        int tiles, const GrRope& rope, const GrScale& scale, hipStream_t st) {
     int tb, kp;
     rows_shape(tiles, K, &tb, &kp);
-    if (tb == 4 && kp > 2) kp = 2;                          // the kernel's launch bounds
     constexpr int ps = GR_PIECE_STEPS;
     const size_t x_bytes = (size_t)kp * 2 * MT * 16 * ps * 4 * 16 + (MT == 1 ? 64 : 0);
     const size_t red_bytes = (size_t)(kp - 1) * tb * MT * 64 * 16;
@@ -360,9 +369,15 @@ static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int
 #define GO(TB_, PS_)                                                                              \
     hipLaunchKernelGGL((gemm_rows_kernel<MT, TB_, MODE, PS_>), grid, block, smem, st, x, wt, y,   \
                        y_dt, rows, N, K, tiles, kp, rope, scale)
-    if (tb == 2) GO(2, GR_PIECE_STEPS);
-    else if (tb == 3) GO(3, GR_PIECE_STEPS);
-    else GO(4, GR_PIECE_STEPS);
+    switch (tb) {
+        case 2: GO(2, GR_PIECE_STEPS); break;
+        case 3: GO(3, GR_PIECE_STEPS); break;
+        case 4: GO(4, GR_PIECE_STEPS); break;
+        case 5: GO(5, GR_PIECE_STEPS); break;
+        case 6: GO(6, GR_PIECE_STEPS); break;
+        case 7: GO(7, GR_PIECE_STEPS); break;
+        default: GO(8, GR_PIECE_STEPS); break;
+    }
 #undef GO
     return illm_launch_status();
 }

@@ -839,7 +839,7 @@ def test_qkv_rope_store_equals_the_three_steps(M, nh, nkv, hd, K, normed, copy, 
 
 # ---------------------------------------------------------------- products of 9 to 128 rows
 # (tiles a block, parts of K)
-_ROWS_SHAPES = [(None, None), (2, 1), (2, 4), (3, 2), (3, 4), (4, 1), (4, 2)]
+_ROWS_SHAPES = [(None, None), (2, 1), (2, 4), (3, 2), (3, 4), (4, 1), (4, 2), (5, 2), (6, 1), (7, 1), (8, 2)]
 
 
 @pytest.fixture
