@@ -77,7 +77,7 @@ int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_s
 
 // Tuning and tests: which prefill attention kernel head sizes up to 128 take: 0 the one with one
 // LDS buffer (which larger head sizes use), 2 the one with two buffers and one barrier a tile
-// (needs a positive scale), 1 (default) the second for head sizes 96 and 128 and sequences of
+// (needs a positive scale), 1 (default) the second for head sizes 64 to 128 and sequences of
 // 1,024 keys or more.
 void illm_set_prefill_two_buffers(int on);
 

@@ -23,6 +23,8 @@
 // grouped heads as src/kern/naive/naive.cpp:576-604.
 #include <math.h>
 
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -255,12 +257,21 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
 
 // The same for head sizes up to 128 with two LDS buffers and one barrier a tile: while a tile is
 // multiplied the next one, already in registers, is written to the other buffer and the one
-// after it is asked for.  K and V^T rows are not padded but swizzled (16-byte units XORed with
-// the row's low bits), so two buffers of both are 512 * HD bytes (64 KB at head size 128, two
-// blocks a compute unit).  V is transposed in registers, 4 keys x 8 dims a thread, and written
-// as 8-byte runs of 4 keys; within a tile of 64 keys the runs are placed in the order in which
-// the first product leaves the scores of a lane (keys 16 m + 4 h + {0..3} and + 8 + {0..3} for
-// half-wave h), so that the A operand of the second product is one 16-byte read.
+// after it is asked for.  It keeps the vector instructions beside the products few: K and V^T
+// rows are padded and the loop is unrolled over the two buffers, so every LDS address is a
+// register fixed for the whole kernel plus an immediate offset; the tile's K and V rows are read
+// at per-thread byte offsets, fixed as well, from a base that moves with the tile (scalar
+// arithmetic), clamped only in a sequence's last tile; V is transposed in registers, 4 keys x 8
+// dims a thread, with one byte permute a pair, and written as 8-byte runs of 4 keys; within a
+// tile of 64 keys the runs are placed in the order in which the first product leaves the scores
+// of a lane (keys 16 m + 4 h + {0..3} and + 8 + {0..3} for half-wave h), so that the A operand of
+// the second product is one 16-byte read.  Two buffers of padded rows are 70 KB at head size 128
+// (two blocks a compute unit fit in its 160 KB).
+template <int B>
+struct PfBuf {
+    static constexpr int v = B;
+};
+
 template <int HD>
 __global__ void __launch_bounds__(256, 2)
 attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
@@ -269,12 +280,12 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
     constexpr int KS = HD / 16;        // k-steps of the first product
     constexpr int DB = HD / 32;        // 32-row blocks of O^T
     constexpr int UK = HD / 8;         // 16-byte units in a K row
-    constexpr int KMASK = (UK % 8 == 0) ? 7 : 3;
-    constexpr int K_TILE = PF_BN * HD;             // elements of a K buffer
-    constexpr int V_TILE = HD * PF_BN;             // elements of a V^T buffer (rows of 64 keys)
+    constexpr int KLD = HD + 8;        // K row stride: 16 bytes of padding
+    constexpr int VLD = PF_BN + 8;     // V^T row stride
+    constexpr int K_TILE = PF_BN * KLD;
+    constexpr int BUF = K_TILE + HD * VLD;         // elements of a buffer: K, then V^T
+    constexpr int NLD = (PF_BN * UK) / 256;        // K units a thread (HD / 32)
     extern __shared__ __attribute__((aligned(16))) bf16_t pf_lds[];
-    bf16_t* ks = pf_lds;                           // [2][64][HD]
-    bf16_t* vts = pf_lds + 2 * K_TILE;             // [2][HD][64]
 
     const int xcd = blockIdx.x % 8, slot_id = blockIdx.x / 8;
     const int hb = xcd * hb_per_xcd + slot_id % hb_per_xcd;
@@ -287,18 +298,23 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
     if (q0 >= len) return;
     const int kvh = h / (nh / nkv);
     const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
+    const uint32_t row_bytes = (uint32_t)(rowlen * 2);
     const int tid = threadIdx.x, wave = wave_index(), lane = tid & 63;
     const int lq = lane & 31, half = lane >> 5;
     const int q_row0 = q0 + wave * 32;
     const int q = q_row0 + lq;
     const int qc = q < len ? q : len - 1;
 
-    uint4 qf[KS];
+    illm_u32x4_t qf[KS];
     {
         const bf16_t* qp = qkv + (size_t)(start + qc) * rowlen + (size_t)h * HD + half * 8;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) qf[s] = *(const uint4*)(qp + s * 16);
+        for (int s = 0; s < KS; ++s) qf[s] = *(const illm_u32x4_t*)(qp + s * 16);
     }
+    // Q is asked for before the first tile and stays there (a scheduling barrier): the wait for
+    // that tile then covers Q, and the loop's products wait for no load.  Asked for later, every
+    // round's first product would wait for the tile after next, which is on its way by then.
+    __builtin_amdgcn_sched_barrier(0);
     f32x16_t o[DB];
 #pragma unroll
     for (int d = 0; d < DB; ++d)
@@ -312,75 +328,73 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
     const int wk_end = min(len, q_row0 + 32);                       // this wave's last key + 1
     const int wk_begin = window > 0 ? max(0, q_row0 - window + 1) : 0;
 
-    // staging.  K: unit u = (key, chunk) as in the kernel above.  V: unit u = (chunk c = u / 16,
-    // key group g = u % 16): keys 4 g .. 4 g + 3, dims 8 c .. 8 c + 7.
-    constexpr int NLD = (PF_BN * HD / 8) / 256;          // K units a thread
-    constexpr int NVU = (2 * HD + 255) / 256;            // V units a thread
-    // (native vector types: arrays of the runtime's uint4 struct are not always kept in registers)
-    illm_u32x4_t kpre[NLD], vpre0[NVU], vpre1[NVU], vpre2[NVU], vpre3[NVU];
+    // Staging.  K: this thread brings chunks chq + 4 it (it < NLD) of key `skey`.  V: keys
+    // 4 g .. 4 g + 3, dims 8 c .. 8 c + 7 (threads with c >= UK, at head sizes below 128, bring
+    // chunk UK - 1 again and write nothing).
+    const int skey = ((tid >> 6) & 3) * 16 + (tid & 15), chq = (tid >> 4) & 3;
+    const int vc = (tid >> 4) < UK ? (tid >> 4) : UK - 1, vg = tid & 15;
+    const bool v_writes = (tid >> 4) < UK;
+    // where the group's 4 keys go in the row of 64, so that the second product's operand, a
+    // lane's 8 keys in the order in which the first product leaves them, is one 16-byte read:
+    // bits (sub, sub, m, a, h) -> (.., h, a)
+    const int vpg = (vg & 12) | ((vg & 1) << 1) | ((vg >> 1) & 1);
+    const char* const kg = (const char*)(qkv + (size_t)start * rowlen + (size_t)(nh + kvh) * HD);
+    const char* const vg_base = (const char*)(qkv + (size_t)start * rowlen + (size_t)(nh + nkv + kvh) * HD);
+    const uint32_t koff_whole = (uint32_t)skey * row_bytes + chq * 16;
+    const uint32_t voff_whole = (uint32_t)(4 * vg) * row_bytes + vc * 16;
+    bf16_t* const kw = pf_lds + skey * KLD + chq * 8;                 // + it * 32
+    bf16_t* const vw = pf_lds + K_TILE + (8 * vc) * VLD + vpg * 4;    // + dim * VLD
+    const bf16_t* const kr = pf_lds + lq * KLD + half * 8;            // + sub * 32 * KLD + st * 16
+    const bf16_t* const vr = pf_lds + K_TILE + lq * VLD + half * 8;   // + d * 32 * VLD + (sub * 4 + mf * 2) * 8
+
+    illm_u32x4_t kpre[NLD], vpre0, vpre1, vpre2, vpre3;
     auto fetch = [&](int k0) __attribute__((always_inline)) {
-#pragma unroll
-        for (int it = 0; it < NLD; ++it) {
-            const int u = tid + it * 256;
-            const int key = ((u >> 6) & 3) * 16 + (u & 15);
-            const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
-            const int krow = min(k0 + key, len - 1);
-            kpre[it] = *(const illm_u32x4_t*)(qkv + (size_t)(start + krow) * rowlen +
-                                              (size_t)(nh + kvh) * HD + ch * 8);
+        uint32_t ko = koff_whole, v0 = voff_whole, v1 = voff_whole + row_bytes,
+                 v2 = voff_whole + 2 * row_bytes, v3 = voff_whole + 3 * row_bytes;
+        if (k0 + PF_BN > len) {                    // the sequence's last tile: rows clamped
+            const int last = len - 1 - k0;
+            ko = (uint32_t)min(skey, last) * row_bytes + chq * 16;
+            v0 = (uint32_t)min(4 * vg + 0, last) * row_bytes + vc * 16;
+            v1 = (uint32_t)min(4 * vg + 1, last) * row_bytes + vc * 16;
+            v2 = (uint32_t)min(4 * vg + 2, last) * row_bytes + vc * 16;
+            v3 = (uint32_t)min(4 * vg + 3, last) * row_bytes + vc * 16;
         }
+        const char* kt = kg + (size_t)k0 * row_bytes;
+        const char* vt = vg_base + (size_t)k0 * row_bytes;
 #pragma unroll
-        for (int it = 0; it < NVU; ++it) {
-            const int u = tid + it * 256;
-            const int c = (u >> 4) < UK ? (u >> 4) : UK - 1, g = u & 15;
-            const bf16_t* vsrc = qkv + (size_t)(nh + nkv + kvh) * HD + c * 8;
-            vpre0[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 0, len - 1)) * rowlen);
-            vpre1[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 1, len - 1)) * rowlen);
-            vpre2[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 2, len - 1)) * rowlen);
-            vpre3[it] = *(const illm_u32x4_t*)(vsrc + (size_t)(start + min(k0 + 4 * g + 3, len - 1)) * rowlen);
-        }
+        for (int it = 0; it < NLD; ++it) kpre[it] = *(const illm_u32x4_t*)(kt + ko + it * 64);
+        vpre0 = *(const illm_u32x4_t*)(vt + v0);
+        vpre1 = *(const illm_u32x4_t*)(vt + v1);
+        vpre2 = *(const illm_u32x4_t*)(vt + v2);
+        vpre3 = *(const illm_u32x4_t*)(vt + v3);
     };
-    auto stage = [&](int buf) __attribute__((always_inline)) {
-        bf16_t* kd = ks + buf * K_TILE;
-        bf16_t* vd = vts + buf * V_TILE;
+    auto stage = [&](auto bc) __attribute__((always_inline)) {
+        constexpr int off = decltype(bc)::v * BUF;
 #pragma unroll
-        for (int it = 0; it < NLD; ++it) {
-            const int u = tid + it * 256;
-            const int key = ((u >> 6) & 3) * 16 + (u & 15);
-            const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
-            *(illm_u32x4_t*)(kd + key * HD + ((ch ^ (key & KMASK)) * 8)) = kpre[it];
-        }
+        for (int it = 0; it < NLD; ++it) *(illm_u32x4_t*)(kw + off + it * 32) = kpre[it];
+        if (v_writes) {
 #pragma unroll
-        for (int it = 0; it < NVU; ++it) {
-            const int u = tid + it * 256;
-            if (NVU * 256 != 2 * HD && u >= 2 * HD) continue;
-            const int c = u >> 4, g = u & 15;
-            // where the group's 4 keys go in the row of 64: bits (sub, sub, m, a, h) -> (.., h, a)
-            const int pg = (g & 12) | ((g & 1) << 1) | ((g >> 1) & 1);
-#pragma unroll
-            for (int dp = 0; dp < 4; ++dp) {                 // dims 2 dp and 2 dp + 1
-                const uint32_t a0 = vpre0[it][dp], a1 = vpre1[it][dp], a2 = vpre2[it][dp], a3 = vpre3[it][dp];
-                const uint2 even = make_uint2((a0 & 0xffffu) | (a1 << 16), (a2 & 0xffffu) | (a3 << 16));
-                const uint2 odd = make_uint2((a0 >> 16) | (a1 & 0xffff0000u), (a2 >> 16) | (a3 & 0xffff0000u));
-                const int d0 = 8 * c + 2 * dp;
-                *(uint2*)(vd + d0 * PF_BN + ((((pg >> 1) ^ (d0 & 7)) * 2 + (pg & 1)) * 4)) = even;
-                *(uint2*)(vd + (d0 + 1) * PF_BN + ((((pg >> 1) ^ ((d0 + 1) & 7)) * 2 + (pg & 1)) * 4)) = odd;
+            for (int dp = 0; dp < 4; ++dp) {                 // dims 2 dp and 2 dp + 1 of the chunk
+                const uint32_t a0 = vpre0[dp], a1 = vpre1[dp], a2 = vpre2[dp], a3 = vpre3[dp];
+                uint2 even, odd;
+                even.x = __builtin_amdgcn_perm(a1, a0, 0x05040100u);
+                even.y = __builtin_amdgcn_perm(a3, a2, 0x05040100u);
+                odd.x = __builtin_amdgcn_perm(a1, a0, 0x07060302u);
+                odd.y = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
+                *(uint2*)(vw + off + (2 * dp) * VLD) = even;
+                *(uint2*)(vw + off + (2 * dp + 1) * VLD) = odd;
             }
         }
     };
-
-    if (k_begin < k_end) {
-        fetch(k_begin);
-        stage(0);
-        if (k_begin + PF_BN < k_end) fetch(k_begin + PF_BN);
-    }
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = k_begin; k0 < k_end; k0 += PF_BN, buf ^= 1) {
+    // One tile of 64 keys at k0 from buffer B; then the next tile, already in registers, goes
+    // into the other buffer and the one after it is asked for.
+    auto tile = [&](auto bc, int k0) __attribute__((always_inline)) {
+        constexpr int B = decltype(bc)::v;
         if (k0 < wk_end && k0 + PF_BN > wk_begin) {                 // something visible to this wave
-            const bf16_t* kb = ks + buf * K_TILE;
-            const bf16_t* vb = vts + buf * V_TILE;
-            // S^T[key][q] for two sub-tiles of 32 keys
-            // (the two sub-tiles' sums alternate, so that no product waits for the one before it)
+            const bf16_t* kb = kr + B * BUF;
+            const bf16_t* vb = vr + B * BUF;
+            // S^T[key][q] for two sub-tiles of 32 keys (their sums alternate, so that no product
+            // waits for the one before it)
             f32x16_t s[2];
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub)
@@ -390,8 +404,7 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
             for (int st = 0; st < KS; ++st)
 #pragma unroll
                 for (int sub = 0; sub < 2; ++sub) {
-                    const int krow = sub * 32 + lq;
-                    const uint4 a = *(const uint4*)(kb + krow * HD + (((st * 2 + half) ^ (krow & KMASK)) * 8));
+                    const illm_u32x4_t a = *(const illm_u32x4_t*)(kb + sub * 32 * KLD + st * 16);
                     s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&a,
                                                                      *(const bf16x8_t*)&qf[st],
                                                                      s[sub], 0, 0, 0);
@@ -415,14 +428,19 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
 #pragma unroll
                     for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[sub][i]);
             }
-            // the running max is kept in scaled units (scale > 0, so the order is the same);
-            // the scale is applied inside the exponential's argument: one multiply-add a score
+            // The reference point of the exponentials (in scaled units: the scale is positive and
+            // is applied inside the exponential's argument, one multiply-add a score) follows the
+            // running max only when that has grown by more than 8, a factor of 256: until then
+            // the weights are at most 256, which float32 sums and bfloat16 weights hold as well
+            // as weights up to 1, and the sums need no rescaling (with random scores some query
+            // of a wave has a new max in most tiles: 64 multiplications a lane).  The division
+            // by the sum of the weights at the end makes the result the same.
             mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE)) * scale_log2;
-            const float m_new = fmaxf(m, mx);
+            const float m_new = (mx > m + 8.0f || m == NEG_INF) ? fmaxf(m, mx) : m;
             const float m_use = (m_new == NEG_INF) ? 0.f : m_new;
             const float alpha = __builtin_amdgcn_exp2f(m - m_use);
             float rs = 0.f;
-            uint4 pb[2][2];
+            illm_u32x4_t pb[2][2];
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub) {
                 float p[16];
@@ -432,16 +450,14 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
                     rs += p[i];
                 }
 #pragma unroll
-                for (int mf = 0; mf < 2; ++mf) {
-                    pb[sub][mf].x = pack_bf16x2(p[8 * mf + 0], p[8 * mf + 1]);
-                    pb[sub][mf].y = pack_bf16x2(p[8 * mf + 2], p[8 * mf + 3]);
-                    pb[sub][mf].z = pack_bf16x2(p[8 * mf + 4], p[8 * mf + 5]);
-                    pb[sub][mf].w = pack_bf16x2(p[8 * mf + 6], p[8 * mf + 7]);
-                }
+                for (int mf = 0; mf < 2; ++mf)
+#pragma unroll
+                    for (int w = 0; w < 4; ++w)
+                        pb[sub][mf][w] = pack_bf16x2(p[8 * mf + 2 * w], p[8 * mf + 2 * w + 1]);
             }
             l = l * alpha + rs;
             m = m_new;
-            if (__any(alpha != 1.f)) {          // the running max moved for some query of the wave
+            if (__any(alpha != 1.f)) {          // the reference moved for some query of the wave
 #pragma unroll
                 for (int d = 0; d < DB; ++d)
 #pragma unroll
@@ -455,21 +471,31 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
                 for (int mf = 0; mf < 2; ++mf)
 #pragma unroll
                     for (int d = 0; d < DB; ++d) {
-                        const int drow = d * 32 + lq;
-                        const uint4 a = *(const uint4*)(vb + drow * PF_BN +
-                                                        (((sub * 4 + mf * 2 + half) ^ (drow & 7)) * 8));
+                        const illm_u32x4_t a =
+                            *(const illm_u32x4_t*)(vb + d * 32 * VLD + (sub * 4 + mf * 2) * 8);
                         o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)&a,
                                                                        *(const bf16x8_t*)&pb[sub][mf],
                                                                        o[d], 0, 0, 0);
                     }
         }
-        // the next tile into the other buffer (last read before the barrier that ended the
-        // previous round), the one after it on its way
         if (k0 + PF_BN < k_end) {
-            stage(buf ^ 1);
+            stage(PfBuf<1 - B>{});
             if (k0 + 2 * PF_BN < k_end) fetch(k0 + 2 * PF_BN);
         }
         __syncthreads();
+    };
+
+    // (k_begin <= q0 < k_end: there is a first tile.  Were this under a condition, the loop's
+    // wait counts would provide for a way in on which Q has not arrived.)
+    fetch(k_begin);
+    __builtin_amdgcn_sched_barrier(0);
+    stage(PfBuf<0>{});
+    if (k_begin + PF_BN < k_end) fetch(k_begin + PF_BN);
+    __syncthreads();
+    for (int k0 = k_begin; k0 < k_end; k0 += 2 * PF_BN) {
+        tile(PfBuf<0>{}, k0);
+        if (k0 + PF_BN >= k_end) break;
+        tile(PfBuf<1>{}, k0 + PF_BN);
     }
     l += __shfl_xor(l, 32, ILLM_WAVE);
     if (q < len) {
@@ -489,9 +515,28 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
 
 // Tuning and tests: 0 sends head sizes up to 128 to the kernel with one LDS buffer always, 2 to the
 // one with two buffers always (the scale must be positive); 1 (default): two buffers for head
-// sizes 96 and 128 and sequences of 1,024 keys or more.
+// sizes 64 to 128 and sequences of 1,024 keys or more.
 static int PF_TWO_BUFFERS = 1;
 extern "C" void illm_set_prefill_two_buffers(int on) { PF_TWO_BUFFERS = on; }
+
+// The two-buffer kernel needs more LDS than a kernel may have without asking: asked for once per
+// device and head size.
+template <int HD>
+static int prefill2_lds_ready(size_t bytes) {
+    static bool ready[64] = {};
+    static std::mutex lock;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ILLM_ERR_LAUNCH;
+    std::lock_guard<std::mutex> hold(lock);
+    if (!ready[dev]) {
+        if (hipFuncSetAttribute((const void*)attn_prefill_mfma2_kernel<HD>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+            return ILLM_ERR_LAUNCH;
+        ready[dev] = true;
+    }
+    return ILLM_OK;
+}
+
 
 template <int HD>
 static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_seqs, int max_len,
@@ -505,11 +550,17 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
     if constexpr (HD <= 128) if (!pg) {
         // measured at 32 heads: head size 128, 2,048 keys 81 -> 76 us, 4,096 keys 236 -> 214; head
         // size 64 and sequences of 512 lose a tenth (a tile more of set-up before the first product)
-        if (PF_TWO_BUFFERS == 2 || (PF_TWO_BUFFERS == 1 && HD >= 96 && max_len >= 1024 && scale > 0.f)) {
-            hipLaunchKernelGGL(attn_prefill_mfma2_kernel<HD>, dim3((unsigned)blocks), dim3(256),
-                               (size_t)512 * HD, st, (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh,
-                               nkv, scale * 1.44269504088896340736f, window, (int)hb_per_xcd,
-                               (int)n_hb, hb_per_xcd * n_qblk <= 64 ? 1 : 0);
+        // measured at 32 heads of size 128: 2,048 keys 81 -> 71 us, 4,096 keys 228 -> 193, 8,192
+        // keys (8 groups) 704 -> 615; size 64, 2,048 keys 46.7 -> 42.7; four sequences of 1,024
+        // 66 -> 64; eight of 512 lose (45 -> 48: a tile more of set-up before the first product)
+        if (PF_TWO_BUFFERS == 2 || (PF_TWO_BUFFERS == 1 && HD >= 64 && max_len >= 1024 && scale > 0.f)) {
+            const size_t lds = (size_t)2 * (PF_BN * (HD + 8) + HD * (PF_BN + 8)) * sizeof(bf16_t);
+            const int rc = prefill2_lds_ready<HD>(lds);
+            if (rc != ILLM_OK) return rc;
+            hipLaunchKernelGGL(attn_prefill_mfma2_kernel<HD>, dim3((unsigned)blocks), dim3(256), lds, st,
+                               (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
+                               scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
+                               hb_per_xcd * n_qblk <= 64 ? 1 : 0);
             return illm_launch_status();
         }
     }
