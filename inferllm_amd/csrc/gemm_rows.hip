@@ -324,8 +324,9 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, vo
 
 // Tiles a block takes (2 to 8) and parts of K (1, 2 or 4; a part has at least 4 pieces).  The
 // blocks run in rounds of one a compute unit and a block's time grows with its tiles, so the tiles
-// are those with the fewest rounds x tiles, the most tiles among equals (the less of X is read);
-// measured at 16 to 64 rows of the q|k|v, gate|up and head matrices of the 7B, 8B and 70B shapes,
+// are those with the fewest rounds x tiles; among equals the most tiles with more than 16 rows
+// (the less of X is read) and the fewest with up to 16 (X is small, more blocks start sooner).
+// Measured at 16 to 64 rows of the q|k|v, gate|up and head matrices of the 7B, 8B and 70B shapes,
 // where this picks the fastest or one within 3 % of it.  Blocks of up to three tiles cut K in two
 // (six waves at least), larger ones do not.
 static int GR_TB = 0, GR_KP = 0;          // tuning and tests: forced values (0: the choice below)
@@ -337,14 +338,14 @@ extern "C" void illm_set_rows_shape(int tb, int kp) {
 #define GR_PIECE_STEPS 2      // k-steps of 32 in a piece (pieces of 128 k measured no better at 16
                               // rows and worse at 64)
 
-static void rows_shape(int tiles, int K, int* tb, int* kp) {
+static void rows_shape(int tiles, int K, int mt, int* tb, int* kp) {
     const int cus = 256;
     int best_tb = 2;
     long long best = -1;
     for (int t = 2; t <= 8; ++t) {
         const int blocks = (tiles + t - 1) / t;
         const long long cost = (long long)((blocks + cus - 1) / cus) * t;
-        if (best < 0 || cost <= best) {
+        if (best < 0 || cost < best || (cost == best && mt > 1)) {
             best = cost;
             best_tb = t;
         }
@@ -360,7 +361,7 @@ template <int MT, int MODE>
 static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int rows, int N, int K,
                        int tiles, const GrRope& rope, const GrScale& scale, hipStream_t st) {
     int tb, kp;
-    rows_shape(tiles, K, &tb, &kp);
+    rows_shape(tiles, K, MT, &tb, &kp);
     constexpr int ps = GR_PIECE_STEPS;
     const size_t x_bytes = (size_t)kp * 2 * MT * 16 * ps * 4 * 16 + (MT == 1 ? 64 : 0);
     const size_t red_bytes = (size_t)(kp - 1) * tb * MT * 64 * 16;

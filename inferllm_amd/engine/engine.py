@@ -108,6 +108,12 @@ class Engine:
                         and ("qkv",) + tuple(w.shape) not in self.plan.rows_from):
                     self.plan.rows_from[("qkv",) + tuple(w.shape)] = ops.measure_rows_from_qkv(
                         w, part.nh, part.nkv, part.hd)
+                # a feed-forward that keeps a fused gate|up matrix likewise
+                w = getattr(part, "w_gate_up", None)
+                if (isinstance(w, ops.Weight) and w.mode == "gate_up" and w.tiled is not None
+                        and w.shape[1] % 64 == 0
+                        and ("gate_up",) + tuple(w.shape) not in self.plan.rows_from):
+                    self.plan.rows_from[("gate_up",) + tuple(w.shape)] = ops.measure_rows_from_gate_up(w)
         limit = self.spec.max_positions
         self.max_seq_len = min(int(max_seq_len), limit) if max_seq_len else limit
         self.max_batch = int(max_batch)

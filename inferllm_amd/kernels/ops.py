@@ -687,9 +687,32 @@ def qkv_rope_store_fits(x, w_qkv, hd: int) -> bool:
     return rows_fits(x, w_qkv, "qkv")
 
 
+def measure_rows_from_gate_up(w_gate_up: "Weight") -> int:
+    """Fewest rows (1, 5, 9, 13 or 17) from which the fused gate|up product of csrc/gemm_rows.hip
+    takes less time than the few-rows one (for the tuner; times both at 16, 12, 8 and 4 rows)."""
+    F2, K = w_gate_up.plain.shape
+    x = torch.zeros((16, K), dtype=torch.bfloat16, device=w_gate_up.plain.device)
+    saved, key = dict(_plan.rows_from), ("gate_up", F2, K)
+
+    def timed(rows: int, threshold: int) -> float:
+        _plan.rows_from[key] = threshold
+        return _cold_time(lambda: gate_up_silu(x[:rows], w_gate_up))
+
+    first = ROWS_FROM
+    try:
+        for rows in (16, 12, 8, 4):
+            if timed(rows, 1) >= 0.97 * timed(rows, ROWS_FROM):
+                break
+            first = rows - 3
+    finally:
+        _plan.rows_from.clear()
+        _plan.rows_from.update(saved)
+    return first
+
+
 def measure_rows_from_qkv(w_qkv: "Weight", nh: int, nkv: int, hd: int) -> int:
-    """Fewest rows (5, 9, 13 or 17) from which the fused q|k|v product of csrc/gemm_rows.hip takes
-    less time than the few-rows one (for the tuner; times both at 16, 12, 8 rows)."""
+    """Fewest rows (1, 5, 9, 13 or 17) from which the fused q|k|v product of csrc/gemm_rows.hip
+    takes less time than the few-rows one (for the tuner; times both at 16, 12, 8 and 4 rows)."""
     N, K = w_qkv.plain.shape
     dev = w_qkv.plain.device
     x = torch.zeros((16, K), dtype=torch.bfloat16, device=dev)
@@ -707,8 +730,8 @@ def measure_rows_from_qkv(w_qkv: "Weight", nh: int, nkv: int, hd: int) -> int:
 
     first = ROWS_FROM
     try:
-        for rows in (16, 12, 8):
-            if timed(rows, 1) >= 0.95 * timed(rows, ROWS_FROM):
+        for rows in (16, 12, 8, 4):
+            if timed(rows, 1) >= 0.97 * timed(rows, ROWS_FROM):
                 break
             first = rows - 3
     finally:

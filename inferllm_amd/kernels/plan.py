@@ -129,9 +129,14 @@ FIXED_CUTS: Dict[tuple, tuple] = {
 # (csrc/gemm_rows.hip) instead of the few-rows kernels, whose waves each read X for themselves.
 # Unlisted shapes: from 17 rows.
 FIXED_ROWS_FROM: Dict[tuple, int] = {
+    # (gate|up: measured alone the shared-X kernel wins from 1 row at these two shapes; in a
+    # whole decode step at 1 and 8 rows, where its operand comes with the norm's sums of squares,
+    # it does not: 318 -> 313 and 2,327 -> 2,322 tokens/s at the 8B shape)
+    ("gate_up", 27648, 5120): 9,
+    ("gate_up", 28672, 4096): 9,   # 12 rows: 42.3 -> 38.1 us, 16 rows: 43.7 -> 37.9
     ("qkv", 6144, 4096): 5,        # 16 rows: 18.2 -> 13.0 us
     ("qkv", 10240, 8192): 5,       # 16 rows: 45.9 -> 30.9 us
-    ("qkv", 12288, 4096): 13,      # 16 rows: 25.0 -> 19.9 us
+    ("qkv", 12288, 4096): 9,       # 16 rows: 25.0 -> 19.9 us
     ("qkv", 15360, 5120): 5,
 }
 

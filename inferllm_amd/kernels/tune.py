@@ -38,7 +38,7 @@ def matrices(engine):
 MARGIN = 0.93       # a table entry must win by 7 %: what is within the clock's noise stays "whole"
 
 
-def tune_config(cfg: dict, max_rows: int, repeats: int, say) -> tuple:
+def tune_config(cfg: dict, max_rows: int, repeats: int, say, rows_only: bool = False) -> tuple:
     import torch
 
     from .. import Engine
@@ -59,7 +59,17 @@ def tune_config(cfg: dict, max_rows: int, repeats: int, say) -> tuple:
                                for _ in range(repeats))
                 rows[key] = votes[len(votes) // 2]
                 say(f"  q|k|v {w.shape[0]} x {w.shape[1]}: shared-X kernel from {rows[key]} rows (runs: {votes})")
+        # a feed-forward that keeps a fused gate|up matrix in its fused kernel's tile order
+        w = getattr(part, "w_gate_up", None)
+        if isinstance(w, ops.Weight) and w.mode == "gate_up" and w.tiled is not None and w.shape[1] % 64 == 0:
+            key = ("gate_up",) + tuple(w.shape)
+            if key not in rows:
+                votes = sorted(ops.measure_rows_from_gate_up(w) for _ in range(repeats))
+                rows[key] = votes[len(votes) // 2]
+                say(f"  gate|up {w.shape[0]} x {w.shape[1]}: shared-X kernel from {rows[key]} rows (runs: {votes})")
     rows = {k: v for k, v in rows.items() if v != ops.ROWS_FROM}
+    if rows_only:
+        return planes, cuts, rows
     for (N, K), w in sorted(matrices(eng).items()):
         plain = ops.plain_weight(w)
         if (isinstance(w, ops.Weight) and w.mode == "plain" and w.tiled is not None and K >= 2 * N
@@ -95,6 +105,8 @@ def main(argv=None) -> int:
     ap.add_argument("configs", nargs="+", help="config.json files")
     ap.add_argument("--max-rows", type=int, default=8192, help="largest step (rows) to plan for")
     ap.add_argument("--repeats", type=int, default=3, help="measurements per entry; the majority wins")
+    ap.add_argument("--rows-only", action="store_true",
+                    help="measure FIXED_ROWS_FROM only (the fused q|k|v and gate|up products)")
     args = ap.parse_args(argv)
     say = lambda m: print(m, file=sys.stderr, flush=True)
     planes, cuts, rows = {}, {}, {}
@@ -102,7 +114,7 @@ def main(argv=None) -> int:
         with open(path, "r", encoding="utf-8") as f:
             cfg = json.load(f)
         say(f"{path}:")
-        p, c, r = tune_config(cfg, args.max_rows, args.repeats, say)
+        p, c, r = tune_config(cfg, args.max_rows, args.repeats, say, args.rows_only)
         planes.update(p)
         cuts.update(c)
         rows.update(r)
