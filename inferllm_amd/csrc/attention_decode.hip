@@ -29,6 +29,13 @@ __device__ __forceinline__ float fexp(float x) {
     return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
 
+__device__ __forceinline__ void unpack8(const illm_u32x4_t& v, float* f) {
+    f[0] = __uint_as_float(v[0] << 16); f[1] = __uint_as_float(v[0] & 0xffff0000u);
+    f[2] = __uint_as_float(v[1] << 16); f[3] = __uint_as_float(v[1] & 0xffff0000u);
+    f[4] = __uint_as_float(v[2] << 16); f[5] = __uint_as_float(v[2] & 0xffff0000u);
+    f[6] = __uint_as_float(v[3] << 16); f[7] = __uint_as_float(v[3] & 0xffff0000u);
+}
+
 __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
     f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
     f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
@@ -88,6 +95,11 @@ __device__ __forceinline__ void combine_block(const float* lds, int row_heads, i
     }
 }
 
+template <bool B>
+struct DecMore {
+    static constexpr bool value = B;
+};
+
 // LPR: lanes per key row (power of two, 8 dims each, LPR * 8 >= head_dim).
 // GC: query heads handled together (power of two >= heads per kv head, at most 8).
 template <int LPR, int GC>
@@ -136,26 +148,58 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
     const int t_lo = t_first + sp * per;
     const int t_hi = min(t_first + n_tiles, t_lo + per);
 
-    for (int t = t_lo + wave; t < t_hi; t += waves) {
+    // Where tile t of the sequence begins in the cache, for this lane: row q of the tile, dims
+    // 8 c .. 8 c + 7 (a lane beyond the head's dims reads the last 8 again; its values are never
+    // used).  A tile of TK keys lies within a page.
+    const int c_read = dim_ok ? c : 0;
+    auto tile_base = [&](int t) __attribute__((always_inline)) {
         const int k0 = t * TK;
         int lp = k0 / page_size;
         if (ring > 0) lp %= ring;
         const int phys = page_table[(size_t)slot * table_stride + lp];
-        const size_t base = (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)hd +
-                            (size_t)q * hd + c * 8;
-        // rows beyond the sequence's length are not read (the last tile of a sequence is half
-        // empty on average: 5 % of the bytes at 640 keys)
-        uint4 kreg[NI], vreg[NI];
+        return (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)hd;
+    };
+    // The loads of a tile are unconditional, so that the wait counts are exact and a tile's loads
+    // stay in flight beside the arithmetic of the one before.  A load instruction whose rows all
+    // lie beyond the sequence's length reads the rows of the last one that has a row again
+    // (lines that are read anyway: no more bytes from memory; the choice is the same for the
+    // whole wave, a scalar offset).  Rows beyond the length that a load does bring may hold anything: their
+    // scores and values are replaced before use.
+    illm_u32x4_t kreg[NI], vreg[NI];
+    auto load_tile = [&](const bf16_t* __restrict__ cache, size_t base, int k0,
+                         illm_u32x4_t (&reg)[NI]) __attribute__((always_inline)) {
+        const bf16_t* src = cache + base + (size_t)q * hd + c_read * 8;
+        const int r_max = ((len - k0 - 1) / KPI) * KPI;   // first row of the last instruction with a row that exists
 #pragma unroll
-        for (int j = 0; j < NI; ++j)
-            kreg[j] = (dim_ok && k0 + j * KPI + q < len)
-                          ? ld16_stream(kcache + base + (size_t)j * KPI * hd)
-                          : make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-            vreg[j] = (dim_ok && k0 + j * KPI + q < len)
-                          ? ld16_stream(vcache + base + (size_t)j * KPI * hd)
-                          : make_uint4(0, 0, 0, 0);
+        for (int j = 0; j < NI; ++j) {
+            const int r = min(j * KPI, r_max);            // (scalar arithmetic)
+            reg[j] = __builtin_nontemporal_load((const illm_u32x4_t*)(src + (size_t)r * hd));
+        }
+    };
+    // K of the next tile is asked for as soon as the scores have used this tile's K, V of the
+    // next tile as soon as the sums have used this tile's V: each load has half a tile's
+    // arithmetic to arrive in, and a wave holds one tile's registers.  The wave's last tile is a
+    // copy of the loop's body that asks for nothing.
+    // (With several heads a wave the registers do not hold that: the tile's loads are all asked
+    // for at its beginning and used as they arrive.)
+    constexpr bool AHEAD = GC == 1;
+    const int t_begin = t_lo + wave;
+    if (AHEAD && t_begin < t_hi) {
+        const size_t base = tile_base(t_begin);
+        load_tile(kcache, base, t_begin * TK, kreg);
+        load_tile(vcache, base, t_begin * TK, vreg);
+    }
+    auto one_tile = [&](auto more, int t) __attribute__((always_inline)) {
+        constexpr bool MORE = AHEAD && decltype(more)::value;
+        const int k0 = t * TK;
+        const int t_next = t + waves;
+        size_t base_next = 0;
+        if constexpr (MORE) base_next = tile_base(t_next);
+        if constexpr (!AHEAD) {
+            const size_t base = tile_base(t);
+            load_tile(kcache, base, k0, kreg);
+            load_tile(vcache, base, k0, vreg);
+        }
 
         // scores: lane (q, c) ends up owning key k0 + c * KPI + q (if c < NI).  Every lane has a
         // share of NI dot products; instead of NI full reductions over the LPR lanes of a row,
@@ -191,6 +235,10 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
             }
             s_own[g] = part[0] * scale;
         }
+        // (scheduling barriers: the compiler would move these loads down to the others)
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MORE) load_tile(kcache, base_next, t_next * TK, kreg);
+        __builtin_amdgcn_sched_barrier(0);
         const int key_own = k0 + c * KPI + q;
         const bool own_ok = (c < NI) && key_own < len && key_own >= kf;
         float p_own[GC];
@@ -220,6 +268,14 @@ attn_decode_bf16_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out
                 for (int i = 0; i < 8; ++i) acc[g][i] = fmaf(pj, ok ? vf8[i] : 0.f, acc[g][i]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MORE) load_tile(vcache, base_next, t_next * TK, vreg);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    if (t_begin < t_hi) {
+        int t = t_begin;
+        for (; t + waves < t_hi; t += waves) one_tile(DecMore<true>{}, t);
+        one_tile(DecMore<false>{}, t);
     }
     // add the row groups' shares
 #pragma unroll
