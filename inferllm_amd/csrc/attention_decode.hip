@@ -622,43 +622,59 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
     const int t_lo = t_first + sp * per;
     const int t_hi = min(t_first + n_tiles, t_lo + per);
 
-    for (int t = t_lo + wave; t < t_hi; t += waves) {
+    // Where tile t of the sequence begins in the cache (a tile of 64 keys lies within a page).
+    auto tile_base = [&](int t) __attribute__((always_inline)) {
         const int k0 = t * TK;
         int lp = k0 / page_size;
         if (ring > 0) lp %= ring;
         const int phys = page_table[(size_t)slot * table_stride + lp];
-        const size_t tile = (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)HD;
-        // rows beyond the sequence's length are not read
-        uint4 ka[4][KS], vr[2][8];
+        return (((size_t)phys * nkv + kvh) * page_size + (k0 % page_size)) * (size_t)HD;
+    };
+    // The loads of a tile are unconditional (exact wait counts: a tile's loads stay in flight
+    // beside the arithmetic of the one before).  A load instruction brings 16 rows of one
+    // sub-tile; one whose sub-tile lies wholly beyond the sequence's length reads the last
+    // sub-tile that has a row again (lines that are read anyway; a scalar offset).  Rows beyond
+    // the length that a load does bring may hold anything: their scores are replaced and their
+    // values set to zero before use.
+    illm_u32x4_t ka[4][KS], vr[2][8];
+    const int r_read = dim_ok ? r : 0;         // (a lane beyond the head's dims: values never used)
+    auto load_k = [&](size_t tile, int k0) __attribute__((always_inline)) {
+        const int sub_max = (len - k0 - 1) / 16;
 #pragma unroll
-        for (int sub = 0; sub < 4; ++sub)
+        for (int sub = 0; sub < 4; ++sub) {
+            const int sb = min(sub, sub_max);
 #pragma unroll
             for (int s = 0; s < KS; ++s)
-                ka[sub][s] = k0 + sub * 16 + r < len
-                                 ? *(const uint4*)(kcache + tile + (size_t)(sub * 16 + r) * HD + s * 32 + q4 * 8)
-                                 : make_uint4(0, 0, 0, 0);
-        // V: slot i of half hb is key (2 hb + i / 4) * 16 + 4 q4 + i % 4, the key whose score this
-        // k group's lanes get at place i % 4 of sub-tile 2 hb + i / 4
+                ka[sub][s] = *(const illm_u32x4_t*)(kcache + tile + (size_t)(sb * 16 + r) * HD + s * 32 + q4 * 8);
+        }
+    };
+    // V: slot i of half hb is key (2 hb + i / 4) * 16 + 4 q4 + i % 4, the key whose score this
+    // k group's lanes get at place i % 4 of sub-tile 2 hb + i / 4
+    auto load_v = [&](size_t tile, int k0) __attribute__((always_inline)) {
+        const int sub_max = (len - k0 - 1) / 16;
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int kt = (2 * hb + i / 4) * 16 + 4 * q4 + (i & 3);
-                vr[hb][i] = (dim_ok && k0 + kt < len)
-                                ? *(const uint4*)(vcache + tile + (size_t)kt * HD + r * 8)
-                                : make_uint4(0, 0, 0, 0);
+                const int sb = min(2 * hb + i / 4, sub_max);
+                vr[hb][i] = *(const illm_u32x4_t*)(vcache + tile + (size_t)(sb * 16 + 4 * q4 + (i & 3)) * HD + r_read * 8);
             }
-        if (k0 < kf) {
-            // a tile with keys before the window: their rows may hold anything (NaN too), and a
-            // probability of zero would not undo that (rows beyond the length were not read)
-#pragma unroll
-            for (int hb = 0; hb < 2; ++hb)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int key = k0 + (2 * hb + i / 4) * 16 + 4 * q4 + (i & 3);
-                    if (key < kf) vr[hb][i] = make_uint4(0, 0, 0, 0);
-                }
-        }
+    };
+    // K of the next tile is asked for as soon as the scores have used this tile's K, V of the
+    // next tile as soon as the sums have used this tile's V; the wave's last tile is a copy of
+    // the loop's body that asks for nothing.
+    const int t_begin = t_lo + wave;
+    if (t_begin < t_hi) {
+        const size_t tile = tile_base(t_begin);
+        load_k(tile, t_begin * TK);
+        load_v(tile, t_begin * TK);
+    }
+    auto one_tile = [&](auto more, int t) __attribute__((always_inline)) {
+        constexpr bool MORE = decltype(more)::value;
+        const int k0 = t * TK;
+        const int t_next = t + waves;
+        size_t tile_next = 0;
+        if constexpr (MORE) tile_next = tile_base(t_next);
         // scores of 4 keys per sub-tile for head r
         float sv[4][4];
         float mx = NEG_INF;
@@ -677,6 +693,10 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
                 mx = fmaxf(mx, sv[sub][i]);
             }
         }
+        // (scheduling barriers: the compiler would move these loads down to the others)
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MORE) load_k(tile_next, t_next * TK);
+        __builtin_amdgcn_sched_barrier(0);
         mx = fmaxf(mx, __shfl_xor(mx, 16, ILLM_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, ILLM_WAVE));
         const float m_new = fmaxf(m, mx);
@@ -707,6 +727,17 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e][i] *= ai;
         }
+        if (k0 < kf || k0 + TK > len) {
+            // a tile with keys before the window or beyond the length: their rows may hold
+            // anything (NaN too), and a probability of zero would not undo that
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int key = k0 + (2 * hb + i / 4) * 16 + 4 * q4 + (i & 3);
+                    if (key < kf || key >= len) vr[hb][i] = (illm_u32x4_t){0u, 0u, 0u, 0u};
+                }
+        }
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
 #pragma unroll
@@ -726,6 +757,14 @@ attn_decode_bf16_gqa_pv_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restric
                                                                *(const dbf16x8_t*)&tr, o[e], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MORE) load_v(tile_next, t_next * TK);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    if (t_begin < t_hi) {
+        int t = t_begin;
+        for (; t + waves < t_hi; t += waves) one_tile(DecMore<true>{}, t);
+        one_tile(DecMore<false>{}, t);
     }
     // this lane's heads 4 q4 + i: their max and sum from the lanes that hold them
     float lh[4], mh[4];
