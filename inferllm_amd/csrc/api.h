@@ -194,7 +194,7 @@ int illm_qkv_rope_store_skinny(const void* X, const void* W, const void* Wt, voi
 int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream);
 
 // Temperature / top-k / top-p / repeat-penalty sampling, one draw per row.
-// scratch: float32 [B][V].  last_tokens: [B][n_last] (-1 = empty) or null.
+// scratch: float32 [2][B][V].  last_tokens: [B][n_last] (-1 = empty) or null.
 // counters[b]: index of the draw in the request's stream; seeds[b]: the request's seed.
 int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V, float temp,
                 int top_k, float top_p, float repeat_penalty, const int32_t* last_tokens,

@@ -104,154 +104,6 @@ extern "C" int illm_argmax(const float* logits, int32_t* out, int B, int V, void
     return illm_launch_status();
 }
 
-// ---------------------------------------------------------------- sampler
-struct Keep {  // an id is kept iff key > t, or key == t and id <= cut
-    uint32_t t;
-    int cut;
-};
-
-__device__ __forceinline__ bool kept(const Keep& k, uint32_t key, int id) {
-    return key > k.t || (key == k.t && id <= k.cut);
-}
-
-// id of the r-th (1-based) kept id whose key equals k.t, in ascending id order
-__device__ int nth_equal_id(const float* s, int lo, int hi, const Keep& k, int r, int* red_i,
-                            int* shared_out) {
-    int mine = 0;
-    for (int i = lo; i < hi; ++i) mine += (order_key(s[i]) == k.t && i <= k.cut) ? 1 : 0;
-    int total;
-    const int before = block_exclusive_scan<int>(mine, red_i, &total);
-    __syncthreads();
-    if (threadIdx.x == 0) *shared_out = k.cut;
-    __syncthreads();
-    if (r > before && r <= before + mine) {
-        int c = before;
-        for (int i = lo; i < hi; ++i)
-            if (order_key(s[i]) == k.t && i <= k.cut && ++c == r) { *shared_out = i; break; }
-    }
-    __syncthreads();
-    return *shared_out;
-}
-
-__global__ void __launch_bounds__(SB)
-sample_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
-              int32_t* __restrict__ out, int V, float temp, int top_k, float top_p,
-              float repeat_penalty, const int32_t* __restrict__ last_tokens, int n_last,
-              const uint64_t* __restrict__ seeds, const int32_t* __restrict__ counters) {
-    __shared__ float red_f[SB / ILLM_WAVE];
-    __shared__ int red_i[SB / ILLM_WAVE];
-    __shared__ int last[256];
-    __shared__ int sh_i;
-    const int b = blockIdx.x, tid = threadIdx.x;
-    const float* row = logits + (size_t)b * V;
-    float* s = scratch + (size_t)b * V;
-    const int chunk = (V + SB - 1) / SB;
-    const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
-    const int nl = last_tokens ? min(n_last, 256) : 0;
-    if (tid < nl) last[tid] = last_tokens[(size_t)b * n_last + tid];
-    __syncthreads();
-
-    // 1. scaled and penalised scores; their max
-    const float inv_temp = 1.0f / temp;
-    float mx = -INFINITY;
-    for (int i = lo; i < hi; ++i) {
-        float l = row[i];
-        bool rep = false;
-        for (int j = 0; j < nl; ++j) rep |= (last[j] == i);
-        float v = l * inv_temp;
-        if (rep) v = l < 0.f ? v * repeat_penalty : v / repeat_penalty;
-        s[i] = v;
-        mx = fmaxf(mx, v);
-    }
-    mx = block_max(mx, red_f);
-
-    // 2. top_k: largest t with count(key >= t) >= k
-    Keep keep = {0u, V};
-    if (top_k > 0 && top_k < V) {
-        uint32_t t = 0;
-        for (int bit = 31; bit >= 0; --bit) {
-            const uint32_t cand = t | (1u << bit);
-            int c = 0;
-            for (int i = lo; i < hi; ++i) c += order_key(s[i]) >= cand ? 1 : 0;
-            if (block_sum_t<int>(c, red_i) >= top_k) t = cand;
-        }
-        int c = 0;
-        for (int i = lo; i < hi; ++i) c += order_key(s[i]) > t ? 1 : 0;
-        const int above = block_sum_t<int>(c, red_i);
-        keep.t = t;
-        keep.cut = nth_equal_id(s, lo, hi, keep, top_k - above, red_i, &sh_i);
-    }
-
-    // 3. top_p over the kept ids, in descending order of score
-    if (top_p < 1.0f) {
-        float z = 0.f;
-        for (int i = lo; i < hi; ++i)
-            if (kept(keep, order_key(s[i]), i)) z += expf(s[i] - mx);
-        z = block_sum_t<float>(z, red_f);
-        const float need = top_p * z;
-        uint32_t t = 0;  // every threshold up to keep.t holds the whole kept mass
-        for (int bit = 31; bit >= 0; --bit) {
-            const uint32_t cand = t | (1u << bit);
-            float mass = 0.f;
-            for (int i = lo; i < hi; ++i) {
-                const uint32_t key = order_key(s[i]);
-                if (key >= cand && kept(keep, key, i)) mass += expf(s[i] - mx);
-            }
-            if (block_sum_t<float>(mass, red_f) >= need) t = cand;
-        }
-        // t is now the largest threshold whose kept mass still reaches top_p
-        float mass = 0.f, eq_p = 0.f;
-        int eq = 0;
-        for (int i = lo; i < hi; ++i) {
-            const uint32_t key = order_key(s[i]);
-            if (!kept(keep, key, i)) continue;
-            if (key > t) mass += expf(s[i] - mx);
-            else if (key == t) { eq += 1; eq_p = expf(s[i] - mx); }
-        }
-        const float above = block_sum_t<float>(mass, red_f);
-        const int n_eq = block_sum_t<int>(eq, red_i);
-        const float one = block_max(eq_p, red_f);
-        int m = one > 0.f ? (int)ceilf((need - above) / one) : n_eq;
-        m = max(1, min(m, n_eq));
-        Keep k2 = {t, keep.t == t ? keep.cut : V};
-        k2.cut = nth_equal_id(s, lo, hi, k2, m, red_i, &sh_i);
-        keep = k2;
-    }
-
-    // 4. inverse CDF over the kept ids in ascending id order
-    float mine = 0.f;
-    for (int i = lo; i < hi; ++i)
-        if (kept(keep, order_key(s[i]), i)) mine += expf(s[i] - mx);
-    float total;
-    const float before = block_exclusive_scan<float>(mine, red_f, &total);
-    const float u = uniform_from(seeds[b], counters[b]);
-    const float target = u * total;
-    __syncthreads();
-    if (tid == 0) sh_i = -1;
-    __syncthreads();
-    if (mine > 0.f && target >= before && target < before + mine) {
-        float c = before;
-        int pick = -1;
-        for (int i = lo; i < hi; ++i) {
-            if (!kept(keep, order_key(s[i]), i)) continue;
-            pick = i;
-            c += expf(s[i] - mx);
-            if (target < c) break;
-        }
-        atomicMax(&sh_i, pick);
-    }
-    __syncthreads();
-    if (sh_i < 0) {
-        // rounding put the target past the last kept id: take that id
-        int lastk = -1;
-        for (int i = lo; i < hi; ++i)
-            if (kept(keep, order_key(s[i]), i)) lastk = i;
-        atomicMax(&sh_i, lastk);
-        __syncthreads();
-    }
-    if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
-}
-
 // Walks of a row by one block wait for each load in turn unless several are asked for at once:
 // these bring eight values at a time, all loads issued before the first is used.
 template <typename F>
@@ -281,6 +133,246 @@ __device__ __forceinline__ void each_in_order8(const float* a, int lo, int hi, F
         for (int u = 0; u < 8; ++u)
             if (base + u < hi) f(base + u, v[u]);
     }
+}
+
+// ---------------------------------------------------------------- sampler
+struct Keep {  // an id is kept iff key > t, or key == t and id <= cut
+    uint32_t t;
+    int cut;
+};
+
+__device__ __forceinline__ bool kept(const Keep& k, uint32_t key, int id) {
+    return key > k.t || (key == k.t && id <= k.cut);
+}
+
+// id of the r-th (1-based) kept id whose key equals k.t, in ascending id order
+__device__ int nth_equal_id(const float* s, int lo, int hi, const Keep& k, int r, int* red_i,
+                            int* shared_out) {
+    int mine = 0;
+    for (int i = lo; i < hi; ++i) mine += (order_key(s[i]) == k.t && i <= k.cut) ? 1 : 0;
+    int total;
+    const int before = block_exclusive_scan<int>(mine, red_i, &total);
+    __syncthreads();
+    if (threadIdx.x == 0) *shared_out = k.cut;
+    __syncthreads();
+    if (r > before && r <= before + mine) {
+        int c = before;
+        for (int i = lo; i < hi; ++i)
+            if (order_key(s[i]) == k.t && i <= k.cut && ++c == r) { *shared_out = i; break; }
+    }
+    __syncthreads();
+    return *shared_out;
+}
+
+// Every pass over the row is coalesced (thread t takes ids t, t + SB, ...; eight loads asked for
+// before the first is used), the probabilities exp(s - max) are computed once into the second
+// half of the scratch, and only the steps that need the ids in order (the tie at a cut, the
+// inverse CDF) walk a thread's own contiguous chunk.  A row of up to 32 ids a thread stays in
+// registers for the two bisections (IN_REGS); a longer one finds the top_p threshold 8 bits a
+// pass from the mass per digit instead of 32 walks.  Measured with top_p alone: 32,000 ids
+// 557 -> 104 us (every pass in chunks and the exponentials recomputed in each, before), 128,256
+// ids and 16 rows 2,190 -> 400 us.
+constexpr int SAMPLE_REG_IDS = 32;      // ids a thread keeps in registers (IN_REGS: V <= 32 * SB)
+
+template <bool IN_REGS>
+__global__ void __launch_bounds__(SB)
+sample_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
+              int32_t* __restrict__ out, int V, float temp, int top_k, float top_p,
+              float repeat_penalty, const int32_t* __restrict__ last_tokens, int n_last,
+              const uint64_t* __restrict__ seeds, const int32_t* __restrict__ counters) {
+    __shared__ float red_f[SB / ILLM_WAVE];
+    __shared__ int red_i[SB / ILLM_WAVE];
+    __shared__ int last[256];
+    __shared__ int sh_i;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const float* row = logits + (size_t)b * V;
+    float* s = scratch + (size_t)b * V;                       // scaled, penalised scores
+    float* pr = scratch + ((size_t)gridDim.x + b) * V;        // exp(s - max)
+    const int chunk = (V + SB - 1) / SB;
+    const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
+    const int nl = last_tokens ? min(n_last, 256) : 0;
+    if (tid < nl) last[tid] = last_tokens[(size_t)b * n_last + tid];
+    __syncthreads();
+
+    // 1. scaled and penalised scores; their max; the probabilities up to their sum
+    const float inv_temp = 1.0f / temp;
+    float mx = -INFINITY;
+    each_strided8(row, V, tid, [&](int i, float l) {
+        bool rep = false;
+        for (int j = 0; j < nl; ++j) rep |= (last[j] == i);
+        float v = l * inv_temp;
+        if (rep) v = l < 0.f ? v * repeat_penalty : v / repeat_penalty;
+        s[i] = v;
+        mx = fmaxf(mx, v);
+    });
+    mx = block_max(mx, red_f);
+    // (a thread reads back what it wrote itself: the same ids)
+    each_strided8(s, V, tid, [&](int i, float v) { pr[i] = expf(v - mx); });
+    __syncthreads();                                          // the chunked walks read others' values
+
+    // The passes below walk the row's (id, key, probability): from registers, or from the
+    // scratch again (a pass of 32,000 ids then waits for the cache four times over, 8 us).
+    constexpr int RV = SAMPLE_REG_IDS;
+    constexpr bool in_regs = IN_REGS;
+    uint32_t rkey[RV];
+    float rp[RV];
+    if constexpr (in_regs) {
+#pragma unroll
+        for (int u = 0; u < RV; ++u) {
+            const int i = tid + u * SB;
+            rkey[u] = i < V ? order_key(s[i]) : 0u;
+            rp[u] = i < V ? pr[i] : 0.f;
+        }
+    }
+    auto walk = [&](auto f) __attribute__((always_inline)) {
+        if constexpr (in_regs) {
+#pragma unroll
+            for (int u = 0; u < RV; ++u)
+                if (tid + u * SB < V) f(tid + u * SB, rkey[u], rp[u]);
+        } else {
+            each_strided8(s, V, tid, [&](int i, float v) { f(i, order_key(v), pr[i]); });
+        }
+    };
+
+    // 2. top_k: largest t with count(key >= t) >= k
+    Keep keep = {0u, V};
+    if (top_k > 0 && top_k < V) {
+        uint32_t t = 0;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = t | (1u << bit);
+            int c = 0;
+            walk([&](int, uint32_t key, float) { c += key >= cand ? 1 : 0; });
+            if (block_sum_t<int>(c, red_i) >= top_k) t = cand;
+        }
+        int c = 0;
+        walk([&](int, uint32_t key, float) { c += key > t ? 1 : 0; });
+        const int above = block_sum_t<int>(c, red_i);
+        keep.t = t;
+        keep.cut = nth_equal_id(s, lo, hi, keep, top_k - above, red_i, &sh_i);
+    }
+
+    // 3. top_p over the kept ids, in descending order of score
+    if (top_p < 1.0f) {
+        float z = 0.f;
+        walk([&](int i, uint32_t key, float p) {
+            if (kept(keep, key, i)) z += p;
+        });
+        z = block_sum_t<float>(z, red_f);
+        const float need = top_p * z;
+        uint32_t t = 0;  // every threshold up to keep.t holds the whole kept mass
+        if constexpr (in_regs) {
+            for (int bit = 31; bit >= 0; --bit) {
+                const uint32_t cand = t | (1u << bit);
+                float mass = 0.f;
+                walk([&](int i, uint32_t key, float p) {
+                    if (key >= cand && kept(keep, key, i)) mass += p;
+                });
+                if (block_sum_t<float>(mass, red_f) >= need) t = cand;
+            }
+        } else {
+            // A longer row is not walked 32 times: the threshold's key comes 8 bits a pass from
+            // the mass per digit, held as integers (p * 2^40, so that the order in which the
+            // waves add them does not matter; 2^17 ids of at most 2^40 stay below 2^63).
+            constexpr int NW = SB / ILLM_WAVE;
+            __shared__ unsigned long long mhist[NW][256];
+            __shared__ unsigned long long sh_total, sh_above;
+            __shared__ int sh_digit;
+            const int wave = tid / ILLM_WAVE;
+            auto fixed = [](float p) { return (unsigned long long)(p * 1099511627776.0f); };
+            unsigned long long mine_fx = 0;
+            walk([&](int i, uint32_t key, float p) {
+                if (kept(keep, key, i)) mine_fx += fixed(p);
+            });
+            if (tid == 0) sh_total = 0;
+            __syncthreads();
+            atomicAdd(&sh_total, mine_fx);
+            __syncthreads();
+            unsigned long long need_fx = (unsigned long long)((double)top_p * (double)sh_total);
+            need_fx = need_fx > 0 ? need_fx : 1;
+            unsigned long long above_fx = 0;         // mass of the keys above the prefix so far
+            for (int pass = 0; pass < 4; ++pass) {
+                const int shift = 24 - 8 * pass;
+                const uint32_t hi_mask = pass ? (0xffffffffu << (shift + 8)) : 0u;
+                for (int i = tid; i < NW * 256; i += SB) (&mhist[0][0])[i] = 0;
+                __syncthreads();
+                walk([&](int i, uint32_t key, float p) {
+                    if ((key & hi_mask) == t && kept(keep, key, i))
+                        atomicAdd(&mhist[wave][(key >> shift) & 255u], fixed(p));
+                });
+                __syncthreads();
+                if (tid < 256) {
+                    unsigned long long m = 0;
+                    for (int w = 0; w < NW; ++w) m += mhist[w][tid];
+                    mhist[0][tid] = m;
+                }
+                if (tid == 0) sh_digit = 0;
+                __syncthreads();
+                if (tid < 256) {
+                    // the largest digit at which the mass from the top reaches what is needed
+                    unsigned long long over = above_fx;
+                    for (int d = tid + 1; d < 256; ++d) over += mhist[0][d];
+                    if (over < need_fx && over + mhist[0][tid] >= need_fx) {
+                        sh_digit = tid;
+                        sh_above = over;
+                    }
+                }
+                __syncthreads();
+                t |= (uint32_t)sh_digit << shift;
+                above_fx = sh_above;
+                __syncthreads();
+            }
+        }
+        // t is now the largest threshold whose kept mass still reaches top_p
+        float mass = 0.f, eq_p = 0.f;
+        int eq = 0;
+        walk([&](int i, uint32_t key, float p) {
+            if (!kept(keep, key, i)) return;
+            if (key > t) mass += p;
+            else if (key == t) { eq += 1; eq_p = p; }
+        });
+        const float above = block_sum_t<float>(mass, red_f);
+        const int n_eq = block_sum_t<int>(eq, red_i);
+        const float one = block_max(eq_p, red_f);
+        int m = one > 0.f ? (int)ceilf((need - above) / one) : n_eq;
+        m = max(1, min(m, n_eq));
+        Keep k2 = {t, keep.t == t ? keep.cut : V};
+        k2.cut = nth_equal_id(s, lo, hi, k2, m, red_i, &sh_i);
+        keep = k2;
+    }
+
+    // 4. inverse CDF over the kept ids in ascending id order
+    float mine = 0.f;
+    each_in_order8(s, lo, hi, [&](int i, float v) {
+        if (kept(keep, order_key(v), i)) mine += pr[i];
+    });
+    float total;
+    const float before = block_exclusive_scan<float>(mine, red_f, &total);
+    const float u = uniform_from(seeds[b], counters[b]);
+    const float target = u * total;
+    __syncthreads();
+    if (tid == 0) sh_i = -1;
+    __syncthreads();
+    if (mine > 0.f && target >= before && target < before + mine) {
+        float c = before;
+        int pick = -1;
+        for (int i = lo; i < hi; ++i) {
+            if (!kept(keep, order_key(s[i]), i)) continue;
+            pick = i;
+            c += pr[i];
+            if (target < c) break;
+        }
+        atomicMax(&sh_i, pick);
+    }
+    __syncthreads();
+    if (sh_i < 0) {
+        // rounding put the target past the last kept id: take that id
+        int lastk = -1;
+        for (int i = lo; i < hi; ++i)
+            if (kept(keep, order_key(s[i]), i)) lastk = i;
+        atomicMax(&sh_i, lastk);
+        __syncthreads();
+    }
+    if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
 }
 
 // ---------------------------------------------------------------- sampler, small top_k
@@ -447,8 +539,12 @@ extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, in
         hipLaunchKernelGGL(sample_topk_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
                            scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
                            seeds, counters);
+    else if (V <= SAMPLE_REG_IDS * SB)
+        hipLaunchKernelGGL(sample_kernel<true>, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
+                           scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
+                           seeds, counters);
     else
-        hipLaunchKernelGGL(sample_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
+        hipLaunchKernelGGL(sample_kernel<false>, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
                            scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
                            seeds, counters);
     return illm_launch_status();

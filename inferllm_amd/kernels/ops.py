@@ -934,7 +934,7 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float,
     _need(temperature > 0 and top_p > 0 and repeat_penalty > 0 and n_last <= 256,
           "sample: temperature, top_p and repeat_penalty must be positive, window <= 256")
     out = torch.empty((B,), dtype=torch.int32, device=logits.device)
-    scratch = torch.empty((B, V), dtype=torch.float32, device=logits.device)
+    scratch = torch.empty((2, B, V), dtype=torch.float32, device=logits.device)
     _check(_lib().illm_sample(
         _p(logits), _p(scratch), _p(out), B, V, ctypes.c_float(temperature), int(top_k),
         ctypes.c_float(top_p), ctypes.c_float(repeat_penalty), _p(last_tokens), n_last, _p(seeds),

@@ -718,7 +718,9 @@ def test_the_uniform_numbers_of_the_tests_and_of_the_host_side_agree():
 @pytest.mark.parametrize("V,temperature,top_k,top_p,penalty", [
     (256, 0.8, 0, 1.0, 1.0), (320, 0.8, 40, 0.95, 1.1), (411, 0.1, 40, 0.95, 1.3), (1000, 1.5, 5, 1.0, 1.0),
     (32000, 1.0, 0, 0.9, 1.0), (300, 0.7, 1, 1.0, 1.0), (128256, 0.9, 50, 0.8, 1.2),
-    (2000, 0.9, 1024, 0.7, 1.1), (2000, 0.9, 1025, 0.7, 1.0), (50, 1.0, 49, 0.5, 1.0), (32000, 0.1, 40, 0.95, 1.1)])
+    (2000, 0.9, 1024, 0.7, 1.1), (2000, 0.9, 1025, 0.7, 1.0), (50, 1.0, 49, 0.5, 1.0), (32000, 0.1, 40, 0.95, 1.1),
+    # rows too long for a thread's registers: top_p alone, with a large top_k, temperature alone
+    (128256, 0.9, 0, 0.8, 1.2), (40000, 1.0, 2000, 0.6, 1.0), (33000, 0.7, 0, 0.999, 1.0), (50000, 1.3, 0, 1.0, 1.0)])
 def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top_p, penalty):
     uniform = R.uniform                                      # the tests' own statement of the hash
     B = 6
