@@ -1,7 +1,7 @@
 from .engine import Engine, parse_dtype
-from .generate import GenerationLoop, GenerationStats
+from .generate import GenerationLoop, GenerationStats, plan_prefill
 from .model import DecoderModel, expected_tensors
 from .step import StepEntry, StepError, StepRunner
 
-__all__ = ["Engine", "parse_dtype", "GenerationLoop", "GenerationStats", "DecoderModel",
+__all__ = ["Engine", "parse_dtype", "GenerationLoop", "GenerationStats", "plan_prefill", "DecoderModel",
            "expected_tensors", "StepEntry", "StepError", "StepRunner"]

@@ -180,8 +180,12 @@ class Engine:
                  top_k: int = 0, top_p: float = 1.0, repeat_penalty: float = 1.0,
                  repeat_last_n: int = 64, seed: int = 0, max_new_tokens: int = 128,
                  stop_token_ids: Optional[Sequence[int]] = None,
-                 include_stop: bool = False, on_token=None) -> List[List[int]]:
+                 include_stop: bool = False, on_token=None,
+                 max_step_tokens: Optional[int] = None) -> List[List[int]]:
         """Generated token ids for every prompt (lists of token ids).
+
+        `max_step_tokens`: most tokens a step of prompts may hold; a batch's prompts are then fed
+        in several steps (models whose mixers can go on from the cache by several tokens).
 
         `stop_token_ids` defaults to the model's eos ids; a stop token ends its
         sequence and is left out of the result unless `include_stop`.  `on_token(request
@@ -197,11 +201,15 @@ class Engine:
             for t in p:
                 if not (0 <= int(t) < vocab):
                     raise ValueError(f"request {i}: token id {t} outside the vocabulary of {vocab}")
+        if max_step_tokens is not None and self.model.one_token_mixers:
+            raise ValueError("max_step_tokens: this model's " + ", ".join(self.model.one_token_mixers)
+                             + " cannot go on from the cache by several tokens")
         loop = GenerationLoop(self.step, sampler, self.alloc_slot, self.free_slot,
                               max_batch=self.max_batch, max_tokens=self.cache.max_tokens,
                               max_seq_len=self.max_seq_len, page_size=self.cache.page_size,
                               sync=lambda: torch.cuda.synchronize(self.device), on_token=on_token,
-                              draw=sampler.draw)
+                              draw=sampler.draw, max_step_tokens=max_step_tokens,
+                              join=lambda pieces: torch.stack([lg[row] for lg, row in pieces]))
         out = loop.run(prompts, params, max_new_tokens, stops, include_stop)
         self.last_stats = loop.stats
         return out

@@ -14,6 +14,11 @@ limit) are known beforehand; a sequence that drew a stop token has one more step
 whose result is dropped.  A draw that looks at the tokens before it (the repeat penalty) gets
 the newest one, which the host has not read yet, from the device as well (`latest`).
 
+With `max_step_tokens` the prompts of a batch are fed in several steps of at most that many
+tokens (`plan_prefill`): a long prompt, or many prompts, need not fit one step's activations.
+A step then holds sequences that go on beside sequences that start, which the step function
+takes from models whose mixers can go on by several tokens.
+
 The loop only decides; computing is behind a few callables, so its decisions can
 be tested without a GPU.  The reference's loop is `application/chat.cpp:221-275`
 over `ModelImp::decode_iter` (src/core/model_imp.cpp:55-79): one sequence, ended by
@@ -51,6 +56,31 @@ class GenerationStats:
                 f"{self.decode_seconds * 1e3:.1f} ms, {dc:.1f} token/s")
 
 
+def plan_prefill(prompt_lens: Sequence[int], limit: int) -> List[List[tuple]]:
+    """The steps that feed prompts of these lengths with at most `limit` tokens a step: lists of
+    (place in the batch, first token, number of tokens).  Prompts are fed in order; a step takes
+    the rest of the prompt that is under way, then goes on with the next ones while it has
+    room."""
+    if limit < 1:
+        raise ValueError(f"max_step_tokens must be at least 1, got {limit}")
+    done = [0] * len(prompt_lens)
+    steps: List[List[tuple]] = []
+    while any(d < n for d, n in zip(done, prompt_lens)):
+        room, step = limit, []
+        for i, n in enumerate(prompt_lens):
+            if done[i] < n and room > 0:
+                take = min(n - done[i], room)
+                step.append((i, done[i], take))
+                done[i] += take
+                room -= take
+        steps.append(step)
+    return steps
+
+
+def _rows_of_lists(pieces):
+    return [logits[row] for logits, row in pieces]
+
+
 @dataclass
 class _Live:
     index: int                 # request index in the call
@@ -77,9 +107,15 @@ class GenerationLoop:
                  free_slot: Callable[[int], None], max_batch: int, max_tokens: int,
                  max_seq_len: int, page_size: int = 64, sync: Optional[Callable[[], None]] = None,
                  on_token: Optional[Callable[[int, int], None]] = None,
-                 draw: Optional[Callable] = None):
+                 draw: Optional[Callable] = None, max_step_tokens: Optional[int] = None,
+                 join: Optional[Callable] = None):
+        """`max_step_tokens`: most tokens the prompts' steps may hold (None: a batch's prompts in
+        one step); `join(pieces)` then puts the sequences' last-token logits, given as (a step's
+        logits, row) in batch order, together in the step function's form (default: a list)."""
         self.step, self.sample = step, sample
         self.draw = draw
+        self.max_step_tokens = max_step_tokens
+        self.join = join or _rows_of_lists
         self.alloc_slot, self.free_slot = alloc_slot, free_slot
         self.max_batch, self.max_tokens, self.max_seq_len = max_batch, max_tokens, max_seq_len
         self.page_size = page_size
@@ -124,6 +160,27 @@ class GenerationLoop:
             return "context"        # the drawn token could not be fed back
         return None
 
+    def _prefill(self, live: Sequence[_Live], prompts):
+        """The batch's prompts through the step function; the logits at every prompt's last
+        token, in batch order."""
+        lens = [s.prompt_len for s in live]
+        if self.max_step_tokens is None or sum(lens) <= self.max_step_tokens:
+            return self.step([StepEntry(s.slot, prompts[s.index], [s.prompt_len - 1]) for s in live])
+        pieces: List[Optional[tuple]] = [None] * len(live)
+        for step in plan_prefill(lens, self.max_step_tokens):
+            entries, owners = [], []
+            for i, start, n in step:
+                s = live[i]
+                ends = start + n == s.prompt_len
+                entries.append(StepEntry(s.slot, prompts[s.index][start:start + n],
+                                         [n - 1] if ends else []))
+                if ends:
+                    owners.append(i)
+            logits = self.step(entries)
+            for row, i in enumerate(owners):
+                pieces[i] = (logits, row)
+        return self.join(pieces)
+
     # ------------------------------------------------------------ the loop
     def run(self, prompts: Sequence[Sequence[int]], params: SamplingParams, max_new_tokens: int,
             stop_token_ids: Sequence[int] = (), include_stop: bool = False) -> List[List[int]]:
@@ -159,8 +216,7 @@ class GenerationLoop:
             self.stats.batches += 1
             self.sync()
             t0 = time.perf_counter()
-            logits = self.step([StepEntry(s.slot, prompts[s.index], [s.prompt_len - 1])
-                                for s in everyone])
+            logits = self._prefill(everyone, prompts)
             pending = self.draw(logits, [s.seed for s in everyone], [0] * len(everyone),
                                 [s.history for s in everyone], None)
             self.sync()
@@ -227,8 +283,7 @@ class GenerationLoop:
             self.stats.batches += 1
             self.sync()
             t0 = time.perf_counter()
-            logits = self.step([StepEntry(s.slot, prompts[s.index], [s.prompt_len - 1])
-                                for s in live])
+            logits = self._prefill(live, prompts)
             tokens = self.sample(logits, [s.seed for s in live], [0] * len(live),
                                  [s.history for s in live])
             self.sync()

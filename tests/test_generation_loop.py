@@ -2,18 +2,19 @@
 batches, stop tokens, sequences that end earlier, limits, slots given back."""
 import pytest
 
-from inferllm_amd.engine import GenerationLoop, StepEntry
+from inferllm_amd.engine import GenerationLoop, StepEntry, plan_prefill
 from inferllm_amd.sampling import SamplingParams, request_seed, uniform
 
 
 class FakeModel:
     """next token = (sum of the sequence so far) % 50; keeps its own view of each slot."""
 
-    def __init__(self, n_slots):
+    def __init__(self, n_slots, takes_cut_prompts=False):
         self.free = list(range(n_slots - 1, -1, -1))
         self.seq = {}
         self.steps = []
         self.max_live = 0
+        self.takes_cut_prompts = takes_cut_prompts     # steps that go on by several tokens
 
     def alloc(self):
         s = self.free.pop()
@@ -27,14 +28,18 @@ class FakeModel:
 
     def step(self, entries, device_tokens=None):
         first = [len(self.seq[e.slot]) == 0 for e in entries]
-        assert all(first) or (not any(first) and all(len(e.tokens) == 1 for e in entries))
+        assert (self.takes_cut_prompts or all(first)
+                or (not any(first) and all(len(e.tokens) == 1 for e in entries)))
         if device_tokens is not None:
             assert not any(first) and len(device_tokens) == len(entries)
         for i, e in enumerate(entries):
             self.seq[e.slot].extend(e.tokens if device_tokens is None else [device_tokens[i]])
         self.steps.append([(e.slot, len(e.tokens)) for e in entries])
         self.max_live = max(self.max_live, len(self.seq))
-        return [sum(self.seq[e.slot]) % 50 for e in entries]
+        # a row for every wanted place, which is the entry's last token if any
+        assert all(list(e.want) in ([], [len(e.tokens) - 1]) for e in entries)
+        rows = [sum(self.seq[e.slot]) % 50 for e in entries if list(e.want)]
+        return rows or None
 
     @staticmethod
     def sample(logits, seeds, counters, histories):
@@ -237,3 +242,39 @@ def test_random_stops_and_limits_give_the_same_with_and_without_running_ahead():
             got.append(loop.run(prompts, SamplingParams(), n_new, stops, include))
             assert not m.seq and len(m.free) == 3
         assert got[0] == got[1] == [expected(p, n_new, stops, include, limit) for p in prompts], trial
+
+
+def test_plan_of_prompts_cut_into_steps():
+    assert plan_prefill([5, 3], 100) == [[(0, 0, 5), (1, 0, 3)]]
+    # the rest of the prompt under way first, then the next ones while there is room
+    assert plan_prefill([10, 3, 4], 6) == [[(0, 0, 6)], [(0, 6, 4), (1, 0, 2)], [(1, 2, 1), (2, 0, 4)]]
+    assert plan_prefill([2, 2, 2], 4) == [[(0, 0, 2), (1, 0, 2)], [(2, 0, 2)]]
+    assert plan_prefill([3], 1) == [[(0, 0, 1)], [(0, 1, 1)], [(0, 2, 1)]]
+    for lens, limit in (([7, 1, 30, 2], 8), ([64, 64], 64), ([1, 1, 1], 2)):
+        steps = plan_prefill(lens, limit)
+        assert all(0 < sum(n for _, _, n in st) <= limit for st in steps)
+        fed = [0] * len(lens)
+        for st in steps:
+            for i, start, n in st:
+                assert start == fed[i]                      # every prompt in order, nothing twice
+                fed[i] += n
+        assert fed == lens
+        assert sum(1 for st in steps if sum(n for _, _, n in st) < limit) <= 1    # only the last step is not full
+    with pytest.raises(ValueError, match="at least 1"):
+        plan_prefill([3], 0)
+
+
+@AHEAD
+@pytest.mark.parametrize("limit", [1, 4, 6, 100])
+def test_prompts_fed_in_several_steps_give_the_same_tokens(ahead, limit):
+    m = FakeModel(3, takes_cut_prompts=True)
+    loop = GenerationLoop(m.step, m.sample, m.alloc, m.release, 3, 64 * 12, 256,
+                          draw=m.draw if ahead else None, max_step_tokens=limit)
+    out = loop.run(PROMPTS, SamplingParams(), 5)
+    assert out == [expected(p, 5) for p in PROMPTS]
+    assert not m.seq and loop.stats.prompt_tokens == sum(map(len, PROMPTS))
+    # no step of prompts holds more tokens than the limit (single-token steps of the batch aside)
+    assert all(sum(n for _, n in st) <= max(limit, 3) for st in m.steps)
+    if limit == 4:
+        # the first batch's prompts of 3, 1 and 5 tokens: [3 + 1], [4 of the third], [its last]
+        assert m.steps[:3] == [[(0, 3), (1, 1)], [(2, 4)], [(2, 1)]]

@@ -17,6 +17,24 @@ DEV = "cuda:0"
 # float32: rounding of sums of a few hundred float32 terms.  bfloat16: activations carry
 # 8 bits (2^-8 = 0.4 %) and pass through up to 3 blocks and the head.
 BUDGET = {"float32": 2e-5, "bfloat16": 3e-2}
+@pytest.mark.parametrize("name,limit", [("A", 5), ("B", 16), ("A", 64)])
+def test_generation_with_prompts_fed_in_several_steps(tmp_path_factory, name, limit):
+    """`max_step_tokens`: the prompts of a batch in steps of at most that many tokens (sequences
+    that go on beside sequences that start); the generated tokens are the plain model's.  A model
+    with a mixer that cannot go on by several tokens refuses."""
+    config = CONFIGS[name]
+    eng, plain, _ = setup(tmp_path_factory, name, "float32", max_batch=3)
+    _, w = _cache[(name, "float32")]
+    prompts = requests_for(config, [23, 1, 40, 9, 64], seed=12)
+    got = eng.generate(prompts, max_new_tokens=5, stop_token_ids=[], max_step_tokens=limit)
+    assert got == [plain_llama.generate_greedy(config, w, p, 5) for p in prompts]
+    eng.cache.check()
+    assert eng.cache.slots.n_held() == 0
+    eng.model.one_token_mixers = ["SomeMixer"]            # (what a model with such a mixer reports)
+    with pytest.raises(ValueError, match="SomeMixer cannot go on"):
+        eng.generate(prompts[:1], max_new_tokens=2, max_step_tokens=4)
+
+
 STORE = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 _cache = {}
