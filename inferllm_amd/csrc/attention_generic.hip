@@ -187,9 +187,14 @@ extern "C" int illm_attn_prefill_paged_generic(const void* qkv, void* out, int d
 }
 
 // ---------------------------------------------------------------- decode
-// grid (heads, sequences, splits); 256 threads; tiles of 256 keys aligned at absolute
-// positions, so a key's place in the sums does not depend on the number of splits
-// beyond the split boundaries.  Each block leaves (acc[hd], max, sum) in `partial`.
+// grid (heads, sequences, splits); 256 threads.  A split takes whole tiles of 256 keys aligned at
+// absolute positions.  A wave takes eight keys at a time, in turn with the block's other waves;
+// lane l holds dims l, l + 64, l + 128, l + 192 of the query and of its sums, so a key's or a
+// value's row is read 256 bytes an instruction (a thread a key, walking its row by itself, took
+// 155 us for 520 keys at head size 128: every load of a wave touched 64 rows), and the eight
+// scores are summed over the wave together, each step handing half of them to the partner lane.
+// The waves' (sums, max, weight) are combined in wave order at the end; each block leaves
+// (acc[hd], max, sum) in `partial`.  Plain float32 arithmetic and expf.
 __global__ void __launch_bounds__(256)
 attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __restrict__ kcache,
                            const void* __restrict__ vcache,
@@ -197,11 +202,12 @@ attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __r
                            int page_size, int ring, const int32_t* __restrict__ seq_slot,
                            const int32_t* __restrict__ seq_len, float* __restrict__ partial,
                            int nsplit, int nh, int nkv, int hd, float scale, int window) {
-    __shared__ float qs[256];
-    __shared__ float ps[256];
-    __shared__ float red[16];
+    constexpr int KU = 8;                  // keys a wave takes at a time
+    constexpr int DL = 4;                  // dims a lane holds (head sizes up to 256)
+    __shared__ float wave_acc[4][256];
+    __shared__ float wave_ml[4][2];
     const int h = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
-    const int tid = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     const int slot = seq_slot[b];
     const int len = seq_len[b];
     const int kvh = h / (nh / nkv);
@@ -212,46 +218,101 @@ attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __r
     const int per_split = (n_tiles + nsplit - 1) / nsplit;
     const int t_lo = first_tile + sp * per_split;
     const int t_hi = min(first_tile + n_tiles, t_lo + per_split);
+    const int k_lo = max(k_first, t_lo * 256), k_hi = min(len, t_hi * 256);
 
-    if (tid < hd) qs[tid] = ld_f(qkv, dt, (size_t)b * rowlen + (size_t)h * hd + tid);
-    float m = NEG_INF, l = 0.f, acc = 0.f;
-    for (int t = t_lo; t < t_hi; ++t) {
-        __syncthreads();
-        const int kj = t * 256 + tid;
-        float s = NEG_INF;
-        if (kj >= k_first && kj < len) {
-            const size_t off = cache_row_offset(page_table, table_stride, slot, kj, page_size,
-                                                ring, nkv, kvh, hd);
+    float q[DL], acc[DL];
+    int dim[DL];                           // (a lane without a dim reads dim 0; its sums are dropped)
+#pragma unroll
+    for (int i = 0; i < DL; ++i) {
+        const int d = lane + 64 * i;
+        dim[i] = d < hd ? d : 0;
+        q[i] = d < hd ? ld_f(qkv, dt, (size_t)b * rowlen + (size_t)h * hd + d) : 0.f;
+        acc[i] = 0.f;
+    }
+    float m = NEG_INF, l = 0.f;
+    for (int k0 = k_lo + wave * KU; k0 < k_hi; k0 += 4 * KU) {
+        // keys beyond the range read its last key again (an existing row) and get no weight
+        size_t off[KU];
+#pragma unroll
+        for (int j = 0; j < KU; ++j)
+            off[j] = cache_row_offset(page_table, table_stride, slot, min(k0 + j, k_hi - 1),
+                                      page_size, ring, nkv, kvh, hd);
+        float part[KU];
+#pragma unroll
+        for (int j = 0; j < KU; ++j) {
             float a = 0.f;
-            for (int d = 0; d < hd; ++d) a = fmaf(qs[d], ld_f(kcache, dt, off + d), a);
-            s = a * scale;
+#pragma unroll
+            for (int i = 0; i < DL; ++i) a = fmaf(q[i], ld_f(kcache, dt, off[j] + dim[i]), a);
+            part[j] = a;
         }
-        const float m_new = fmaxf(m, block_max(s, red));
-        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
-        const float p = (s == NEG_INF) ? 0.f : expf(s - m_new);
-        ps[tid] = p;
-        const float psum = block_sum(p, red);
+        // eight sums over 64 lanes: three steps that halve what a lane keeps (the sums whose
+        // number has the lane's bit), then three plain ones; sum j ends in the lanes with
+        // (lane & 7) == j
+#pragma unroll
+        for (int bit = 1, n = KU / 2; bit < KU; bit <<= 1, n >>= 1) {
+            const bool up = (lane & bit) != 0;
+#pragma unroll
+            for (int k = 0; k < n; ++k) {
+                const float keep = up ? part[2 * k + 1] : part[2 * k];
+                const float send = up ? part[2 * k] : part[2 * k + 1];
+                part[k] = keep + __shfl_xor(send, bit, ILLM_WAVE);
+            }
+        }
+        float mine = part[0];
+#pragma unroll
+        for (int o = KU; o < 64; o <<= 1) mine += __shfl_xor(mine, o, ILLM_WAVE);
+        float s[KU];
+#pragma unroll
+        for (int j = 0; j < KU; ++j) {
+            const float v = __shfl(mine, j, ILLM_WAVE) * scale;
+            s[j] = k0 + j < k_hi ? v : NEG_INF;
+        }
+        float mx = s[0];
+#pragma unroll
+        for (int j = 1; j < KU; ++j) mx = fmaxf(mx, s[j]);
+        const float m_new = fmaxf(m, mx);          // finite: key k0 is in the range
+        const float alpha = (m == NEG_INF) ? 0.f : expf(m - m_new);
+        float psum = 0.f, pv[KU];
+#pragma unroll
+        for (int j = 0; j < KU; ++j) {
+            pv[j] = (s[j] == NEG_INF) ? 0.f : expf(s[j] - m_new);
+            psum += pv[j];
+        }
         l = l * alpha + psum;
         m = m_new;
-        __syncthreads();
-        if (tid < hd) {
-            float a = acc * alpha;
-            const int jn = min(256, len - t * 256);
-            for (int j = 0; j < jn; ++j) {
-                const float pj = ps[j];
-                if (pj == 0.f) continue;
-                const size_t off = cache_row_offset(page_table, table_stride, slot, t * 256 + j,
-                                                    page_size, ring, nkv, kvh, hd);
-                a = fmaf(pj, ld_f(vcache, dt, off + tid), a);
-            }
-            acc = a;
+#pragma unroll
+        for (int i = 0; i < DL; ++i) {
+            float a = acc[i] * alpha;
+#pragma unroll
+            for (int j = 0; j < KU; ++j) a = fmaf(pv[j], ld_f(vcache, dt, off[j] + dim[i]), a);
+            acc[i] = a;
         }
     }
+    // the waves' results, combined in wave order
+#pragma unroll
+    for (int i = 0; i < DL; ++i) wave_acc[wave][lane + 64 * i] = acc[i];
+    if (lane == 0) {
+        wave_ml[wave][0] = m;
+        wave_ml[wave][1] = l;
+    }
+    __syncthreads();
+    float mb = NEG_INF;
+    for (int w = 0; w < 4; ++w) mb = fmaxf(mb, wave_ml[w][0]);
+    float lb = 0.f, f[4];
+    for (int w = 0; w < 4; ++w) {
+        f[w] = (wave_ml[w][0] == NEG_INF) ? 0.f : expf(wave_ml[w][0] - mb);
+        lb += f[w] * wave_ml[w][1];
+    }
     float* pp = partial + (((size_t)b * nh + h) * nsplit + sp) * (size_t)(hd + 2);
-    if (tid < hd) pp[tid] = acc;
+    const int tid = threadIdx.x;
+    if (tid < hd) {
+        float a = 0.f;
+        for (int w = 0; w < 4; ++w) a += f[w] * wave_acc[w][tid];
+        pp[tid] = a;
+    }
     if (tid == 0) {
-        pp[hd] = m;
-        pp[hd + 1] = l;
+        pp[hd] = mb;
+        pp[hd + 1] = lb;
     }
 }
 

@@ -409,9 +409,11 @@ def test_gate_up_silu(M, F, K):
 
 
 @pytest.mark.parametrize("ydt", DTYPES)
-@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 100, 136), (16, 33, 1000), (5, 320, 96), (3, 7, 4), (9, 11008, 4096)])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 100, 136), (16, 33, 1000), (5, 320, 96), (3, 7, 4), (9, 11008, 4096),
+                                   (17, 100, 136), (64, 320, 96), (100, 33, 1000), (128, 4096, 512)])
 def test_gemv_rows_f32(ydt, M, N, K):
-    """The 32-bit path's product of few rows: float32 sums, W read once."""
+    """The 32-bit path's product of few rows: float32 sums, W read once for every 16 rows; a
+    row's result is the same bits whatever rows stand beside it."""
     x, w = rnd(M, K, seed=1), rnd(N, K, seed=2)
     assert ops().gemv_rows_f32_fits(x.to(DEV), w.to(DEV))
     got = ops().linear(x.to(DEV), w.to(DEV), ydt)
@@ -420,7 +422,10 @@ def test_gemv_rows_f32(ydt, M, N, K):
         torch.testing.assert_close(got.double().cpu(), want, atol=2e-6 * math.sqrt(K) * 4, rtol=1e-5)
     else:
         close(got, want, ydt, scale=math.sqrt(K))
-    assert not ops().gemv_rows_f32_fits(rnd(17, K).to(DEV), w.to(DEV))
+    if ydt == torch.float32 and M > 1:
+        alone = ops().linear(x[M - 1:].contiguous().to(DEV), w.to(DEV), ydt)
+        assert torch.equal(alone[0], got[M - 1])
+    assert not ops().gemv_rows_f32_fits(rnd(129, K).to(DEV), w.to(DEV))
     assert not ops().gemv_rows_f32_fits(x.to(DEV).to(torch.bfloat16), w.to(DEV))
 
 
