@@ -42,6 +42,11 @@ int illm_rope_store(void* qkv, int dt, const float* cos_sin, int max_pos, int ro
 int illm_gemm_generic(const void* X, int x_dt, const void* W, int w_dt, void* Y, int y_dt,
                       int M, int N, int K, void* stream);
 
+// The same product for float32 X and W with K % 16 == 0 on the matrix cores' float32 instruction
+// (float32 operands, products and sums), for many rows.
+int illm_gemm_f32_mfma(const float* X, const float* W, void* Y, int y_dt, int M, int N, int K,
+                       void* stream);
+
 // The same product for M <= 16 rows when X and W are float32 and K % 4 == 0: W is read once
 // (decoding on the 32-bit path); plain float32 multiply-adds.
 int illm_gemv_rows_f32(const float* X, const float* W, void* Y, int y_dt, int M, int N, int K,
@@ -74,6 +79,10 @@ int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_s
                                  const void* kcache, const void* vcache, const int32_t* page_table,
                                  int table_stride, int page_size, int ring, int n_seqs, int max_len,
                                  int nh, int nkv, int hd, float scale, int window, void* stream);
+
+// Tests: whether float32 prompts with head sizes 32, 64, 96 and 128 take the kernel on the matrix
+// cores' float32 instruction (1, default) or the multiply-add kernel of every other size (0).
+void illm_set_attn_f32_mfma(int on);
 
 // Tuning and tests: which prefill attention kernel head sizes up to 128 take: 0 the one with one
 // LDS buffer (which larger head sizes use), 2 the one with two buffers and one barrier a tile

@@ -2,7 +2,8 @@
 // of heads and groups, float32 or bfloat16 storage: one kernel for whole prompts
 // (keys and values of the step itself) and one for a single new token per sequence
 // over the paged cache.  These are the kernels of the 32-bit path and the
-// fallback for sizes the MFMA kernels do not take.
+// fallback for sizes the MFMA kernels do not take.  Float32 prompts with head sizes
+// 32 to 128 take a third kernel, on the matrix cores' float32 instruction.
 //
 // What they compute is the reference's chain scores -> scale and mask -> softmax
 // -> context (src/core/op.cpp:485-498; src/kern/naive/naive.cpp:606-632, :531-553,
@@ -140,6 +141,164 @@ attn_prefill_generic_kernel(const void* __restrict__ qkv, void* __restrict__ out
     }
 }
 
+// The same attention for float32 storage and head sizes 32, 64, 96 and 128 on the matrix cores'
+// float32 instruction (MFMA 32x32x2: float32 operands, products and sums), 8 times the kernel
+// above at 2,048 tokens.  grid (tiles of 128 queries, heaviest first; heads; sequences); a wave
+// takes 32 queries.  Both products are kept transposed so that a lane's column is its query:
+// scores^T = K . Q^T puts the 16 scores of query (lane % 32) into a lane and its partner 32 lanes
+// on (max and sum: one exchange), and in context^T = V^T . P^T the lane's own 16 weights are the
+// second operand as they stand, the keys of a step being 8 g + v for the lower half of the wave
+// and 8 g + 4 + v for the upper.  Keys and values go through LDS 32 keys at a time (K padded by
+// one float a row); the next tile's loads are in flight while this one is multiplied.
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+#define FQ 128  // query rows of a block
+#define FK 32   // keys of a tile
+
+template <int HD, bool PAGED>
+__global__ void __launch_bounds__(256, 2)
+attn_prefill_f32_mfma_kernel(const float* __restrict__ qkv, float* __restrict__ out,
+                             const int32_t* __restrict__ cu, int nh, int nkv, float scale,
+                             int window, AttnPages pg) {
+    constexpr int KLD = HD + 1;
+    constexpr int NT = HD / 32;                  // tiles of 32 dims; float4 of a thread a tile
+    __shared__ float ks[FK * KLD];
+    __shared__ __align__(16) float vs[FK * HD];
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int start = cu[b], len = cu[b + 1] - start;
+    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * FQ;
+    if (q0 >= len) return;
+    const int pos0 = PAGED ? pg.seq_start[b] : 0;
+    const int slot = PAGED ? pg.seq_slot[b] : 0;
+    const int total = pos0 + len;
+    const int kvh = h / (nh / nkv);
+    const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+    const int col = lane & 31, half = lane >> 5;
+    const int qrow = q0 + 32 * wave + col;                 // row within the step's rows of the sequence
+    const int qpos = pos0 + qrow;
+    const bool wave_has_rows = q0 + 32 * wave < len;
+
+    // the query row: dims 2 s + half
+    float q[HD / 2];
+    {
+        const float4* src = (const float4*)(qkv + (size_t)(start + min(qrow, len - 1)) * rowlen + (size_t)h * HD);
+#pragma unroll
+        for (int j = 0; j < HD / 4; ++j) {
+            const float4 x = src[j];
+            q[2 * j] = half ? x.y : x.x;
+            q[2 * j + 1] = half ? x.w : x.z;
+        }
+    }
+    const float* kbase = PAGED ? (const float*)pg.kcache : qkv + (size_t)(nh + kvh) * HD;
+    const float* vbase = PAGED ? (const float*)pg.vcache : qkv + (size_t)(nh + nkv + kvh) * HD;
+    f32x4_t kreg[NT], vreg[NT];                  // (native vectors: arrays of HIP's float4 stay in memory)
+    auto fetch = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            const int e = tid + 256 * i, row = e / (HD / 4), dq = e % (HD / 4);
+            const int kj = min(k0 + row, total - 1);       // keys past the end: a valid row, masked below
+            const size_t at = (PAGED ? cache_row_offset(pg.page_table, pg.table_stride, slot, kj,
+                                                        pg.page_size, pg.ring, nkv, kvh, HD)
+                                     : (size_t)(start + kj) * rowlen) + 4 * dq;
+            kreg[i] = *(const f32x4_t*)(kbase + at);
+            vreg[i] = *(const f32x4_t*)(vbase + at);
+        }
+    };
+    auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            const int e = tid + 256 * i, row = e / (HD / 4), dq = e % (HD / 4);
+            float* kd = ks + row * KLD + 4 * dq;
+            kd[0] = kreg[i].x; kd[1] = kreg[i].y; kd[2] = kreg[i].z; kd[3] = kreg[i].w;
+            *(f32x4_t*)(vs + row * HD + 4 * dq) = vreg[i];
+        }
+    };
+    f32x16_t o[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[t][v] = 0.f;
+    float m_i = NEG_INF, l_i = 0.f;
+
+    const int k_hi = min(total, pos0 + q0 + FQ);
+    int k_lo = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
+    k_lo = (k_lo / FK) * FK;
+    const int wq_lo = pos0 + q0 + 32 * wave, wq_hi = wq_lo + 31;
+    const int k_last = k_lo + ((k_hi - 1 - k_lo) / FK) * FK;
+    fetch(k_lo);
+    for (int k0 = k_lo; k0 < k_hi; k0 += FK) {
+        __syncthreads();
+        stage();
+        __syncthreads();
+        fetch(min(k0 + FK, k_last));              // (unconditional: the last tile is asked for twice)
+        // a wave leaves out tiles that lie after all its queries or before all their windows
+        if (!wave_has_rows || k0 > wq_hi || (window > 0 && k0 + FK - 1 <= wq_lo - window)) continue;
+        f32x16_t sc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+        const float* kr = ks + col * KLD + half;
+#pragma unroll
+        for (int s = 0; s < HD / 2; ++s)
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[2 * s], q[s], sc, 0, 0, 0);
+        float tm = NEG_INF;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int kj = k0 + 8 * (v >> 2) + 4 * half + (v & 3);
+            const bool ok = qrow < len && kj <= qpos && (window <= 0 || kj > qpos - window);
+            sc[v] = ok ? sc[v] * scale : NEG_INF;
+            tm = fmaxf(tm, sc[v]);
+        }
+        tm = fmaxf(tm, __shfl_xor(tm, 32, ILLM_WAVE));
+        const float m_new = fmaxf(m_i, tm);
+        const float alpha = (m_new == NEG_INF) ? 1.f : expf(m_i - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            sc[v] = (sc[v] == NEG_INF) ? 0.f : expf(sc[v] - m_new);
+            psum += sc[v];
+        }
+        psum += __shfl_xor(psum, 32, ILLM_WAVE);
+        l_i = l_i * alpha + psum;
+        m_i = m_new;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[t][v] *= alpha;
+        const float* vr = vs + 4 * half * HD + col;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = 8 * (v >> 2) + (v & 3);         // + 4 * half, in vr
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                o[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[key * HD + 32 * t], sc[v], o[t], 0, 0, 0);
+        }
+    }
+    if (qrow < len) {
+        const float inv = 1.0f / l_i;
+        float* dst = out + (size_t)(start + qrow) * nh * HD + (size_t)h * HD + 4 * half;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *(float4*)(dst + 32 * t + 8 * g) = make_float4(o[t][4 * g] * inv, o[t][4 * g + 1] * inv,
+                                                               o[t][4 * g + 2] * inv, o[t][4 * g + 3] * inv);
+    }
+}
+
+static int g_attn_f32_mfma = 1;
+extern "C" void illm_set_attn_f32_mfma(int on) { g_attn_f32_mfma = on ? 1 : 0; }
+
+template <int HD, bool PAGED>
+static int launch_prefill_f32_mfma(const void* qkv, void* out, const int32_t* cu_seqlens, int n_seqs,
+                                   int max_len, int nh, int nkv, float scale, int window,
+                                   const AttnPages& pg, hipStream_t stream) {
+    hipLaunchKernelGGL((attn_prefill_f32_mfma_kernel<HD, PAGED>), dim3((max_len + FQ - 1) / FQ, nh, n_seqs),
+                       dim3(256), 0, stream, (const float*)qkv, (float*)out, cu_seqlens, nh, nkv, scale,
+                       window, pg);
+    return illm_launch_status();
+}
+
 template <bool PAGED>
 static int launch_prefill_generic(const void* qkv, void* out, int dt, const int32_t* cu_seqlens,
                                   int n_seqs, int max_len, int nh, int nkv, int hd, float scale,
@@ -148,6 +307,15 @@ static int launch_prefill_generic(const void* qkv, void* out, int dt, const int3
         !illm_dtype_ok(dt) || nh > 65535 || n_seqs > 65535)
         return ILLM_ERR_ARG;
     if (n_seqs == 0 || max_len == 0) return ILLM_OK;
+    if (dt == ILLM_F32 && g_attn_f32_mfma) {
+        switch (hd) {
+            case 32: return launch_prefill_f32_mfma<32, PAGED>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, pg, stream);
+            case 64: return launch_prefill_f32_mfma<64, PAGED>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, pg, stream);
+            case 96: return launch_prefill_f32_mfma<96, PAGED>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, pg, stream);
+            case 128: return launch_prefill_f32_mfma<128, PAGED>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, pg, stream);
+            default: break;
+        }
+    }
     const size_t smem = ((size_t)(AQ + 2 * AK) * (hd + 1) + AQ * (AK + 1)) * sizeof(float);
     if (smem > 48 * 1024) {
         if (hipFuncSetAttribute((const void*)attn_prefill_generic_kernel<PAGED>,

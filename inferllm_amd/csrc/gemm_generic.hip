@@ -3,7 +3,10 @@
 // reduced-precision mode).  Each output element is summed over k in ascending
 // order, whatever its row's place in the batch, so a row gives the same bits
 // whether it comes alone or among others.  This is the matrix product of the
-// 32-bit path and the fallback for shapes the MFMA kernels do not take.
+// 32-bit path and the fallback for shapes the MFMA kernels do not take.  Two more
+// kernels below serve the 32-bit path's common cases faster, both in float32
+// throughout: few rows (W read once) and many rows (the matrix cores' float32
+// instruction).
 //
 // The reference's float product is the same sum (src/kern/naive/naive.cpp:363-379);
 // its GPU path calls cublasSgemm (src/kern/gpu/kernel_gpu.cu:420-435).
@@ -74,6 +77,128 @@ extern "C" int illm_gemm_generic(const void* X, int x_dt, const void* W, int w_d
     if (gy > 65535) return ILLM_ERR_ARG;
     hipLaunchKernelGGL(gemm_generic_kernel, dim3((N + GT - 1) / GT, gy), dim3(256), 0,
                        (hipStream_t)stream, X, x_dt, W, w_dt, Y, y_dt, M, N, K);
+    return illm_launch_status();
+}
+
+
+// ---------------------------------------------------------------- many rows, float32
+// The same product for float32 X and W with K a multiple of 16, on the matrix cores' float32
+// instruction (MFMA 32x32x2: float32 operands, float32 products and sums; nothing is rounded to
+// a shorter type).  The multiply-add tile above reaches 45 TFLOP/s, 0.57 of what the vector units
+// give without packed instructions; the matrix cores' float32 rate is twice the vector units'.
+// A block of four waves takes 128 x 128 outputs, a wave 64 x 64 (2 x 2 MFMA tiles); both
+// operands go through LDS k-major (16 k a stage, two buffers, the next stage's loads in flight
+// while this one is multiplied).  The MFMA's rows are W's (n) and its columns X's (m), so a lane
+// holds 4 consecutive n of one m: 16-byte stores.  An output element is summed over k in
+// ascending pairs whatever its row's place in the batch.
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+#define FM_T 128     // outputs of a block along m and along n
+#define FM_K 16      // k a stage
+#define FM_LD 130    // LDS row stride in floats (4 * FM_LD = 8 mod 32: the stores of a half-wave,
+                     // 8 rows x 4 k-quads, fall into 32 different banks)
+
+__global__ void __launch_bounds__(256)
+gemm_f32_mfma_kernel(const float* __restrict__ X, const float* __restrict__ W, void* __restrict__ Y,
+                     int y_dt, int M, int N, int K) {
+    __shared__ float xs[2][FM_K][FM_LD];
+    __shared__ float ws[2][FM_K][FM_LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+    const int r = lane & 31, kh = lane >> 5;
+    const int wm = wave & 1, wn = wave >> 1;
+    const int m0 = blockIdx.y * FM_T, n0 = blockIdx.x * FM_T;
+
+    // staging: thread t brings 4 k (quad t % 4) of rows t / 4 and t / 4 + 64 of both operands;
+    // rows beyond the matrix read its last row (their outputs are not stored)
+    const int s_row = tid >> 2, s_kq = tid & 3;
+    const float* xsrc[2];
+    const float* wsrc[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        xsrc[e] = X + (size_t)min(m0 + s_row + 64 * e, M - 1) * K + s_kq * 4;
+        wsrc[e] = W + (size_t)min(n0 + s_row + 64 * e, N - 1) * K + s_kq * 4;
+    }
+    float4 xg[2], wg[2];
+    auto fetch = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            xg[e] = *(const float4*)(xsrc[e] + k0);
+            wg[e] = *(const float4*)(wsrc[e] + k0);
+        }
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int row = s_row + 64 * e;
+            xs[buf][s_kq * 4 + 0][row] = xg[e].x; xs[buf][s_kq * 4 + 1][row] = xg[e].y;
+            xs[buf][s_kq * 4 + 2][row] = xg[e].z; xs[buf][s_kq * 4 + 3][row] = xg[e].w;
+            ws[buf][s_kq * 4 + 0][row] = wg[e].x; ws[buf][s_kq * 4 + 1][row] = wg[e].y;
+            ws[buf][s_kq * 4 + 2][row] = wg[e].z; ws[buf][s_kq * 4 + 3][row] = wg[e].w;
+        }
+    };
+    f32x16_t acc[2][2];                    // [n tile][m tile]
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += FM_K, buf ^= 1) {
+        const bool more = k0 + FM_K < K;
+        if (more) fetch(k0 + FM_K);
+#pragma unroll
+        for (int s = 0; s < FM_K / 2; ++s) {
+            float a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = ws[buf][2 * s + kh][wn * 64 + 32 * i + r];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = xs[buf][2 * s + kh][wm * 64 + 32 * j + r];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) stage(buf ^ 1);          // (last read before the barrier that ended the stage before)
+        __syncthreads();
+    }
+    // acc[i][j][v]: n = n0 + wn * 64 + 32 i + 8 (v / 4) + 4 kh + v % 4, m = m0 + wm * 64 + 32 j + r
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int m = m0 + wm * 64 + 32 * j + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wn * 64 + 32 * i + 8 * g + 4 * kh;
+                const size_t at = (size_t)m * N + n;
+                if (n + 3 < N && (N & 3) == 0 && y_dt == ILLM_F32) {
+                    *(float4*)((float*)Y + at) = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1],
+                                                             acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (n + v < N) st_f(Y, y_dt, at + v, acc[i][j][4 * g + v]);
+                }
+            }
+    }
+}
+
+// float32 X [M, K] and W [N, K], K % 16 == 0; Y float32 or bfloat16.  Else ILLM_ERR_ARG.
+extern "C" int illm_gemm_f32_mfma(const float* X, const float* W, void* Y, int y_dt, int M, int N,
+                                  int K, void* stream) {
+    if (M <= 0 || N <= 0 || K <= 0 || (K % FM_K) || !illm_dtype_ok(y_dt) || !X || !W || !Y)
+        return ILLM_ERR_ARG;
+    const int gy = (M + FM_T - 1) / FM_T;
+    if (gy > 65535) return ILLM_ERR_ARG;
+    hipLaunchKernelGGL(gemm_f32_mfma_kernel, dim3((N + FM_T - 1) / FM_T, gy), dim3(256), 0,
+                       (hipStream_t)stream, X, W, Y, y_dt, M, N, K);
     return illm_launch_status();
 }
 

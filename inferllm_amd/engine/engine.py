@@ -41,7 +41,7 @@ class Engine:
 
     dtype "bfloat16": bfloat16 matrices, activations and cache, float32 residual
     stream, statistics and logits.  dtype "float32": everything in true
-    float32 (own multiply-add kernels; no matrix-core or reduced-precision mode).
+    float32 (own kernels: float32 operands, products and sums; no reduced-precision mode).
 
     `decode_copies`: keep a second copy of every matrix in the layout of the few-rows kernels
     (decoding reads that one, prompts the row-major one), or with "thin" of the down projections

@@ -199,6 +199,25 @@ def gemm_generic(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> to
     return y
 
 
+def gemm_f32_mfma_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.float32 and w.dtype == torch.float32 and x.dim() == 2 and w.dim() == 2
+            and x.shape[0] >= 1 and x.shape[1] == w.shape[1] and x.shape[1] % 16 == 0
+            and x.is_contiguous() and w.is_contiguous())
+
+
+def gemm_f32_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M, K] . w [N, K]^T, both float32, on the matrix cores' float32 instruction (float32
+    operands, products and sums; no shorter type anywhere).  For many rows."""
+    _gpu(x, w)
+    _need(gemm_f32_mfma_fits(x, w), "gemm_f32_mfma: operands not taken")
+    M, K = x.shape
+    N = w.shape[0]
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_gemm_f32_mfma(_p(x), _p(w), _p(y), _code(y), M, N, K, _stream()),
+           "gemm_f32_mfma")
+    return y
+
+
 class Weight:
     """A matrix [N, K] of a product with, optionally, a second copy laid out for the few-rows
     kernels (`tile_weight`).  Wherever the ops take a weight they take this or a plain tensor."""
@@ -503,6 +522,8 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     if x.dtype == torch.float32 or w.dtype == torch.float32:
         if gemv_rows_f32_fits(x, w):
             return gemv_rows_f32(x, w, out_dtype)
+        if gemm_f32_mfma_fits(x, w):
+            return gemm_f32_mfma(x, w, out_dtype)
         return gemm_generic(x, w, out_dtype)
     M, K = x.shape
     if M == 0:

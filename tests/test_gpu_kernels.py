@@ -227,10 +227,47 @@ def test_attn_prefill_mfma(nh, nkv, hd, lens, window):
         lib.illm_set_prefill_two_buffers(1)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,lens,window", [
+    (4, 4, 128, [300, 129, 128, 1], 0), (8, 1, 64, [257, 64], 0), (3, 3, 96, [200], 0), (6, 2, 32, [127, 130], 0),
+    (4, 2, 128, [400], 100), (2, 2, 64, [333, 5], 64), (2, 1, 32, [300], 7), (3, 1, 96, [31, 32, 33, 161], 33),
+    (32, 8, 128, [600, 130, 577, 64], 0), (2, 1, 128, [1500, 40], 0)])
+def test_attn_prefill_f32_matrix_cores(nh, nkv, hd, lens, window):
+    """Float32 prompts with head sizes 32 to 128: the kernel on the matrix cores' float32
+    instruction (blocks of 128 query rows, tiles of 32 keys) and the multiply-add kernel, both
+    within the float32 budget of the plain implementation."""
+    T = sum(lens)
+    qkv = rnd(T, (nh + 2 * nkv) * hd, seed=19)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    scale = 1.0 / math.sqrt(hd)
+    want = R.attn_prefill(qkv, cu, len(lens), max(lens), nh, nkv, hd, scale, window)
+    lib = ops()._lib()
+    try:
+        for on in (1, 0):
+            lib.illm_set_attn_f32_mfma(on)
+            got = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), len(lens), max(lens), nh, nkv, hd, scale, window)
+            close(got, want, torch.float32, scale=2)
+    finally:
+        lib.illm_set_attn_f32_mfma(1)
+
+
+def test_attn_prefill_f32_finds_one_far_key():
+    """One early key is made to stand out for a late query of another block and wave: the
+    output is that key's value; a query before the key does not see it."""
+    nh, nkv, hd, n = 2, 1, 128, 700
+    qkv = rnd(n, (nh + 2 * nkv) * hd, seed=3)
+    view = qkv.view(n, nh + 2 * nkv, hd)
+    view[37, nh] = view[650, 1] * 30
+    cu = torch.tensor([0, n], dtype=torch.int32)
+    got = ops().attn_prefill(qkv.to(DEV), cu.to(DEV), 1, n, nh, nkv, hd, 1.0, 0).cpu().view(n, nh, hd)
+    torch.testing.assert_close(got[650, 1], view[37, nh + nkv], atol=1e-4, rtol=1e-4)
+    assert not torch.allclose(got[30, 1], view[37, nh + nkv], atol=0.1)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,hd,starts,rows,page", [
     (4, 2, 32, [0, 70, 5], [40, 30, 1], 64), (8, 8, 128, [200, 0], [130, 64], 64), (3, 1, 48, [17, 64], [9, 200], 64),
-    (6, 2, 24, [3], [5], 16), (2, 2, 256, [63], [66], 64), (32, 8, 128, [1000, 37, 0], [300, 27, 129], 64)])
+    (6, 2, 24, [3], [5], 16), (2, 2, 256, [63], [66], 64), (32, 8, 128, [1000, 37, 0], [300, 27, 129], 64),
+    (5, 5, 96, [130, 0], [131, 300], 32), (4, 1, 64, [31], [290], 16)])
 def test_attn_prefill_paged(dtype, nh, nkv, hd, starts, rows, page):
     """A step's rows that go on from tokens the cache holds (a prompt cut into steps): attention
     over the paged cache at absolute positions, several sequences with different starts (0
@@ -427,6 +464,31 @@ def test_gemv_rows_f32(ydt, M, N, K):
         assert torch.equal(alone[0], got[M - 1])
     assert not ops().gemv_rows_f32_fits(rnd(129, K).to(DEV), w.to(DEV))
     assert not ops().gemv_rows_f32_fits(x.to(DEV).to(torch.bfloat16), w.to(DEV))
+
+
+@pytest.mark.parametrize("ydt", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(129, 128, 16), (130, 33, 48), (200, 411, 80), (257, 129, 1008), (1, 5, 32),
+                                   (300, 1000, 4096), (2048, 130, 512)])
+def test_gemm_f32_mfma(ydt, M, N, K):
+    """The 32-bit path's product of many rows, on the matrix cores' float32 instruction: float32
+    accuracy (a product with operands rounded to a shorter type would miss this budget by two
+    orders), edges that are no multiple of the tile, and a row's result the same bits wherever
+    it stands in the batch."""
+    x, w = rnd(M, K, seed=1), rnd(N, K, seed=2)
+    assert ops().gemm_f32_mfma_fits(x.to(DEV), w.to(DEV))
+    got = ops().gemm_f32_mfma(x.to(DEV), w.to(DEV), ydt)
+    want = R.linear(x, w, torch.float64)
+    if ydt == torch.float32:
+        torch.testing.assert_close(got.double().cpu(), want, atol=2e-6 * math.sqrt(K) * 4, rtol=1e-5)
+    else:
+        close(got, want, ydt, scale=math.sqrt(K))
+    if ydt == torch.float32 and M > 2:
+        part = ops().gemm_f32_mfma(x[M // 2 + 1:].contiguous().to(DEV), w.to(DEV), ydt)
+        assert torch.equal(part, got[M // 2 + 1:])
+    if M > 128:
+        assert torch.equal(ops().linear(x.to(DEV), w.to(DEV), ydt), got)
+    assert not ops().gemm_f32_mfma_fits(rnd(M, K + 8).to(DEV), rnd(N, K + 8).to(DEV))
+    assert not ops().gemm_f32_mfma_fits(x.to(DEV).to(torch.bfloat16), w.to(DEV))
 
 
 def _decode_copy(w, mode="plain", **geometry):
