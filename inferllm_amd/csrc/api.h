@@ -47,6 +47,14 @@ int illm_gemm_generic(const void* X, int x_dt, const void* W, int w_dt, void* Y,
 int illm_gemm_f32_mfma(const float* X, const float* W, void* Y, int y_dt, int M, int N, int K,
                        void* stream);
 
+// The same product for M <= 128 rows of float32 X and W with K % 32 == 0, W read once, on the
+// matrix cores' float32 instruction with operands straight from memory.
+int illm_gemm_rows_f32_mfma(const float* X, const float* W, void* Y, int y_dt, int M, int N, int K,
+                            void* stream);
+// Tests: tiles of 16 rows of W a block of that kernel takes (1 or 2; 0: the library's choice).
+// The sums are the same bits either way.
+void illm_set_rows_f32_tiles(int tiles);
+
 // The same product for M <= 16 rows when X and W are float32 and K % 4 == 0: W is read once
 // (decoding on the 32-bit path); plain float32 multiply-adds.
 int illm_gemv_rows_f32(const float* X, const float* W, void* Y, int y_dt, int M, int N, int K,

@@ -203,6 +203,123 @@ extern "C" int illm_gemm_f32_mfma(const float* X, const float* W, void* Y, int y
 }
 
 
+// ---------------------------------------------------------------- up to 128 rows, float32
+// The same product for up to 128 float32 rows and K a multiple of 32, bound by reading W once:
+// MFMA 16x16x4 float32 with operands straight from memory.  A block of 8 waves takes 16 rows of
+// W; the waves take pieces of 32 k in turn (wave w pieces w, w + 8, ...: eight neighbouring
+// 128-byte segments of a row at a time).  Lane l reads 16 bytes at k = 4 (l / 16) + 16 q of row
+// l % 16, of W and of every 16 rows of X alike: element j of that load is the operand of an
+// MFMA whose four k are 4 g + j + 16 q, the same four for both operands, so nothing is
+// permuted.  The waves' sums are added through LDS in wave order: the order of a sum depends on
+// K only, not on the row's place or on the number of rows.
+typedef float f32x4v_t __attribute__((ext_vector_type(4)));
+
+template <int RT, int CT>                      // tiles of 16 rows of X, tiles of 16 rows of W
+__global__ void __launch_bounds__(512)
+gemm_rows_f32_mfma_kernel(const float* __restrict__ X, const float* __restrict__ W, void* __restrict__ Y,
+                          int y_dt, int M, int N, int K) {
+    __shared__ f32x4v_t part[8][RT * CT][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16 * CT;
+    const float* wsrc[CT];
+#pragma unroll
+    for (int c = 0; c < CT; ++c) wsrc[c] = W + (size_t)min(n0 + 16 * c + r16, N - 1) * K + 4 * g;
+    const float* xsrc[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) xsrc[t] = X + (size_t)min(16 * t + r16, M - 1) * K + 4 * g;
+    f32x4v_t acc[RT][CT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int c = 0; c < CT; ++c) acc[t][c] = (f32x4v_t){0.f, 0.f, 0.f, 0.f};
+    constexpr int U = RT * CT <= 2 ? 4 : (RT <= 4 ? 2 : 1);   // pieces asked for together
+    const int pieces = K / 32;
+    for (int p = wave; p < pieces; p += 8 * U) {
+        f32x4v_t wr[U][CT][2], xr[U][RT][2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k0 = 32 * min(p + 8 * u, pieces - 1);      // (past the end: a piece read again, not used)
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+#pragma unroll
+                for (int c = 0; c < CT; ++c)
+                    wr[u][c][q] = __builtin_nontemporal_load((const f32x4v_t*)(wsrc[c] + k0 + 16 * q));
+#pragma unroll
+                for (int t = 0; t < RT; ++t) xr[u][t][q] = *(const f32x4v_t*)(xsrc[t] + k0 + 16 * q);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (p + 8 * u < pieces) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int t = 0; t < RT; ++t)
+#pragma unroll
+                            for (int c = 0; c < CT; ++c)
+                                acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(wr[u][c][q][j], xr[u][t][q][j],
+                                                                                 acc[t][c], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int c = 0; c < CT; ++c) part[wave][t * CT + c][lane] = acc[t][c];
+    __syncthreads();
+    // acc[t][c][v]: n = n0 + 16 c + 4 g + v, m = 16 t + r16; a thread adds the eight waves' sums
+    for (int e = tid; e < RT * CT * 64; e += 512) {
+        const int tc = e >> 6, l = e & 63;
+        f32x4v_t sum = part[0][tc][l];
+#pragma unroll
+        for (int w = 1; w < 8; ++w) sum += part[w][tc][l];
+        const int m = 16 * (tc / CT) + (l & 15), n = n0 + 16 * (tc % CT) + 4 * (l >> 4);
+        if (m >= M) continue;
+        const size_t at = (size_t)m * N + n;
+        if (n + 3 < N && (N & 3) == 0 && y_dt == ILLM_F32) {
+            *(f32x4v_t*)((float*)Y + at) = sum;
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n + v < N) st_f(Y, y_dt, at + v, sum[v]);
+        }
+    }
+}
+
+static int g_rows_f32_tiles = 0;     // tests: W tiles a block (1 or 2); 0: the library's choice
+extern "C" void illm_set_rows_f32_tiles(int tiles) { g_rows_f32_tiles = tiles == 1 || tiles == 2 ? tiles : 0; }
+
+// float32 X [M <= 128, K] and W [N, K], K % 32 == 0; Y float32 or bfloat16.  Else ILLM_ERR_ARG.
+extern "C" int illm_gemm_rows_f32_mfma(const float* X, const float* W, void* Y, int y_dt, int M, int N,
+                                       int K, void* stream) {
+    if (M <= 0 || M > 128 || N <= 0 || K <= 0 || (K % 32) || !illm_dtype_ok(y_dt) || !X || !W || !Y)
+        return ILLM_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    // two tiles of W a block halve what the blocks read of X together: from 17 rows on, where
+    // that is most of the traffic, if there are still two blocks for every compute unit
+    // (measured at 64 rows: 22016 x 4096 263 -> 204 us, 12288 x 4096 the same, 4096 x 4096 49 -> 65)
+    const int rt = (M + 15) / 16;
+    const int ct = g_rows_f32_tiles ? g_rows_f32_tiles : (rt >= 2 && N >= 32 * 512 ? 2 : 1);
+    const dim3 grid((N + 16 * ct - 1) / (16 * ct)), block(512);
+#define ILLM_ROWS_F32(RT)                                                                             \
+    case RT:                                                                                          \
+        if (ct == 2)                                                                                  \
+            hipLaunchKernelGGL((gemm_rows_f32_mfma_kernel<RT, 2>), grid, block, 0, st, X, W, Y, y_dt, M, N, K); \
+        else                                                                                          \
+            hipLaunchKernelGGL((gemm_rows_f32_mfma_kernel<RT, 1>), grid, block, 0, st, X, W, Y, y_dt, M, N, K); \
+        break;
+    switch (rt) {
+        ILLM_ROWS_F32(1) ILLM_ROWS_F32(2) ILLM_ROWS_F32(3) ILLM_ROWS_F32(4)
+        ILLM_ROWS_F32(5) ILLM_ROWS_F32(6) ILLM_ROWS_F32(7) ILLM_ROWS_F32(8)
+    }
+#undef ILLM_ROWS_F32
+    return illm_launch_status();
+}
+
+
 // ---------------------------------------------------------------- few rows, float32
 // The same product for M <= 16 rows of float32 X and float32 W (decoding on the 32-bit path),
 // bound by reading W once: a block of 4 waves takes R = 64 / MR rows of W (MR = M rounded up to

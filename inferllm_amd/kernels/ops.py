@@ -330,7 +330,8 @@ def _operand(x):
 
 GEMV_F32_MAX_ROWS = 128    # up to here 16 rows at a time, W read once for each 16, beat the
                            # multiply-add tile, whose blocks each walk all of K (measured at the
-                           # 7B shape: a decode step of 64 rows 146 -> 45 ms)
+                           # 7B shape: a decode step of 64 rows 146 -> 45 ms); where K is a
+                           # multiple of 32 `gemm_rows_f32_mfma` takes these rows instead
 
 
 def gemv_rows_f32_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -351,6 +352,30 @@ def gemv_rows_f32(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> t
         rows = min(16, M - m0)
         _check(_lib().illm_gemv_rows_f32(_p(x[m0:m0 + rows]), _p(w), _p(y[m0:m0 + rows]), _code(y),
                                          rows, N, K, _stream()), "gemv_rows_f32")
+    return y
+
+
+ROWS_F32_MFMA_FROM = 9     # measured streaming over many matrices of the 7B shapes: up to 8 rows
+                           # `gemv_rows_f32` reads W at 4.5 to 5.5 TB/s against 3.2 to 4.0; at 16 rows
+                           # it is 2.4 to 2.9 against 3.1 to 3.4, at 64 rows 0.7 against 1.4 to 1.8
+
+
+def gemm_rows_f32_mfma_fits(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.float32 and w.dtype == torch.float32 and x.dim() == 2 and w.dim() == 2
+            and 1 <= x.shape[0] <= 128 and x.shape[1] % 32 == 0
+            and x.shape[1] == w.shape[1] and x.is_contiguous() and w.is_contiguous())
+
+
+def gemm_rows_f32_mfma(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [M <= 128, K] . w [N, K]^T, both float32, W read once, on the matrix cores' float32
+    instruction.  A row's sum does not depend on the other rows or on their number."""
+    _gpu(x, w)
+    _need(gemm_rows_f32_mfma_fits(x, w), "gemm_rows_f32_mfma: operands not taken")
+    M, K = x.shape
+    N = w.shape[0]
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    _check(_lib().illm_gemm_rows_f32_mfma(_p(x), _p(w), _p(y), _code(y), M, N, K, _stream()),
+           "gemm_rows_f32_mfma")
     return y
 
 
@@ -520,6 +545,8 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     if isinstance(w, Weight) and not (x.dtype == torch.bfloat16 and 1 <= x.shape[0] <= SKINNY_BEST_ROWS):
         w = w.plain                                      # only the few-rows kernel reads the copy
     if x.dtype == torch.float32 or w.dtype == torch.float32:
+        if x.shape[0] >= ROWS_F32_MFMA_FROM and gemm_rows_f32_mfma_fits(x, w):
+            return gemm_rows_f32_mfma(x, w, out_dtype)
         if gemv_rows_f32_fits(x, w):
             return gemv_rows_f32(x, w, out_dtype)
         if gemm_f32_mfma_fits(x, w):

@@ -453,17 +453,51 @@ def test_gemv_rows_f32(ydt, M, N, K):
     row's result is the same bits whatever rows stand beside it."""
     x, w = rnd(M, K, seed=1), rnd(N, K, seed=2)
     assert ops().gemv_rows_f32_fits(x.to(DEV), w.to(DEV))
-    got = ops().linear(x.to(DEV), w.to(DEV), ydt)
+    got = ops().gemv_rows_f32(x.to(DEV), w.to(DEV), ydt)
     want = R.linear(x, w, torch.float64)
     if ydt == torch.float32:
         torch.testing.assert_close(got.double().cpu(), want, atol=2e-6 * math.sqrt(K) * 4, rtol=1e-5)
     else:
         close(got, want, ydt, scale=math.sqrt(K))
     if ydt == torch.float32 and M > 1:
-        alone = ops().linear(x[M - 1:].contiguous().to(DEV), w.to(DEV), ydt)
+        alone = ops().gemv_rows_f32(x[M - 1:].contiguous().to(DEV), w.to(DEV), ydt)
         assert torch.equal(alone[0], got[M - 1])
+    if K % 32 or M < ops().ROWS_F32_MFMA_FROM:
+        assert torch.equal(ops().linear(x.to(DEV), w.to(DEV), ydt), got)
     assert not ops().gemv_rows_f32_fits(rnd(129, K).to(DEV), w.to(DEV))
     assert not ops().gemv_rows_f32_fits(x.to(DEV).to(torch.bfloat16), w.to(DEV))
+
+
+@pytest.mark.parametrize("ydt", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 100, 160), (16, 33, 992), (5, 320, 96), (3, 7, 32), (9, 11008, 4096),
+                                   (17, 100, 256), (64, 320, 96), (100, 33, 1024), (128, 4096, 512), (70, 16400, 64),
+                                   (33, 22016, 4096)])
+def test_gemm_rows_f32_mfma(ydt, M, N, K):
+    """The 32-bit path's product of up to 128 rows on the matrix cores' float32 instruction:
+    float32 accuracy, edges, one and two tiles of W a block with the same bits, and a row's result
+    the same bits whatever rows stand beside it."""
+    x, w = rnd(M, K, seed=1), rnd(N, K, seed=2)
+    assert ops().gemm_rows_f32_mfma_fits(x.to(DEV), w.to(DEV))
+    got = ops().gemm_rows_f32_mfma(x.to(DEV), w.to(DEV), ydt)
+    if M >= ops().ROWS_F32_MFMA_FROM:
+        assert torch.equal(ops().linear(x.to(DEV), w.to(DEV), ydt), got)
+    want = R.linear(x, w, torch.float64)
+    if ydt == torch.float32:
+        torch.testing.assert_close(got.double().cpu(), want, atol=2e-6 * math.sqrt(K) * 4, rtol=1e-5)
+    else:
+        close(got, want, ydt, scale=math.sqrt(K))
+    lib = ops()._lib()
+    try:
+        for tiles in (1, 2):
+            lib.illm_set_rows_f32_tiles(tiles)
+            assert torch.equal(ops().gemm_rows_f32_mfma(x.to(DEV), w.to(DEV), ydt), got)
+    finally:
+        lib.illm_set_rows_f32_tiles(0)
+    if M > 1:
+        alone = ops().gemm_rows_f32_mfma(x[M - 1:].contiguous().to(DEV), w.to(DEV), ydt)
+        assert torch.equal(alone[0], got[M - 1])
+    assert not ops().gemm_rows_f32_mfma_fits(rnd(129, K).to(DEV), w.to(DEV))
+    assert not ops().gemm_rows_f32_mfma_fits(rnd(M, K + 16).to(DEV), rnd(N, K + 16).to(DEV))
 
 
 @pytest.mark.parametrize("ydt", DTYPES)
