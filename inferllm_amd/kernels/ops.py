@@ -452,12 +452,15 @@ def linear_planes_fits(x, w) -> bool:
 def _cold_time(fn, reps: int = 5) -> float:
     """Median milliseconds of `fn` with the last-level cache flushed before every run: a decode
     step streams gigabytes between two uses of a matrix, so its products always run cold, and a
-    matrix of tens of megabytes timed back to back would be served from the cache."""
-    flush = torch.empty(1 << 28, dtype=torch.int16, device=torch.cuda.current_device())   # 512 MB
+    matrix of tens of megabytes timed back to back would be served from the cache.  The flush
+    reads: after a fill the cache is full of lines to be written back, which costs a kernel
+    whose loads allocate in it tens of microseconds that it does not pay in a step (measured
+    against streaming over many copies of a matrix, which the reading flush agrees with)."""
+    flush = torch.zeros(1 << 28, dtype=torch.int16, device=torch.cuda.current_device())   # 512 MB
     fn()
     times = []
     for _ in range(reps):
-        flush.zero_()
+        flush.sum()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
         fn()
