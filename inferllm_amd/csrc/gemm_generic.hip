@@ -323,7 +323,7 @@ extern "C" int illm_gemm_rows_f32_mfma(const float* X, const float* W, void* Y, 
 // ---------------------------------------------------------------- few rows, float32
 // The same product for M <= 16 rows of float32 X and float32 W (decoding on the 32-bit path),
 // bound by reading W once: a block of 4 waves takes R = 64 / MR rows of W (MR = M rounded up to
-// 4, 8 or 16), the waves split K in interleaved pieces of 256, a lane multiplies 4 consecutive k
+// 8 or 16), the waves split K in interleaved pieces of 256, a lane multiplies 4 consecutive k
 // of every W row with every X row (plain multiply-adds, float32), and the R * MR sums of a wave
 // are added over its lanes by a halving exchange that leaves sum number l in lane l.  The waves'
 // sums are added in wave order.  The order of a sum depends on K only, not on the row's place.
@@ -345,9 +345,9 @@ gemv_rows_f32_kernel(const float* __restrict__ X, const float* __restrict__ W, v
         for (int m = 0; m < MR; ++m) acc[r][m] = 0.f;
 
     for (int k = (wave * 64 + lane) * 4; k < K; k += 4 * 256) {      // K is a multiple of 4
-        float4 w[R];
+        f32x4v_t w[R];                                   // (W is used once: loads that do not stay in the caches)
 #pragma unroll
-        for (int r = 0; r < R; ++r) w[r] = *(const float4*)(wrow[r] + k);
+        for (int r = 0; r < R; ++r) w[r] = __builtin_nontemporal_load((const f32x4v_t*)(wrow[r] + k));
 #pragma unroll
         for (int m = 0; m < MR; ++m) {
             const float4 x = *(const float4*)(X + (size_t)min(m, M - 1) * K + k);
@@ -393,9 +393,9 @@ extern "C" int illm_gemv_rows_f32(const float* X, const float* W, void* Y, int y
                                   int K, void* stream) {
     if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K % 4) || !illm_dtype_ok(y_dt)) return ILLM_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    if (M <= 4)
-        hipLaunchKernelGGL(gemv_rows_f32_kernel<4>, dim3((N + 15) / 16), dim3(256), 0, st, X, W, Y, y_dt, M, N, K);
-    else if (M <= 8)
+    // (a block of 16 rows of W for up to 4 rows of X was slower than this one of 8 at three of
+    // the four 7B shapes: 72 against 60 us for 22016 x 4096, 34 against 36 for 4096 x 11008)
+    if (M <= 8)
         hipLaunchKernelGGL(gemv_rows_f32_kernel<8>, dim3((N + 7) / 8), dim3(256), 0, st, X, W, Y, y_dt, M, N, K);
     else
         hipLaunchKernelGGL(gemv_rows_f32_kernel<16>, dim3((N + 3) / 4), dim3(256), 0, st, X, W, Y, y_dt, M, N, K);
