@@ -66,7 +66,7 @@ int illm_attn_prefill_generic(const void* qkv, void* out, int dt, const int32_t*
                               int n_seqs, int max_len, int nh, int nkv, int hd, float scale,
                               int window, void* stream);
 
-// The same on the matrix cores for bfloat16 and head_dim % 32 == 0 (else ILLM_ERR_ARG).
+// The same on the matrix cores for bfloat16 and head_dim % 16 == 0 (else ILLM_ERR_ARG).
 int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens, int n_seqs,
                            int max_len, int nh, int nkv, int hd, float scale, int window,
                            void* stream);

@@ -1,5 +1,6 @@
 // Causal attention of whole prompts for bfloat16 on the matrix cores (MFMA 32x32x16),
-// head sizes that are multiples of 32 up to 256, any number of heads and groups,
+// head sizes that are multiples of 16 up to 256 (the last block of 32 dims of the second
+// product is half used when the size is no multiple of 32), any number of heads and groups,
 // ragged batches.
 //
 // A block of 4 waves takes 128 consecutive query rows of one (sequence, head); a
@@ -57,9 +58,10 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     constexpr int KLD = HD + 8;        // K tile row stride: 16 bytes of padding
     constexpr int VLD = PF_BN + 4;     // V^T row stride
     constexpr int KS = HD / 16;        // k-steps of the first product
-    constexpr int DB = HD / 32;        // 32-row blocks of O^T
+    constexpr int DB = (HD + 31) / 32; // 32-row blocks of O^T (the last one half used when HD % 32 == 16)
+    constexpr int CH = HD / 8;         // 16-byte chunks of a row
     __shared__ __attribute__((aligned(16))) bf16_t ks[PF_BN * KLD];
-    __shared__ __attribute__((aligned(16))) bf16_t vts[HD * VLD];
+    __shared__ __attribute__((aligned(16))) bf16_t vts[DB * 32 * VLD];
 
     // XCD x takes the (sequence, head) pairs [x * hb_per_xcd, (x + 1) * hb_per_xcd); within
     // it, slots run over those pairs first and over query blocks, last block first, second
@@ -87,6 +89,9 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     const int qc = q < len ? q : len - 1;
     const int qp = pos0 + q;                            // its position
 
+    if constexpr (HD % 32 != 0) {       // rows of V^T beyond the head size: operands of sums nobody stores
+        for (int e = threadIdx.x; e < (DB * 32 - HD) * VLD; e += 256) vts[HD * VLD + e] = 0;
+    }
     uint4 qf[KS];
     {
         const bf16_t* qp = qkv + (size_t)(start + qc) * rowlen + (size_t)h * HD + half * 8;
@@ -106,7 +111,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
     const int wk_end = min(total, pos0 + q_row0 + 32);              // this wave's last key + 1
     const int wk_begin = window > 0 ? max(0, pos0 + q_row0 - window + 1) : 0;
 
-    constexpr int NLD = (PF_BN * HD / 8) / 256;     // 16-byte pieces of K (and of V) per thread
+    constexpr int NLD = (PF_BN * CH + 255) / 256;   // 16-byte pieces of K (and of V) per thread
     uint4 kpre[NLD], vpre[NLD];
     auto fetch = [&](int k0) {
         size_t page_base = 0;                           // PAGED: the tile's page, this kv head
@@ -120,7 +125,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
         for (int it = 0; it < NLD; ++it) {
             const int u = tid + it * 256;
             const int key = ((u >> 6) & 3) * 16 + (u & 15);
-            const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
+            const int ch = min((u >> 8) * 4 + ((u >> 4) & 3), CH - 1);   // (HD % 32 == 16: the last round's upper half loads a chunk again)
             const int krow = min(k0 + key, total - 1);
             if (PAGED) {
                 const size_t at = (page_base + krow % pg.page_size) * HD + ch * 8;
@@ -142,6 +147,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
             const int u = tid + it * 256;
             const int key = ((u >> 6) & 3) * 16 + (u & 15);
             const int ch = (u >> 8) * 4 + ((u >> 4) & 3);
+            if (HD % 32 != 0 && ch >= CH) continue;
             const uint4 kv = kpre[it], vv = vpre[it];
             *(uint4*)(ks + key * KLD + ch * 8) = kv;
             bf16_t* vd = vts + (ch * 8) * VLD + key;
@@ -247,6 +253,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ou
         for (int d = 0; d < DB; ++d)
 #pragma unroll
             for (int b4 = 0; b4 < 4; ++b4) {
+                if (d * 32 + 8 * b4 >= HD) continue;
                 uint2 v;
                 v.x = pack_bf16x2(o[d][4 * b4 + 0] * inv, o[d][4 * b4 + 1] * inv);
                 v.y = pack_bf16x2(o[d][4 * b4 + 2] * inv, o[d][4 * b4 + 3] * inv);
@@ -547,7 +554,7 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
     const long long hb_per_xcd = (n_hb + 7) / 8;
     const long long blocks = 8 * hb_per_xcd * n_qblk;
     if (blocks > 0x7fffffffLL) return ILLM_ERR_ARG;
-    if constexpr (HD <= 128) if (!pg) {
+    if constexpr (HD <= 128 && HD % 32 == 0) if (!pg) {
         // measured at 32 heads: head size 128, 2,048 keys 81 -> 76 us, 4,096 keys 236 -> 214; head
         // size 64 and sequences of 512 lose a tenth (a tile more of set-up before the first product)
         // measured at 32 heads of size 128: 2,048 keys 81 -> 71 us, 4,096 keys 228 -> 193, 8,192
@@ -578,12 +585,12 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
     return illm_launch_status();
 }
 
-// Takes bfloat16 and head_dim in {32, 64, 96, 128, 160, 192, 224, 256}; else ILLM_ERR_ARG.
+// Takes bfloat16 and a head_dim that is a multiple of 16 up to 256; else ILLM_ERR_ARG.
 extern "C" int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t* cu_seqlens,
                                       int n_seqs, int max_len, int nh, int nkv, int hd,
                                       float scale, int window, void* stream) {
     if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
-        hd % 32)
+        hd % 16)
         return ILLM_ERR_ARG;
     if (n_seqs == 0 || max_len == 0) return ILLM_OK;
     hipStream_t st = (hipStream_t)stream;
@@ -595,6 +602,14 @@ extern "C" int illm_attn_prefill_bf16(const void* qkv, void* out, const int32_t*
         case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
         case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
         case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 16: return launch_prefill<16>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 48: return launch_prefill<48>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 80: return launch_prefill<80>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 112: return launch_prefill<112>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 144: return launch_prefill<144>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 176: return launch_prefill<176>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 208: return launch_prefill<208>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
+        case 240: return launch_prefill<240>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
         default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st);
     }
 }
@@ -609,7 +624,7 @@ extern "C" int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const in
                                             int page_size, int ring, int n_seqs, int max_len, int nh,
                                             int nkv, int hd, float scale, int window, void* stream) {
     if (n_seqs < 0 || max_len < 0 || nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || hd > 256 ||
-        hd % 32 || !seq_slot || !seq_start || !kcache || !vcache || !page_table ||
+        hd % 16 || !seq_slot || !seq_start || !kcache || !vcache || !page_table ||
         table_stride <= 0 || page_size <= 0 || page_size % PF_BN)
         return ILLM_ERR_ARG;
     if (n_seqs == 0 || max_len == 0) return ILLM_OK;
@@ -624,6 +639,14 @@ extern "C" int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const in
         case 160: return launch_prefill<160>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
         case 192: return launch_prefill<192>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
         case 224: return launch_prefill<224>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 16: return launch_prefill<16>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 48: return launch_prefill<48>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 80: return launch_prefill<80>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 112: return launch_prefill<112>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 144: return launch_prefill<144>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 176: return launch_prefill<176>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 208: return launch_prefill<208>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
+        case 240: return launch_prefill<240>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
         default: return launch_prefill<256>(qkv, out, cu_seqlens, n_seqs, max_len, nh, nkv, scale, window, st, &pg);
     }
 }

@@ -878,7 +878,7 @@ def attn_prefill(qkv: torch.Tensor, cu_seqlens: torch.Tensor, n_seqs: int, max_l
     _need(qkv.dim() == 2 and qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_prefill: packed qkv rows")
     _need(nh % nkv == 0, "attn_prefill: heads must be a multiple of kv heads")
     out = torch.empty((T, nh * hd), dtype=qkv.dtype, device=qkv.device)
-    if qkv.dtype == torch.bfloat16 and hd % 32 == 0:
+    if qkv.dtype == torch.bfloat16 and hd % 16 == 0:
         _check(_lib().illm_attn_prefill_bf16(
             _p(qkv), _p(out), _p(cu_seqlens), n_seqs, max_len, nh, nkv, hd,
             ctypes.c_float(scale), window, _stream()), f"attn_prefill_bf16 (head_dim {hd})")
@@ -908,7 +908,7 @@ def attn_prefill_paged(qkv: torch.Tensor, cu_seqlens: torch.Tensor, seq_slot: to
           "attn_prefill_paged: cache shape or dtype")
     _need(qkv.shape[1] == (nh + 2 * nkv) * hd, "attn_prefill_paged: packed qkv rows")
     out = torch.empty((T, nh * hd), dtype=qkv.dtype, device=qkv.device)
-    if qkv.dtype == torch.bfloat16 and hd % 32 == 0 and page_size % 64 == 0:
+    if qkv.dtype == torch.bfloat16 and hd % 16 == 0 and page_size % 64 == 0:
         _check(_lib().illm_attn_prefill_paged_bf16(
             _p(qkv), _p(out), _p(cu_seqlens), _p(seq_slot), _p(seq_start), _p(kcache), _p(vcache),
             _p(page_table), page_table.shape[1], page_size, ring, n_seqs, max_len, nh, nkv, hd,

@@ -206,6 +206,9 @@ def test_attn_prefill(dtype, nh, nkv, hd, lens, window):
 @pytest.mark.parametrize("nh,nkv,hd,lens,window", [
     (4, 4, 128, [300, 129, 128, 1], 0), (8, 1, 64, [257, 64], 0), (3, 3, 96, [200], 0), (6, 2, 32, [127, 130], 0),
     (2, 1, 160, [70], 0), (4, 2, 128, [400], 100), (2, 2, 64, [333, 5], 64), (5, 5, 224, [66], 0), (2, 2, 192, [129], 7),
+    # head sizes that are no multiple of 32: the last block of dims is half used
+    (4, 2, 80, [300, 129, 1], 0), (3, 1, 16, [200, 65], 0), (2, 2, 48, [333], 40), (6, 3, 112, [257], 0),
+    (2, 1, 144, [130], 0), (1, 1, 240, [70, 3], 0), (2, 2, 176, [129], 9), (2, 1, 208, [64], 0),
     # more blocks than the chip holds at once (heaviest first, not paired), and a long sequence
     (32, 8, 128, [600, 130, 577, 64], 0), (2, 1, 128, [2500, 40], 0)])
 def test_attn_prefill_mfma(nh, nkv, hd, lens, window):
@@ -267,7 +270,8 @@ def test_attn_prefill_f32_finds_one_far_key():
 @pytest.mark.parametrize("nh,nkv,hd,starts,rows,page", [
     (4, 2, 32, [0, 70, 5], [40, 30, 1], 64), (8, 8, 128, [200, 0], [130, 64], 64), (3, 1, 48, [17, 64], [9, 200], 64),
     (6, 2, 24, [3], [5], 16), (2, 2, 256, [63], [66], 64), (32, 8, 128, [1000, 37, 0], [300, 27, 129], 64),
-    (5, 5, 96, [130, 0], [131, 300], 32), (4, 1, 64, [31], [290], 16)])
+    (5, 5, 96, [130, 0], [131, 300], 32), (4, 1, 64, [31], [290], 16),
+    (4, 2, 80, [70, 0], [200, 130], 64), (2, 1, 16, [5], [300], 64), (3, 3, 112, [129], [64], 128), (2, 1, 240, [64], [70], 64)])
 def test_attn_prefill_paged(dtype, nh, nkv, hd, starts, rows, page):
     """A step's rows that go on from tokens the cache holds (a prompt cut into steps): attention
     over the paged cache at absolute positions, several sequences with different starts (0
