@@ -207,8 +207,11 @@ int illm_qkv_rope_store_skinny(const void* X, const void* W, const void* Wt, voi
                                int nh, int nkv, int hd, const float* ssq, int parts, float eps,
                                int waves_wanted, void* stream);
 
-// out[b] = index of the largest logit of row b (lowest index on ties).
-int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream);
+// out[b] = index of the largest logit of row b (lowest index on ties).  A row is cut into
+// `parts` (1 to 64) that blocks of their own take; scratch: 2 x B x parts 32-bit words (may be
+// null when parts == 1).
+int illm_argmax(const float* logits, int32_t* out, void* scratch, int B, int V, int parts,
+                void* stream);
 
 // Temperature / top-k / top-p / repeat-penalty sampling, one draw per row.
 // scratch: float32 [2][B][V].  last_tokens: [B][n_last] (-1 = empty) or null.

@@ -67,43 +67,6 @@ __device__ __forceinline__ T block_exclusive_scan(T v, T* red, T* total) {
     return before + inc - v;
 }
 
-// ---------------------------------------------------------------- argmax
-__global__ void __launch_bounds__(SB)
-argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int V) {
-    __shared__ float bv[SB / ILLM_WAVE];
-    __shared__ int bi[SB / ILLM_WAVE];
-    const float* row = logits + (size_t)blockIdx.x * V;
-    float best = -INFINITY;
-    int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += SB) {
-        const float v = row[i];
-        if (v > best || (v == best && i < idx) || idx == 0x7fffffff) {
-            if (!(v != v)) { best = v; idx = i; }   // NaN never wins
-        }
-    }
-#pragma unroll
-    for (int o = ILLM_WAVE / 2; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(best, o, ILLM_WAVE);
-        const int oi = __shfl_xor(idx, o, ILLM_WAVE);
-        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
-    }
-    const int lane = threadIdx.x & (ILLM_WAVE - 1), w = threadIdx.x / ILLM_WAVE;
-    if (lane == 0) { bv[w] = best; bi[w] = idx; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int i = 1; i < SB / ILLM_WAVE; ++i)
-            if (bv[i] > best || (bv[i] == best && bi[i] < idx)) { best = bv[i]; idx = bi[i]; }
-        out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
-    }
-}
-
-extern "C" int illm_argmax(const float* logits, int32_t* out, int B, int V, void* stream) {
-    if (B < 0 || V <= 0) return ILLM_ERR_ARG;
-    if (B == 0) return ILLM_OK;
-    hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits, out, V);
-    return illm_launch_status();
-}
-
 // Walks of a row by one block wait for each load in turn unless several are asked for at once:
 // these bring eight values at a time, all loads issued before the first is used.
 template <typename F>
@@ -133,6 +96,82 @@ __device__ __forceinline__ void each_in_order8(const float* a, int lo, int hi, F
         for (int u = 0; u < 8; ++u)
             if (base + u < hi) f(base + u, v[u]);
     }
+}
+
+// ---------------------------------------------------------------- argmax
+// The lowest id among the largest values of a row; NaN never wins, a row of nothing else gives 0.
+// A row is cut into gridDim.x parts (a block each, eight loads in flight a thread) that leave
+// (value, id) pairs; the second kernel takes the best of a row's parts.  With one part the
+// first kernel writes the id itself.
+__device__ __forceinline__ void argmax_take(float& best, int& idx, float v, int i) {
+    if (v > best || (v == best && i < idx) || idx == 0x7fffffff) {
+        if (!(v != v)) { best = v; idx = i; }
+    }
+}
+
+__global__ void __launch_bounds__(SB)
+argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, float* __restrict__ part_v,
+              int32_t* __restrict__ part_i, int V, int chunk) {
+    __shared__ float bv[SB / ILLM_WAVE];
+    __shared__ int bi[SB / ILLM_WAVE];
+    const int lo = blockIdx.x * chunk, n = min(chunk, V - lo);
+    const float* row = logits + (size_t)blockIdx.y * V + lo;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    each_strided8(row, n, threadIdx.x, [&](int i, float v) { argmax_take(best, idx, v, lo + i); });
+#pragma unroll
+    for (int o = ILLM_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, ILLM_WAVE);
+        const int oi = __shfl_xor(idx, o, ILLM_WAVE);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int lane = threadIdx.x & (ILLM_WAVE - 1), w = threadIdx.x / ILLM_WAVE;
+    if (lane == 0) { bv[w] = best; bi[w] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < SB / ILLM_WAVE; ++i)
+            if (bv[i] > best || (bv[i] == best && bi[i] < idx)) { best = bv[i]; idx = bi[i]; }
+        if (gridDim.x == 1) {
+            out[blockIdx.y] = idx == 0x7fffffff ? 0 : idx;
+        } else {
+            part_v[blockIdx.y * gridDim.x + blockIdx.x] = best;
+            part_i[blockIdx.y * gridDim.x + blockIdx.x] = idx;
+        }
+    }
+}
+
+// one wave a row over its parts (at most 64)
+__global__ void __launch_bounds__(ILLM_WAVE)
+argmax_parts_kernel(const float* __restrict__ part_v, const int32_t* __restrict__ part_i,
+                    int32_t* __restrict__ out, int parts) {
+    const int lane = threadIdx.x;
+    float best = lane < parts ? part_v[blockIdx.x * parts + lane] : -INFINITY;
+    int idx = lane < parts ? part_i[blockIdx.x * parts + lane] : 0x7fffffff;
+#pragma unroll
+    for (int o = ILLM_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, ILLM_WAVE);
+        const int oi = __shfl_xor(idx, o, ILLM_WAVE);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    if (lane == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+}
+
+// scratch: parts x B floats and as many int32 behind them (parts > 1), parts <= 64.
+extern "C" int illm_argmax(const float* logits, int32_t* out, void* scratch, int B, int V, int parts,
+                           void* stream) {
+    if (B < 0 || V <= 0 || parts < 1 || parts > ILLM_WAVE || (parts > 1 && !scratch) || B > 65535)
+        return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    const int chunk = (V + parts - 1) / parts;
+    parts = (V + chunk - 1) / chunk;                       // (no part without values)
+    float* pv = (float*)scratch;
+    int32_t* pi = (int32_t*)scratch + (size_t)B * parts;
+    hipLaunchKernelGGL(argmax_kernel, dim3(parts, B), dim3(SB), 0, (hipStream_t)stream, logits, out, pv, pi,
+                       V, chunk);
+    if (parts > 1)
+        hipLaunchKernelGGL(argmax_parts_kernel, dim3(B), dim3(ILLM_WAVE), 0, (hipStream_t)stream, pv, pi,
+                           out, parts);
+    return illm_launch_status();
 }
 
 // ---------------------------------------------------------------- sampler

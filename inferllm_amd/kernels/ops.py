@@ -974,7 +974,11 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "argmax: float32 [B, V]")
     B, V = logits.shape
     out = torch.empty((B,), dtype=torch.int32, device=logits.device)
-    _check(_lib().illm_argmax(_p(logits), _p(out), B, V, _stream()), "argmax")
+    # a row in parts of 2,048 ids or more, about 512 blocks in all: one block a row walks a long
+    # row alone (128,256 ids: 56 us whatever the batch)
+    parts = max(1, min(64, V // 2048, 512 // max(B, 1)))
+    scratch = torch.empty((2, B, parts), dtype=torch.int32, device=logits.device) if parts > 1 else None
+    _check(_lib().illm_argmax(_p(logits), _p(out), _p(scratch), B, V, parts, _stream()), "argmax")
     return out
 
 

@@ -783,7 +783,8 @@ def test_attn_decode_finds_one_far_key(dtype):
         close(got[kvh * (nh // nkv)], vc[pg, kvh, r], dtype)
 
 
-@pytest.mark.parametrize("B,V", [(1, 256), (3, 320), (2, 32000), (64, 411), (1, 128256)])
+@pytest.mark.parametrize("B,V", [(1, 256), (3, 320), (2, 32000), (64, 411), (1, 128256), (5, 128256), (64, 32000),
+                                 (9, 4099)])
 def test_argmax(B, V):
     logits = rnd(B, V, seed=4)
     logits[0, V - 1] = 50.0
@@ -792,6 +793,14 @@ def test_argmax(B, V):
     got = ops().argmax(logits.to(DEV)).cpu()
     assert got.tolist() == R.argmax(logits).tolist()
     assert got[0] == V - 1 and (B == 1 or got[1] == 3)
+    # ties across the parts a long row is cut into, a NaN above everything, a row of NaN alone
+    logits[0, V - 1] = 0.0
+    logits[0, 5] = 70.0; logits[0, V - 2] = 70.0; logits[0, V // 2] = float("nan")
+    if B > 2:
+        logits[2] = float("nan")
+    got = ops().argmax(logits.to(DEV)).cpu()
+    assert got[0] == 5 and (B <= 2 or got[2] == 0)
+    assert got.tolist()[3:] == R.argmax(logits).tolist()[3:]
 
 
 def interval_ok(logits_row, token, u, temperature, top_k, top_p, penalty, last):
