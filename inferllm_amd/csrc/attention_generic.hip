@@ -363,15 +363,17 @@ extern "C" int illm_attn_prefill_paged_generic(const void* qkv, void* out, int d
 // scores are summed over the wave together, each step handing half of them to the partner lane.
 // The waves' (sums, max, weight) are combined in wave order at the end; each block leaves
 // (acc[hd], max, sum) in `partial`.  Plain float32 arithmetic and expf.
+// A wave asks for the keys and the values of its next eight keys together, before it works on
+// the eight it has: one trip to memory a round instead of two, and that one beside the arithmetic.
+template <int DT, int DL>                  // storage type; dims a lane holds (head sizes up to 64 DL)
 __global__ void __launch_bounds__(256)
-attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __restrict__ kcache,
+attn_decode_generic_kernel(const void* __restrict__ qkv, const void* __restrict__ kcache,
                            const void* __restrict__ vcache,
                            const int32_t* __restrict__ page_table, int table_stride,
                            int page_size, int ring, const int32_t* __restrict__ seq_slot,
                            const int32_t* __restrict__ seq_len, float* __restrict__ partial,
                            int nsplit, int nh, int nkv, int hd, float scale, int window) {
     constexpr int KU = 8;                  // keys a wave takes at a time
-    constexpr int DL = 4;                  // dims a lane holds (head sizes up to 256)
     __shared__ float wave_acc[4][256];
     __shared__ float wave_ml[4][2];
     const int h = blockIdx.x, b = blockIdx.y, sp = blockIdx.z;
@@ -394,23 +396,30 @@ attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __r
     for (int i = 0; i < DL; ++i) {
         const int d = lane + 64 * i;
         dim[i] = d < hd ? d : 0;
-        q[i] = d < hd ? ld_f(qkv, dt, (size_t)b * rowlen + (size_t)h * hd + d) : 0.f;
+        q[i] = d < hd ? ld_f(qkv, DT, (size_t)b * rowlen + (size_t)h * hd + d) : 0.f;
         acc[i] = 0.f;
     }
     float m = NEG_INF, l = 0.f;
-    for (int k0 = k_lo + wave * KU; k0 < k_hi; k0 += 4 * KU) {
-        // keys beyond the range read its last key again (an existing row) and get no weight
-        size_t off[KU];
+    // keys beyond the range read its last key again (an existing row) and get no weight
+    auto load = [&](int k0, float (&kk)[KU][DL], float (&vv)[KU][DL]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < KU; ++j)
-            off[j] = cache_row_offset(page_table, table_stride, slot, min(k0 + j, k_hi - 1),
-                                      page_size, ring, nkv, kvh, hd);
+        for (int j = 0; j < KU; ++j) {
+            const size_t off = cache_row_offset(page_table, table_stride, slot, min(k0 + j, k_hi - 1),
+                                                page_size, ring, nkv, kvh, hd);
+#pragma unroll
+            for (int i = 0; i < DL; ++i) {
+                kk[j][i] = ld_f(kcache, DT, off + dim[i]);
+                vv[j][i] = ld_f(vcache, DT, off + dim[i]);
+            }
+        }
+    };
+    auto work = [&](int k0, const float (&kk)[KU][DL], const float (&vv)[KU][DL]) __attribute__((always_inline)) {
         float part[KU];
 #pragma unroll
         for (int j = 0; j < KU; ++j) {
             float a = 0.f;
 #pragma unroll
-            for (int i = 0; i < DL; ++i) a = fmaf(q[i], ld_f(kcache, dt, off[j] + dim[i]), a);
+            for (int i = 0; i < DL; ++i) a = fmaf(q[i], kk[j][i], a);
             part[j] = a;
         }
         // eight sums over 64 lanes: three steps that halve what a lane keeps (the sums whose
@@ -452,8 +461,23 @@ attn_decode_generic_kernel(const void* __restrict__ qkv, int dt, const void* __r
         for (int i = 0; i < DL; ++i) {
             float a = acc[i] * alpha;
 #pragma unroll
-            for (int j = 0; j < KU; ++j) a = fmaf(pv[j], ld_f(vcache, dt, off[j] + dim[i]), a);
+            for (int j = 0; j < KU; ++j) a = fmaf(pv[j], vv[j][i], a);
             acc[i] = a;
+        }
+    };
+    int k0 = k_lo + wave * KU;
+    if (k0 < k_hi) {                                   // (else the wave has no key: k_hi - 1 may not be a row)
+        float k_a[KU][DL], v_a[KU][DL], k_b[KU][DL], v_b[KU][DL];
+        load(k0, k_a, v_a);
+        while (true) {
+            load(k0 + 4 * KU, k_b, v_b);               // (past the range: its last key again, not used)
+            work(k0, k_a, v_a);
+            k0 += 4 * KU;
+            if (k0 >= k_hi) break;
+            load(k0 + 4 * KU, k_a, v_a);
+            work(k0, k_b, v_b);
+            k0 += 4 * KU;
+            if (k0 >= k_hi) break;
         }
     }
     // the waves' results, combined in wave order
@@ -517,10 +541,21 @@ extern "C" int illm_attn_decode_generic(const void* qkv, void* out, int dt, cons
         nsplit <= 0 || nsplit > 65535 || B > 65535 || page_size <= 0 || table_stride <= 0)
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
-    hipLaunchKernelGGL(attn_decode_generic_kernel, dim3(nh, B, nsplit), dim3(256), 0,
-                       (hipStream_t)stream, qkv, dt, kcache, vcache, page_table, table_stride,
-                       page_size, ring, seq_slot, seq_len, partial, nsplit, nh, nkv, hd, scale,
-                       window);
+#define ILLM_DECODE_GENERIC(DT, DL)                                                                   \
+    hipLaunchKernelGGL((attn_decode_generic_kernel<DT, DL>), dim3(nh, B, nsplit), dim3(256), 0,       \
+                       (hipStream_t)stream, qkv, kcache, vcache, page_table, table_stride, page_size, \
+                       ring, seq_slot, seq_len, partial, nsplit, nh, nkv, hd, scale, window)
+    const int dl = (hd + 63) / 64;
+    if (dt == ILLM_F32) {
+        if (dl == 1) ILLM_DECODE_GENERIC(ILLM_F32, 1);
+        else if (dl == 2) ILLM_DECODE_GENERIC(ILLM_F32, 2);
+        else ILLM_DECODE_GENERIC(ILLM_F32, 4);
+    } else {
+        if (dl == 1) ILLM_DECODE_GENERIC(ILLM_BF16, 1);
+        else if (dl == 2) ILLM_DECODE_GENERIC(ILLM_BF16, 2);
+        else ILLM_DECODE_GENERIC(ILLM_BF16, 4);
+    }
+#undef ILLM_DECODE_GENERIC
     hipLaunchKernelGGL(attn_decode_merge_kernel, dim3(nh, B), dim3(64), 0, (hipStream_t)stream,
                        (const float*)partial, out, dt, nsplit, nh, hd);
     return illm_launch_status();
