@@ -159,7 +159,10 @@ int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y,
 int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M, int N, int K,
                        int splits, void* stream);
 int illm_gemm_mid_splits(int N, int K);
-void illm_set_mid_tiles_per_wave(int n);      // tuning: 1 or 2 (0: by the number of tiles)
+void illm_set_mid_tiles_per_wave(int n);
+// Tuning and tests: rows of X a launch of that kernel takes, 64 or 128 (default); W is read once
+// a launch.
+void illm_set_mid_rows_a_launch(int rows);      // tuning: 1 or 2 (0: by the number of tiles)
 
 // Tuning and tests: 0 switches off the variant of the residual-adding product in which, for K up
 // to 4096 and at most 512 tiles, 8 waves each take their whole share of K at once (default 1).

@@ -152,6 +152,9 @@ static const int MID_BLOCKS_WANTED = 512;
 static int MID_TILES_PER_WAVE = 0;       // 0: by the number of tiles; 1 or 2: forced (tuning)
 extern "C" void illm_set_mid_tiles_per_wave(int n) { MID_TILES_PER_WAVE = (n == 1 || n == 2) ? n : 0; }
 
+static int MID_ROWS_A_LAUNCH = 128;      // tuning and tests: 64 or 128 rows of X a launch
+extern "C" void illm_set_mid_rows_a_launch(int rows) { MID_ROWS_A_LAUNCH = rows == 64 ? 64 : 128; }
+
 static int mid_ntb(int N) {
     return MID_TILES_PER_WAVE ? MID_TILES_PER_WAVE : ((N + 15) / 16 >= 512 ? 2 : 1);
 }
@@ -188,8 +191,9 @@ extern "C" int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_
     const int ntb = mid_ntb(N);
     const size_t y_elem = (splits > 1 || y_dt == ILLM_F32) ? 4 : 2;
     const size_t plane_stride = (size_t)M * N;
-    for (int m0 = 0; m0 < M; m0 += 64) {
-        const int rows = M - m0 < 64 ? M - m0 : 64;
+    const int a_launch = MID_ROWS_A_LAUNCH;
+    for (int m0 = 0; m0 < M; m0 += a_launch) {
+        const int rows = M - m0 < a_launch ? M - m0 : a_launch;
         const int mt = (rows + 15) / 16;
         const bf16_t* x = (const bf16_t*)X + (size_t)m0 * K;
         void* y = (char*)Y + (size_t)m0 * N * y_elem;
@@ -201,6 +205,7 @@ extern "C" int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_
             launched = true;                                                                  \
         }
         GO(1, 1) GO(2, 1) GO(3, 1) GO(4, 1) GO(1, 2) GO(2, 2) GO(3, 2) GO(4, 2)
+        GO(5, 1) GO(6, 1) GO(7, 1) GO(8, 1) GO(5, 2) GO(6, 2) GO(7, 2) GO(8, 2)
 #undef GO
         if (!launched) return ILLM_ERR_ARG;
         const int rc = illm_launch_status();

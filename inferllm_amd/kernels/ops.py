@@ -416,12 +416,11 @@ def linear_add(x: torch.Tensor, w, into: torch.Tensor, norm=None,
     return NormedRows(into, weight, eps, act_dtype, xb, ssq)
 
 
-MID_MAX_ROWS = 128       # beyond 64 rows the kernel runs once per 64 (the vendor GEMM reads the
-                         # thin matrices at 1.6 TB/s at 128 rows: 58.6 us for the 7B down projection)
+MID_MAX_ROWS = 128       # rows a launch of the kernel takes (the vendor GEMM reads the thin matrices
+                         # at 1.6 TB/s at 128 rows: 58.6 us for the 7B down projection)
 MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the norm that adds the
                          # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
                          # K >= 2 N (the down projection) and the same time when K = N
-PLANES_TWICE_MIN_ROWS = 112
 PLANES_MIN_ELEMENTS = 1 << 22   # smaller matrices are not measured (both ways take a few
                                 # microseconds and the clock would decide): no planes below 17 rows
 
@@ -441,12 +440,13 @@ def current_plan() -> Plan:
 
 def linear_planes_fits(x, w) -> bool:
     """Whether `linear_planes` takes these operands: up to 128 bfloat16 rows and a matrix with a
-    decode copy in plain tile order that has few rows for its length (K >= 2 N)."""
+    decode copy in plain tile order that has few rows for its length (K >= 2 N; from 65 rows on
+    K >= N, where the vendor GEMM is at its worst)."""
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == "plain"
             and isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and x.dim() == 2
             and 1 <= x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.plain.shape[1]
             and w.plain.shape[0] % 4 == 0 and w.plain.shape[0] <= MID_MAX_COLS
-            and w.plain.shape[1] >= 2 * w.plain.shape[0])
+            and w.plain.shape[1] >= (2 if x.shape[0] <= 64 else 1) * w.plain.shape[0])
 
 
 _flush: Dict[int, torch.Tensor] = {}
@@ -514,12 +514,10 @@ def linear_planes_pays(x, w) -> bool:
     16 rows, the 70B's 105 against 77, a 5120 x 13824 one 34 against 30 at 4 rows): by the
     plan's table; a plan that measures times a shape it lacks once, outside graph capture."""
     rows = x.shape[0]
-    if rows > 64:
-        # two launches of the kernel, W read twice: that beats the vendor GEMM when the second
-        # is nearly full (128 rows, the bucket of 65 to 128 sequences: 50 against 63 us for the
-        # 7B down projection, 164 against 205 for the 70B one) and loses at 80 rows
-        return rows >= PLANES_TWICE_MIN_ROWS
     if rows > SKINNY_BEST_ROWS:
+        # (65 to 128 rows, one launch, product and the norm that adds its planes against the
+        # vendor GEMM and its norm: the 7B down projection 28 to 33 us against 38 to 64, the 70B
+        # one 86 to 101 against 134 to 221, 4096 x 4096 18 to 22 against 20 to 29)
         return True
     key = tuple(w.plain.shape)
     first = _plan.planes_from.get(key)

@@ -717,10 +717,12 @@ def _plain_copy(w):
                                           (50, 84, 1184, 5), (48, 20, 64, 1), (31, 72, 352, 3),
                                           (64, 36, 2048, 16), (20, 8192, 16384, 0),
                                           (1, 40, 96, 0), (7, 100, 224, 2), (16, 4096, 11008, 0),
-                                          (65, 40, 96, 0), (100, 84, 1184, 4), (128, 4096, 11008, 0)])
+                                          (65, 40, 96, 0), (100, 84, 1184, 4), (128, 4096, 11008, 0),
+                                          (81, 36, 2048, 16), (97, 132, 352, 3), (113, 4096, 4096, 0), (128, 8192, 8192, 0)])
 def test_linear_planes(M, N, K, splits, tiles_per_wave):
-    """The product for up to 128 rows (64 a launch), K cut into ranges: the planes add up to x . w^T, and what
-    `add_rmsnorm` makes of them is the residual add and norm of the product."""
+    """The product for up to 128 rows, K cut into ranges: the planes add up to x . w^T, and what
+    `add_rmsnorm` makes of them is the residual add and norm of the product.  Beyond 64 rows one
+    launch and two of 64 rows give the same bits."""
     o = ops()
     if N >= 8192 and tiles_per_wave:
         return                   # the large case is there for the library's own choice of tiles
@@ -734,6 +736,14 @@ def test_linear_planes(M, N, K, splits, tiles_per_wave):
         o._lib().illm_set_mid_tiles_per_wave(0)
     assert planes.dtype == torch.float32 and planes.shape[1:] == (M, N)
     assert splits == 0 or planes.shape[0] == splits
+    if M > 64:
+        o._lib().illm_set_mid_tiles_per_wave(tiles_per_wave)
+        o._lib().illm_set_mid_rows_a_launch(64)
+        try:
+            assert torch.equal(o.linear_planes(x.to(DEV), wc, splits), planes)
+        finally:
+            o._lib().illm_set_mid_tiles_per_wave(0)
+            o._lib().illm_set_mid_rows_a_launch(128)
     want = R.linear(x, w, torch.float64)
     torch.testing.assert_close(planes.double().sum(0).cpu(), want, atol=2e-4 * math.sqrt(K), rtol=1e-5)
     into = rnd(M, N, seed=3) * 10
@@ -756,6 +766,9 @@ def test_linear_planes_refuses_what_it_does_not_take():
     assert not o.linear_planes_fits(x.float(), _plain_copy(w))
     wide = rnd(256, 256, dtype=torch.bfloat16).to(DEV)                      # K < 2 N: the vendor GEMM's
     assert not o.linear_planes_fits(x, _plain_copy(wide))
+    many = rnd(100, 256, dtype=torch.bfloat16).to(DEV)                      # but from 65 rows K = N is taken
+    assert o.linear_planes_fits(many, _plain_copy(wide)) and o.linear_planes_pays(many, _plain_copy(wide))
+    assert not o.linear_planes_fits(many, _plain_copy(rnd(512, 256, dtype=torch.bfloat16).to(DEV)))
     gate_up = o.Weight(w, o.tile_weight(w, o.tile_rows(64, "gate_up")), "gate_up")
     assert not o.linear_planes_fits(x, gate_up)                            # another kernel's tile order
     with pytest.raises(Exception):
