@@ -152,7 +152,7 @@ int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y,
                          int K, const void* nw, int nw_dt, void* xb, float* ssq_out,
                          int waves_wanted, void* stream);
 
-// Y = X[M, K] . W[N, K]^T for M up to 128 (64 rows a launch) from the tiled copy Wt of W, K a
+// Y = X[M, K] . W[N, K]^T for M up to 128 from the tiled copy Wt of W, K a
 // multiple of 32, X shared by a block's waves through LDS.  splits == 1: Y is [M, N] of y_dt;
 // splits > 1: K is cut into that many ranges and Y is float32 [splits][M][N], the planes to be
 // added by the caller (illm_add_rmsnorm takes them).  illm_gemm_mid_splits: the splits to use.
@@ -173,7 +173,7 @@ void illm_set_skinny_one_shot(int on);
 // products on the matrix cores (default 1).
 void illm_set_gqa_pv_on_matrix_cores(int on);
 
-// Products of 1 to 128 bfloat16 rows (meant for 9 and more; 64 rows a launch) from the tiled copy
+// Products of 1 to 128 bfloat16 rows (meant for 9 and more) from the tiled copy
 // Wt of W, K a multiple of 64, X shared by a block's waves through LDS, K cut inside the block
 // (csrc/gemm_rows.hip).  illm_gemm_rows_bf16: Y[M, N] = X . W^T (plain tiles), float32 or bfloat16.
 // illm_gemm_rows_gateup_silu: Y[M, F] = silu(X . Wg^T) * (X . Wu^T) from the gate|up tiles.
@@ -192,6 +192,8 @@ int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int 
 // Tuning and tests: tiles a block of these products takes (2 to 8) and parts of K (1, 2, 4;
 // four tiles and more: 1, 2); 0: the library's own choice.
 void illm_set_rows_shape(int tb, int kp);
+// Tuning and tests: rows of X a launch of these products takes, 64 or 128 (default).
+void illm_set_rows_a_launch(int rows);
 
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
 // product, `ssq` included.  waves_wanted: waves per block (0: the default choice).

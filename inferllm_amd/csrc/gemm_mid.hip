@@ -1,4 +1,4 @@
-// Y[M, N] = X[M, K] . W[N, K]^T for up to 64 rows a launch (decoding larger batches), bfloat16 operands,
+// Y[M, N] = X[M, K] . W[N, K]^T for up to 128 rows (decoding larger batches), bfloat16 operands,
 // float32 accumulation on the matrix cores, from the tiled copy of W
 // ([tile of 16 rows][K / 32][16 rows][32 k], see gemm_skinny.hip).
 //
@@ -174,8 +174,7 @@ extern "C" int illm_gemm_mid_splits(int N, int K) {
     return (pieces + per - 1) / per;
 }
 
-// Takes bfloat16 X [M, K] with M in 1..128 (more than 64 rows: 64 at a time, W read again for
-// each) and the tiled copy Wt of W [N, K], K a multiple of 32.  splits == 1: Y is [M, N] of y_dt.
+// Takes bfloat16 X [M, K] with M in 1..128 and the tiled copy Wt of W [N, K], K a multiple of 32.  splits == 1: Y is [M, N] of y_dt.
 // splits > 1: Y is float32 [splits][M][N], whose planes the caller adds up.  Otherwise
 // ILLM_ERR_ARG.
 extern "C" int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M, int N,

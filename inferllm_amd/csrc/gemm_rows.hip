@@ -57,7 +57,7 @@ struct GrScale {
 // GR_PIECE: k-steps of 32 in a piece.  A block of four or more tiles has at most two parts of K,
 // one of two or three tiles up to four.
 template <int MT, int TB, int MODE, int GR_PIECE>
-__global__ void __launch_bounds__(64 * TB * (TB >= 4 ? 2 : 4))
+__global__ void __launch_bounds__(64 * TB * (TB >= 4 ? 2 : 4) / (MT > 4 ? 2 : 1))
 gemm_rows_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ Wt, void* __restrict__ Y,
                  int y_dt, int M, int N, int K, int tiles, int kp, GrRope rope, GrScale scale) {
     constexpr int UNITS = MT * 16 * GR_PIECE * 4;            // 16-byte units of a part's X piece
@@ -352,7 +352,8 @@ static void rows_shape(int tiles, int K, int mt, int* tb, int* kp) {
     }
     *tb = GR_TB ? GR_TB : best_tb;
     *kp = GR_KP ? GR_KP : (*tb <= 3 ? 2 : 1);
-    if (*tb >= 4 && *kp > 2) *kp = 2;                       // the kernel's launch bounds
+    const int kp_max = (*tb >= 4 ? 2 : 4) / (mt > 4 ? 2 : 1);   // the kernel's launch bounds
+    if (*kp > kp_max) *kp = kp_max;
     const int pieces = (K / 32 + GR_PIECE_STEPS - 1) / GR_PIECE_STEPS;
     while (*kp > 1 && pieces / *kp < 4) *kp /= 2;
 }
@@ -383,13 +384,17 @@ static int launch_rows(const bf16_t* x, const bf16_t* wt, void* y, int y_dt, int
     return illm_launch_status();
 }
 
+static int GR_ROWS_A_LAUNCH = 128;        // tuning and tests: 64 or 128 rows of X a launch
+extern "C" void illm_set_rows_a_launch(int rows) { GR_ROWS_A_LAUNCH = rows == 64 ? 64 : 128; }
+
 template <int MODE>
 static int rows_product(const void* X, const void* Wt, void* Y, int y_dt, int M, int N, int K,
                         int tiles, GrRope rope, const GrScale& scale, hipStream_t st) {
-    // more than 64 rows: 64 at a time, W read again for each
+    // more rows than a launch takes: W is read again for each
     const size_t y_elem = y_dt == ILLM_F32 ? 4 : 2;
-    for (int m0 = 0; m0 < M; m0 += 64) {
-        const int rows = M - m0 < 64 ? M - m0 : 64;
+    const int a_launch = GR_ROWS_A_LAUNCH;
+    for (int m0 = 0; m0 < M; m0 += a_launch) {
+        const int rows = M - m0 < a_launch ? M - m0 : a_launch;
         const int mt = (rows + 15) / 16;
         const bf16_t* x = (const bf16_t*)X + (size_t)m0 * K;
         void* y = (char*)Y + (size_t)m0 * N * y_elem;
@@ -403,7 +408,11 @@ static int rows_product(const void* X, const void* Wt, void* Y, int y_dt, int M,
             case 1: rc = launch_rows<1, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
             case 2: rc = launch_rows<2, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
             case 3: rc = launch_rows<3, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
-            default: rc = launch_rows<4, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
+            case 4: rc = launch_rows<4, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
+            case 5: rc = launch_rows<5, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
+            case 6: rc = launch_rows<6, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
+            case 7: rc = launch_rows<7, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
+            default: rc = launch_rows<8, MODE>(x, (const bf16_t*)Wt, y, y_dt, rows, N, K, tiles, rp, scale, st); break;
         }
         if (rc != ILLM_OK) return rc;
     }

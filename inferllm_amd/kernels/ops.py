@@ -670,11 +670,14 @@ def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return _run_plan(x, w, plan)
 
 
-ROWS_MAX = 128           # rows the products of csrc/gemm_rows.hip take (64 a launch)
-ROWS_FUSED_MAX = 64      # rows up to which the fused q|k|v and gate|up products are taken: beyond
-                         # a launch's 64 rows W is read twice and the vendor GEMM with the
-                         # elementwise kernels behind it wins (measured at 128 rows of the 7B
-                         # shapes: q|k|v 47 against 33 + 5 us, gate|up 84 against 46 + 4)
+ROWS_MAX = 128           # rows the products of csrc/gemm_rows.hip take, all in one launch
+ROWS_FUSED_MAX = 128     # and the fused q|k|v and gate|up products (measured against the vendor
+                         # GEMM with the elementwise kernel behind it, 80 / 96 / 128 rows: gate|up
+                         # of the 7B shape 39 / 40 / 44 against 50 / 50 / 49 us, of the 8B shape
+                         # 46 / 48 / 52 against 73 / 59 / 61; q|k|v 12288 x 4096 26 / 27 / 36
+                         # against 30 / 33 / 34 + 5; in two launches of 64 rows they lost)
+ROWS_QKV_SMALL_MAX = 96  # q|k|v matrices of fewer than 8192 rows: 6144 x 4096 takes 21 / 24 / 34
+                         # against 23 / 23 / 25 + 5
 ROWS_FROM = 17           # from this many rows they are taken unless the plan says otherwise for
                          # the shape (up to 16 rows the few-rows kernels are the other way)
 
@@ -690,6 +693,8 @@ def rows_fits(x, w, mode: str) -> bool:
     `NormedRows`, up to 16) and a weight with a decode copy in `mode`'s tile order."""
     xt = x.xb if isinstance(x, NormedRows) else x
     most = 16 if isinstance(x, NormedRows) else (ROWS_MAX if mode == "plain" else ROWS_FUSED_MAX)
+    if mode == "qkv" and isinstance(w, Weight) and w.plain.shape[0] < 8192:
+        most = min(most, ROWS_QKV_SMALL_MAX)
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == mode
             and isinstance(xt, torch.Tensor) and xt.dtype == torch.bfloat16 and xt.dim() == 2
             and 1 <= xt.shape[0] <= most
@@ -745,7 +750,8 @@ PLAIN_WAVES = 0          # and for the plain few-rows product
 
 def qkv_rope_store_fits(x, w_qkv, hd: int) -> bool:
     """Whether the one-kernel q|k|v product + rotation + cache store takes these operands: up to
-    16 rows always, up to 64 with a decode copy of the matrix in q|k|v tile order."""
+    16 rows always, up to 128 (96 for small matrices) with a decode copy of the matrix in q|k|v
+    tile order."""
     if not (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and hd % 16 == 0):
         return False
     if 1 <= x.shape[0] <= SKINNY_BEST_ROWS and x.shape[1] % 8 == 0:

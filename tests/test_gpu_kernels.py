@@ -994,10 +994,13 @@ def test_linear_rows(M, N, K, tb, kp, rows_shape):
         got = o.linear_rows(x.to(DEV), wc, ydt)
         assert got.dtype == ydt
         close(got, want, ydt, scale=0.2 * math.sqrt(K))
-    # a row's result does not depend on the other rows of the step: the same bits
-    alone = o.linear_rows(x[M - 1:].to(DEV), wc, torch.float32)
-    among = o.linear_rows(x.to(DEV), wc, torch.float32)[M - 1]
-    assert torch.equal(alone[0], among)
+    # a row's result does not depend on the other rows of the step: the same bits (beyond 64 rows
+    # a block has half as many parts of K at most, so a forced number of parts may hold for the
+    # row alone and not for the step: another order of summation)
+    if not (M > 64 and kp is not None and kp > (1 if tb >= 4 else 2)):
+        alone = o.linear_rows(x[M - 1:].to(DEV), wc, torch.float32)
+        among = o.linear_rows(x.to(DEV), wc, torch.float32)[M - 1]
+        assert torch.equal(alone[0], among)
 
 
 def test_linear_rows_takes_the_norm_and_refuses_what_it_does_not_take(rows_shape):
@@ -1021,9 +1024,10 @@ def test_linear_rows_takes_the_norm_and_refuses_what_it_does_not_take(rows_shape
 
 
 @pytest.mark.parametrize("tb,kp", _ROWS_SHAPES)
-@pytest.mark.parametrize("M,F,K", [(17, 172, 64), (64, 11008, 4096), (40, 50, 192), (64, 203, 320), (33, 8, 1024)])
+@pytest.mark.parametrize("M,F,K", [(17, 172, 64), (64, 11008, 4096), (40, 50, 192), (64, 203, 320), (33, 8, 1024),
+                                   (65, 50, 192), (100, 172, 128), (128, 2056, 512), (113, 203, 320)])
 def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, rows_shape):
-    """17 to 64 rows: the product and the SiLU-multiply in one kernel, from the gate|up tiles."""
+    """17 to 128 rows: the product and the SiLU-multiply in one kernel, from the gate|up tiles."""
     o = ops()
     rows_shape(tb, kp)
     x = rnd(M, K, dtype=torch.bfloat16, seed=1)
@@ -1044,10 +1048,12 @@ def test_gate_up_silu_of_many_rows(M, F, K, tb, kp, rows_shape):
 
 @pytest.mark.parametrize("tb,kp", _ROWS_SHAPES)
 @pytest.mark.parametrize("M,nh,nkv,hd,K", [(17, 4, 2, 32, 64), (64, 32, 32, 128, 4096), (40, 6, 3, 64, 256),
-                                           (64, 8, 1, 96, 128), (33, 3, 3, 48, 192), (50, 2, 1, 16, 1024)])
+                                           (64, 8, 1, 96, 128), (33, 3, 3, 48, 192), (50, 2, 1, 16, 1024),
+                                           (65, 4, 2, 32, 64), (96, 6, 3, 64, 256), (128, 48, 8, 128, 256),
+                                           (113, 40, 40, 128, 128)])
 def test_qkv_rope_store_of_many_rows(M, nh, nkv, hd, K, tb, kp, rows_shape):
-    """17 to 64 sequences decoding together: the q|k|v product, the rotation and the cache store
-    in one kernel against the three steps."""
+    """17 to 128 sequences decoding together (96 for matrices of fewer than 8192 rows): the q|k|v
+    product, the rotation and the cache store in one kernel against the three steps."""
     from inferllm_amd.parts.position import rotary_table
     o = ops()
     rows_shape(tb, kp)
