@@ -228,7 +228,7 @@ def main() -> int:
     ctx_len = shape_cfg["max_position_embeddings"]
     headline = args.shape == "llama2-7b" and args.dtype == "bfloat16" and not args.no_points
     long_ctx = 3800
-    max_b = max(args.batch, 1 if args.no_points else 64)
+    max_b = max(args.batch, 1 if args.no_points else (128 if headline else 64))
     per_seq = -(-(args.prompt + args.steps + args.warmup + 2) // 64) * 64     # whole cache pages
     room = max(max_b * max(per_seq, 1024), 4096)
     if headline:
@@ -266,6 +266,8 @@ def main() -> int:
             v, _, f = b.decode_run(batch, few, 4, args.prompt)
             points[name], points[name + "_hbm_frac"] = round(v, 2), round(f, 4)
         if headline:
+            v, _, f = b.decode_run(128, 64, 4, args.prompt)
+            points["decode_b128"], points["decode_b128_hbm_frac"] = round(v, 2), round(f, 4)
             # long contexts: the cache's share of a step's bytes grows from a seventh to nine tenths
             for name, batch in (("decode_b8_ctx3800", 8), ("decode_b64_ctx3800", 64)):
                 v, _, f = b.decode_run(batch, 64, 4, long_ctx)
