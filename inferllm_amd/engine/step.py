@@ -42,10 +42,13 @@ class StepEntry:
 
 
 def _bucket(n: int) -> int:
+    """Rows of the graph that a decode step of n sequences is replayed from: powers of two, and
+    from 16 on the sizes half way between them too (24, 48, 96, ...: the products' time grows
+    with their tiles of 16 rows, so 96 rows cost less than 128)."""
     b = 1
     while b < n:
         b *= 2
-    return b
+    return b * 3 // 4 if b >= 32 and n <= b * 3 // 4 else b
 
 
 def _length_class(n: int, limit: int) -> int:

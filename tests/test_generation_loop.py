@@ -278,3 +278,16 @@ def test_prompts_fed_in_several_steps_give_the_same_tokens(ahead, limit):
     if limit == 4:
         # the first batch's prompts of 3, 1 and 5 tokens: [3 + 1], [4 of the third], [its last]
         assert m.steps[:3] == [[(0, 3), (1, 1)], [(2, 4)], [(2, 1)]]
+
+
+def test_rows_of_the_decode_graphs():
+    """A decode step of n sequences is replayed from a graph of at least n rows: powers of two,
+    and from 24 on the sizes half way between them; never fewer rows than sequences, and from 17
+    sequences on less than half as many again."""
+    from inferllm_amd.engine.step import _bucket
+    assert [_bucket(n) for n in (1, 2, 3, 8, 9, 16, 17, 24, 25, 33, 48, 49, 65, 96, 97, 129, 193)] == \
+           [1, 2, 4, 8, 16, 16, 24, 24, 32, 48, 48, 64, 96, 96, 128, 192, 256]
+    for n in range(1, 600):
+        b = _bucket(n)
+        assert n <= b and (b < 2 * n or n == 1) and (n < 17 or 2 * b < 3 * n)
+        assert b == _bucket(b)
