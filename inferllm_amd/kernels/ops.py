@@ -440,13 +440,13 @@ def current_plan() -> Plan:
 
 def linear_planes_fits(x, w) -> bool:
     """Whether `linear_planes` takes these operands: up to 128 bfloat16 rows and a matrix with a
-    decode copy in plain tile order that has few rows for its length (K >= 2 N; from 65 rows on
-    K >= N, where the vendor GEMM is at its worst)."""
+    decode copy in plain tile order that has few rows for its length (K >= 2 N; from 17 rows on
+    K >= N)."""
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == "plain"
             and isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and x.dim() == 2
             and 1 <= x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.plain.shape[1]
             and w.plain.shape[0] % 4 == 0 and w.plain.shape[0] <= MID_MAX_COLS
-            and w.plain.shape[1] >= (2 if x.shape[0] <= 64 else 1) * w.plain.shape[0])
+            and w.plain.shape[1] >= (2 if x.shape[0] <= SKINNY_BEST_ROWS else 1) * w.plain.shape[0])
 
 
 _flush: Dict[int, torch.Tensor] = {}
@@ -517,7 +517,8 @@ def linear_planes_pays(x, w) -> bool:
     if rows > SKINNY_BEST_ROWS:
         # (65 to 128 rows, one launch, product and the norm that adds its planes against the
         # vendor GEMM and its norm: the 7B down projection 28 to 33 us against 38 to 64, the 70B
-        # one 86 to 101 against 134 to 221, 4096 x 4096 18 to 22 against 20 to 29)
+        # one 86 to 101 against 134 to 221, 4096 x 4096 18 to 22 against 20 to 29; 17 to 64 rows
+        # of 4096 x 4096 15 to 18 against 17 to 19, of 5120 x 5120 17 to 22 against 21 to 31)
         return True
     key = tuple(w.plain.shape)
     first = _plan.planes_from.get(key)

@@ -764,9 +764,9 @@ def test_linear_planes_refuses_what_it_does_not_take():
     assert o.linear_planes_fits(x[:16], _plain_copy(w)) and o.linear_planes_pays(x, _plain_copy(w))
     assert not o.linear_planes_fits(rnd(129, 256, dtype=torch.bfloat16).to(DEV), _plain_copy(w))
     assert not o.linear_planes_fits(x.float(), _plain_copy(w))
-    wide = rnd(256, 256, dtype=torch.bfloat16).to(DEV)                      # K < 2 N: the vendor GEMM's
-    assert not o.linear_planes_fits(x, _plain_copy(wide))
-    many = rnd(100, 256, dtype=torch.bfloat16).to(DEV)                      # but from 65 rows K = N is taken
+    wide = rnd(256, 256, dtype=torch.bfloat16).to(DEV)                      # K < 2 N: not up to 16 rows
+    assert not o.linear_planes_fits(x[:16], _plain_copy(wide)) and o.linear_planes_fits(x, _plain_copy(wide))
+    many = rnd(100, 256, dtype=torch.bfloat16).to(DEV)                      # from 17 rows K = N is taken
     assert o.linear_planes_fits(many, _plain_copy(wide)) and o.linear_planes_pays(many, _plain_copy(wide))
     assert not o.linear_planes_fits(many, _plain_copy(rnd(512, 256, dtype=torch.bfloat16).to(DEV)))
     gate_up = o.Weight(w, o.tile_weight(w, o.tile_rows(64, "gate_up")), "gate_up")
