@@ -420,7 +420,7 @@ MID_MAX_ROWS = 128       # rows a launch of the kernel takes (the vendor GEMM re
                          # at 1.6 TB/s at 128 rows: 58.6 us for the 7B down projection)
 MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the norm that adds the
                          # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
-                         # K >= 2 N (the down projection) and the same time when K = N
+                         # K >= 2 N (the down projection) and 0.8 to 0.95 when K = N
 PLANES_MIN_ELEMENTS = 1 << 22   # smaller matrices are not measured (both ways take a few
                                 # microseconds and the clock would decide): no planes below 17 rows
 
