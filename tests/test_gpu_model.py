@@ -598,6 +598,53 @@ def test_kernel_timing_reports_every_op(tmp_path_factory):
     assert "share" in t.table()
 
 
+def test_real_layer_sizes_with_many_sequences(tmp_path_factory, monkeypatch):
+    """Two layers of the LLaMA-2-7B sizes with 40, then 25 sequences decoding together: steps of
+    17 to 128 rows take the kernels that share X through LDS (fused q|k|v with rotation and
+    store, gate|up with SiLU-multiply, o and down as planes, the head) from graphs of 48 and of
+    32 rows, and no product of such a step goes to the vendor GEMM."""
+    import inferllm_amd as I
+    from inferllm_amd import StepEntry
+    config = {"architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "intermediate_size": 11008,
+              "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 32,
+              "vocab_size": 32000, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+              "max_position_embeddings": 512, "tie_word_embeddings": False,
+              "bos_token_id": 1, "eos_token_id": 2}
+    d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=12, dtype=torch.bfloat16, gain=2.0)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=40, max_seq_len=64,
+                                   poison_freed=True)
+    assert eng.decode_copies is True
+    n, tail = 40, 5
+    reqs = requests_for(config, [5 + (3 * i) % 6 + tail for i in range(n)], seed=5)
+    heads = [len(r) - tail for r in reqs]
+    slots = [eng.alloc_slot() for _ in reqs]
+    eng.step([StepEntry(s, r[:h], []) for s, r, h in zip(slots, reqs, heads)])
+    vendor = []
+    real = torch.matmul
+    monkeypatch.setattr(torch, "matmul", lambda *a, **k: vendor.append(tuple(a[0].shape)) or real(*a, **k))
+    live = list(range(n))
+    got = {i: [] for i in live}
+    for t in range(tail):
+        if t == 3:                                       # 15 sequences end: 25 go on, in a graph of 32 rows
+            for i in live[25:]:
+                eng.free_slot(slots[i])
+            live = live[:25]
+        out = eng.step([StepEntry(slots[i], [reqs[i][heads[i] + t]], [0]) for i in live])
+        for row, i in enumerate(live):
+            got[i].append(out[row:row + 1].clone())
+    monkeypatch.setattr(torch, "matmul", real)
+    assert not vendor, f"products of decode steps went to the vendor GEMM: rows x width {sorted(set(vendor))}"
+    assert sorted(size for size, _ in eng.runner._graphs) == [32, 48]
+    for i in (0, 7, 16, 24, 25, 33, 39):                 # the plain model is slow at these sizes
+        want = plain_llama.forward_logits(config, w, reqs[i])[heads[i]:heads[i] + len(got[i])]
+        per_pos = (torch.cat(got[i]).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+        assert float(per_pos.max()) < BUDGET["bfloat16"], f"request {i}: {per_pos.tolist()}"
+    for i in live:
+        eng.free_slot(slots[i])
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("nkv,ffn", [(32, 11008), (8, 14336)])
 def test_real_layer_sizes_in_bfloat16(tmp_path_factory, nkv, ffn):
     """Two layers of the LLaMA-2-7B sizes (width 4096, 32 heads of 128, feed-forward 11008,
