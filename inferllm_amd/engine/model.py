@@ -116,9 +116,12 @@ class DecoderModel:
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             if getattr(layer, "takes_next_norm", False):
-                # the norm that will meet this block's output, for kernels that prepare it
-                nxt = (getattr(self.layers[self.schedule[i + 1].layer], "mixer_norm", None)
-                       if i + 1 < len(self.schedule) else self.final_norm)
+                # the norm that will meet this block's output, for kernels that prepare it; none if
+                # the block that follows does not say that it takes rows prepared for its norm
+                # (it then finds the sum in x, or a plain tensor still to be added)
+                after = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
+                nxt = (self.final_norm if after is None else
+                       after.mixer_norm if getattr(after, "takes_prepared_rows", False) else None)
                 pending = layer.forward(x, pending, ctx, e.cache_line, e.writes_cache, next_norm=nxt)
             else:
                 pending = layer.forward(x, pending, ctx, e.cache_line, e.writes_cache)

@@ -163,6 +163,13 @@ class PositionEncoding(Part):
 
 
 class Block(Part):
+    # `takes_next_norm`: `forward` also takes `next_norm=`, the norm that will meet what the block
+    # hands on, and may hand on None (the sum is in x already) or `ops.NormedRows` prepared for it.
+    # `takes_prepared_rows`: the block accepts `ops.NormedRows` as `pending`.  Both False: the
+    # plain protocol, `pending` is None or a tensor (or planes, if its first norm adds planes).
+    takes_next_norm = False
+    takes_prepared_rows = False
+
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm,
                  feed_forward_norm: Norm, position: Optional[PositionEncoding]):
         super().__init__()

@@ -19,6 +19,7 @@ class PreNormBlock(Block):
     """
 
     takes_next_norm = True
+    takes_prepared_rows = True
 
     @staticmethod
     def _enter(norm, part, x, pending, ctx):

@@ -662,3 +662,138 @@ def test_toy_routed_feed_forward_and_learned_positions(tmp_path):
         out = eng.step([I.StepEntry(s, [r[n + j]], [0]) for s, r, n in zip(slots, reqs, head)])
         for b in range(2):
             assert rel(out[b], want[b][0][head[b] + j]) < 2e-5, (b, j)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_and_toy_arrangement_of_a_block(tmp_path, dtype):
+    """The last two kinds of parts as toys of the test: a norm that subtracts the mean and has a
+    bias (float32 statistics, no planes, nothing a product's kernel may take over), and a block
+    in which mixer and feed-forward read the same normed rows and both results are added.
+    Registered, built from a spec next to a layer of the library's own parts, stepped whole and
+    token by token in a batch of two, under decode graphs, against a plain computation."""
+    import inferllm_amd as I
+    from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from inferllm_amd.parts import Block, Norm, register_part
+    from inferllm_amd.weights import TensorWant, write_safetensors
+    from tiny import random_ids, read_weights
+    E, V, nh, nkv, hd, F, eps, P_MAX, theta = 64, 90, 4, 2, 16, 96, 1e-4, 96, 5000.0
+
+    @register_part("norm", "toy_layer_norm_" + dtype)
+    class ToyLayerNorm(Norm):
+        def __init__(self, size, eps, tensors=None):
+            super().__init__(tensors)
+            self.size, self.eps = size, eps
+
+        def shapes(self):
+            return {"weight": TensorWant((self.size,), init="ones_normal", keep_stored=True),
+                    "bias": TensorWant((self.size,), keep_stored=True)}
+
+        def load(self, tensors):
+            self.weight = self._take(tensors, "weight").float()
+            self.bias = self._take(tensors, "bias").float()
+
+        def forward(self, x, delta, ctx, row_idx=None):
+            if row_idx is None:
+                if delta is not None:
+                    x.add_(delta.float())
+                rows = x
+            else:
+                rows = x[row_idx.long()]
+                if delta is not None:
+                    rows = rows + delta[row_idx.long()].float()
+            mean = rows.mean(dim=-1, keepdim=True)
+            var = ((rows - mean) ** 2).mean(dim=-1, keepdim=True)
+            return ((rows - mean) * torch.rsqrt(var + self.eps) * self.weight + self.bias).to(ctx.act_dtype)
+
+    @register_part("block", "toy_parallel_" + dtype)
+    class ToyParallelBlock(Block):
+        def forward(self, x, pending, ctx, line, writes_cache):
+            h = self.mixer_norm.forward(x, pending, ctx)
+            a = self.mixer.forward(h, ctx, line, writes_cache, self.position)
+            return a.float() + self.feed_forward.forward(h, ctx).float()
+
+    @register_architecture("ToyParallelForTests_" + dtype)
+    class Cfg:
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": ["ToyParallelForTests_" + dtype]}
+
+        def to_spec(self):
+            rms = lambda n: PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": n})
+            ln = lambda n: PartSpec("toy_layer_norm_" + dtype, {"size": E, "eps": eps}, {"weight": n + ".w", "bias": n + ".b"})
+            rope = PartSpec("rotary", {"head_dim": hd, "rotary_dim": hd, "theta": theta, "max_positions": P_MAX,
+                                       "pairing": "half"})
+            att = lambda i: PartSpec("attention", {"hidden_size": E, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd},
+                                     {k: f"l{i}.{k}" for k in "qkvo"})
+            ffn = lambda i: PartSpec("swiglu", {"hidden_size": E, "intermediate_size": F},
+                                     {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"})
+            layers = [LayerSpec("toy_parallel_" + dtype, att(0), ffn(0), ln("l0.n1"), ln("l0.unused"), rope),
+                      LayerSpec("pre_norm", att(1), ffn(1), rms("l1.n1"), ln("l1.n2"), rope),
+                      LayerSpec("toy_parallel_" + dtype, att(2), ffn(2), rms("l2.n1"), rms("l2.unused"), rope)]
+            return ModelSpec("ToyParallelForTests_" + dtype, V, E, P_MAX,
+                             PartSpec("token_embedding", {"vocab_size": V, "hidden_size": E}, {"weight": "emb"}),
+                             layers, [ScheduleEntry(i, i) for i in range(3)], ln("nf"),
+                             PartSpec("lm_head", {"hidden_size": E, "vocab_size": V}, {"weight": "head"}))
+
+    d = I.write_random_model(str(tmp_path / "parallel"), Cfg(), seed=8,
+                             dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    w = read_weights(d)
+    for n in list(w):
+        if n.endswith(".b"):
+            w[n] = (w[n].float() * 10 + 0.5).to(w[n].dtype)          # biases must matter
+        elif w[n].dim() == 2 and n not in ("emb", "head"):
+            w[n] = (w[n].float() * 4).to(w[n].dtype)                  # and so must the layers
+    write_safetensors(str(tmp_path / "parallel" / "model.safetensors"), w.items())
+    w = {n: t.double() for n, t in w.items()}
+
+    def layer_norm(x, n):
+        mean = x.mean(-1, keepdim=True)
+        var = ((x - mean) ** 2).mean(-1, keepdim=True)
+        return (x - mean) / torch.sqrt(var + eps) * w[n + ".w"] + w[n + ".b"]
+
+    def attention(h, i, S):
+        q = P.linear(h, w[f"l{i}.q"]).reshape(S, nh, hd)
+        k = P.linear(h, w[f"l{i}.k"]).reshape(S, nkv, hd)
+        v = P.linear(h, w[f"l{i}.v"]).reshape(S, nkv, hd)
+        q = P.rope_rotate_half(q, range(S), theta, hd)
+        k = P.rope_rotate_half(k, range(S), theta, hd)
+        rep = nh // nkv
+        k, v = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
+        return P.linear(P.causal_attention(q, k, v), w[f"l{i}.o"])
+
+    def ffn(h, i):
+        return P.swiglu_ffn(h, w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+
+    def plain(ids):
+        S = len(ids)
+        x = P.embedding(w["emb"], ids)
+        h = layer_norm(x, "l0.n1")
+        x = x + attention(h, 0, S) + ffn(h, 0)
+        x = x + attention(P.rms_norm(x, w["l1.n1"], eps), 1, S)
+        x = x + ffn(layer_norm(x, "l1.n2"), 1)
+        h = P.rms_norm(x, w["l2.n1"], eps)
+        x = x + attention(h, 2, S) + ffn(h, 2)
+        return P.linear(layer_norm(x, "nf"), w["head"])
+
+    budget = 2e-5 if dtype == "float32" else 3e-2
+    eng = I.Engine.from_pretrained(d, dtype=dtype, max_batch=2, max_seq_len=P_MAX)
+    assert eng.runner.use_graphs
+    reqs = [random_ids(n, V, 7 * n) for n in (37, 9)]
+    want = [plain(r) for r in reqs]
+    slots = [eng.alloc_slot(), eng.alloc_slot()]
+    head = [len(r) - 4 for r in reqs]
+    out = eng.step([I.StepEntry(s, r[:n], list(range(n))) for s, r, n in zip(slots, reqs, head)])
+    assert rel(out[:head[0]], want[0][:head[0]]) < budget and rel(out[head[0]:], want[1][:head[1]]) < budget
+    for j in range(4):                                        # the first of these is captured, the rest replayed
+        out = eng.step([I.StepEntry(s, [r[n + j]], [0]) for s, r, n in zip(slots, reqs, head)])
+        for b in range(2):
+            assert rel(out[b], want[b][head[b] + j]) < budget, (b, j)
+    # the plain computation is not blind to the toys: without the biases, or with the second
+    # arrangement for the first layer, it gives other logits
+    saved = w["l0.n1.b"].clone()
+    w["l0.n1.b"] = torch.zeros_like(saved)
+    assert rel(plain(reqs[1]), want[1]) > 10 * budget
+    w["l0.n1.b"] = saved
