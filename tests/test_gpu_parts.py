@@ -797,3 +797,112 @@ def test_toy_norm_and_toy_arrangement_of_a_block(tmp_path, dtype):
     w["l0.n1.b"] = torch.zeros_like(saved)
     assert rel(plain(reqs[1]), want[1]) > 10 * budget
     w["l0.n1.b"] = saved
+
+
+def test_toy_embedding_and_toy_head(tmp_path):
+    """The two ends as toys of the test: an embedding that scales its rows by sqrt(width), and a
+    head with a bias whose logits are capped softly by a tanh.  Registered, built around one
+    layer of the library's own parts, stepped whole and token by token, against a plain
+    computation; generation through the entry point follows the plain argmax."""
+    import inferllm_amd as I
+    from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from inferllm_amd.kernels import ops
+    from inferllm_amd.parts import Embedding, Head, register_part
+    from inferllm_amd.weights import TensorWant, write_safetensors
+    from tiny import random_ids, read_weights
+    E, V, nh, hd, F, eps, P_MAX, theta, cap = 48, 77, 3, 16, 80, 1e-5, 64, 10000.0, 3.0
+
+    @register_part("embedding", "toy_scaled_embedding")
+    class ScaledEmbedding(Embedding):
+        def __init__(self, vocab_size, hidden_size, tensors=None):
+            super().__init__(tensors)
+            self.V, self.E = vocab_size, hidden_size
+
+        def shapes(self):
+            return {"weight": TensorWant((self.V, self.E))}
+
+        def load(self, tensors):
+            self.weight = self._take(tensors, "weight").contiguous()
+
+        def forward(self, ctx):
+            return ops.embed(ctx.tokens, self.weight) * math.sqrt(self.E)
+
+    @register_part("head", "toy_capped_head")
+    class CappedHead(Head):
+        def __init__(self, hidden_size, vocab_size, cap, tensors=None):
+            super().__init__(tensors)
+            self.E, self.V, self.cap = hidden_size, vocab_size, cap
+
+        def shapes(self):
+            return {"weight": TensorWant((self.V, self.E)), "bias": TensorWant((self.V,), keep_stored=True)}
+
+        def load(self, tensors):
+            self.weight = self._take(tensors, "weight").contiguous()
+            self.bias = self._take(tensors, "bias").float()
+
+        def forward(self, h, ctx):
+            z = ops.linear(h, self.weight, out_dtype=torch.float32) + self.bias
+            return self.cap * torch.tanh(z / self.cap)
+
+    @register_architecture("ToyEndsForTests")
+    class Cfg:
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": ["ToyEndsForTests"]}
+
+        def to_spec(self):
+            norm = lambda n: PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": n})
+            rope = PartSpec("rotary", {"head_dim": hd, "rotary_dim": hd, "theta": theta, "max_positions": P_MAX,
+                                       "pairing": "half"})
+            layer = LayerSpec("pre_norm",
+                              PartSpec("attention", {"hidden_size": E, "num_heads": nh, "num_kv_heads": nh, "head_dim": hd},
+                                       {k: f"l0.{k}" for k in "qkvo"}),
+                              PartSpec("swiglu", {"hidden_size": E, "intermediate_size": F},
+                                       {"gate": "l0.g", "up": "l0.u", "down": "l0.d"}),
+                              norm("l0.n1"), norm("l0.n2"), rope)
+            return ModelSpec("ToyEndsForTests", V, E, P_MAX,
+                             PartSpec("toy_scaled_embedding", {"vocab_size": V, "hidden_size": E}, {"weight": "emb"}),
+                             [layer], [ScheduleEntry(0, 0)], norm("nf"),
+                             PartSpec("toy_capped_head", {"hidden_size": E, "vocab_size": V, "cap": cap},
+                                      {"weight": "head", "bias": "head.b"}))
+
+    d = I.write_random_model(str(tmp_path / "ends"), Cfg(), seed=9)
+    w = read_weights(d)
+    w["head"] = w["head"] * 30.0                                # logits well into the cap
+    w["head.b"] = w["head.b"] * 50.0
+    write_safetensors(str(tmp_path / "ends" / "model.safetensors"), w.items())
+    w = {n: t.double() for n, t in w.items()}
+
+    def plain(ids):
+        S = len(ids)
+        x = P.embedding(w["emb"], ids) * math.sqrt(E)
+        h = P.rms_norm(x, w["l0.n1"], eps)
+        q, k, v = (P.linear(h, w[f"l0.{n}"]).reshape(S, nh, hd) for n in "qkv")
+        q, k = P.rope_rotate_half(q, range(S), theta, hd), P.rope_rotate_half(k, range(S), theta, hd)
+        x = x + P.linear(P.causal_attention(q, k, v), w["l0.o"])
+        x = x + P.swiglu_ffn(P.rms_norm(x, w["l0.n2"], eps), w["l0.g"], w["l0.u"], w["l0.d"])
+        z = P.linear(P.rms_norm(x, w["nf"], eps), w["head"]) + w["head.b"]
+        return cap * torch.tanh(z / cap)
+
+    eng = I.Engine.from_pretrained(d, dtype="float32", max_batch=2, max_seq_len=P_MAX)
+    ids = random_ids(30, V, 4)
+    want = plain(ids)
+    assert float(want.abs().max()) > 0.9 * cap                 # the cap is at work
+    s = eng.alloc_slot()
+    out = eng.step([I.StepEntry(s, ids[:26], list(range(26)))])
+    assert rel(out, want[:26]) < 2e-5
+    for j in range(26, 30):
+        assert rel(eng.step([I.StepEntry(s, [ids[j]], [0])])[0], want[j]) < 2e-5
+    eng.free_slot(s)
+    prompt = ids[:12]
+    got = eng.generate([prompt], max_new_tokens=5, stop_token_ids=[])[0]
+    seq = list(prompt)
+    for t in got:
+        logits = plain(seq)[-1]
+        top2 = torch.topk(logits, 2).values
+        if float(top2[0] - top2[1]) > 1e-4:                      # a near tie may go either way
+            assert t == int(torch.argmax(logits))
+        seq.append(t)
