@@ -598,6 +598,52 @@ def test_kernel_timing_reports_every_op(tmp_path_factory):
     assert "share" in t.table()
 
 
+def test_head_size_80_in_bfloat16(tmp_path_factory):
+    """A LLaMA of width 2560 with 32 heads of 80 (grouped in fours), a head size that is no
+    multiple of 32: the matrix-core prompt kernel with its last block of dims half used, the
+    fused q|k|v product with rotation, decode attention, whole prompts (one longer than a block
+    of 128 query rows) and single tokens, 3 and then 20 sequences together."""
+    import inferllm_amd as I
+    from inferllm_amd import StepEntry
+    config = {"architectures": ["LlamaForCausalLM"], "hidden_size": 2560, "intermediate_size": 6912,
+              "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8,
+              "vocab_size": 4000, "rms_norm_eps": 1e-6, "rope_theta": 10000.0,
+              "max_position_embeddings": 512, "tie_word_embeddings": False,
+              "bos_token_id": 1, "eos_token_id": 2}
+    d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=13, dtype=torch.bfloat16, gain=2.0)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=20, max_seq_len=256,
+                                   poison_freed=True)
+    assert eng.spec.layers[0].mixer.params["head_dim"] == 80
+    tail = 4
+    reqs = requests_for(config, [170, 23, 70] + [6 + i % 5 for i in range(17)], seed=7)
+    heads = [len(r) - tail for r in reqs]
+    slots = [eng.alloc_slot() for _ in reqs]
+    out = eng.step([StepEntry(s, r[:h], list(range(h)) if i < 3 else []) for i, (s, r, h) in enumerate(zip(slots, reqs, heads))])
+    got = {i: [] for i in range(len(reqs))}
+    at = 0
+    for i in range(3):
+        got[i].append(out[at:at + heads[i]].clone())
+        at += heads[i]
+    for t in range(tail):
+        live = range(3) if t < 2 else range(len(reqs))
+        if t == 2:                                       # the short ones catch up, then all 20 go on together
+            for u in range(2):
+                eng.step([StepEntry(slots[i], [reqs[i][heads[i] + u]], []) for i in range(3, len(reqs))])
+        out = eng.step([StepEntry(slots[i], [reqs[i][heads[i] + t]], [0]) for i in live])
+        for row, i in enumerate(live):
+            got[i].append(out[row:row + 1].clone())
+    for i in (0, 1, 2, 5, 19):
+        want = plain_llama.forward_logits(config, w, reqs[i])
+        want = want[:len(reqs[i])] if i < 3 else want[heads[i] + 2:heads[i] + tail]
+        per_pos = (torch.cat(got[i]).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+        assert float(per_pos.max()) < BUDGET["bfloat16"], \
+            f"request {i}: first bad position {int((per_pos >= BUDGET['bfloat16']).nonzero()[0])} of {len(per_pos)}"
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
+
+
 def test_real_layer_sizes_with_many_sequences(tmp_path_factory, monkeypatch):
     """Two layers of the LLaMA-2-7B sizes with 40, then 25 sequences decoding together: steps of
     17 to 128 rows take the kernels that share X through LDS (fused q|k|v with rotation and
