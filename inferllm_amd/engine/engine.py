@@ -175,6 +175,15 @@ class Engine:
         """See `StepRunner.step`.  The returned tensor is valid until the next step."""
         return self.runner.step(entries, device_tokens)
 
+    def warm_up(self, batch_sizes: Optional[Sequence[int]] = None, longest: int = 1) -> int:
+        """Capture the decode graphs for these numbers of sequences (default: every size up to
+        `max_batch` that has a graph of its own) with contexts up to `longest` keys, so that the
+        first decode step of such a batch does not pay for the capture.  Returns how many graphs
+        were captured."""
+        if batch_sizes is None:
+            batch_sizes = range(1, self.max_batch + 1)
+        return self.runner.warm_up(batch_sizes, min(int(longest), self.max_seq_len))
+
     # ------------------------------------------------------------ generation
     def generate(self, prompts: Sequence[Sequence[int]], temperature: float = 0.0,
                  top_k: int = 0, top_p: float = 1.0, repeat_penalty: float = 1.0,

@@ -235,6 +235,30 @@ class StepRunner:
             return g.logits[:B]
         return g.logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
 
+    @torch.no_grad()
+    def warm_up(self, batch_sizes: Sequence[int], longest: int = 1) -> int:
+        """Capture the graphs that decode steps of these numbers of sequences, none longer than
+        `longest` keys, would be replayed from, before the first of them comes (a capture costs
+        one eager run of the step and the capture itself, tens of milliseconds).  No sequence's
+        cache or state is touched.  Returns the number of graphs captured now."""
+        if not self.use_graphs:
+            return 0
+        if self.plan is not None:
+            ops.use_plan(self.plan)
+        self.cache.upload(lengths=False)
+        done = 0
+        for n in sorted(set(int(b) for b in batch_sizes)):
+            if n < 1:
+                raise StepError("warm_up: batch sizes are positive")
+            key = (_bucket(n), _length_class(max(int(longest), 1), self.cache.max_seq_len))
+            g = self._graphs.get(key)
+            if g is None:
+                g = self._graphs[key] = _DecodeGraph(self, *key)
+            if g.graph is None:
+                self._capture(g)
+                done += 1
+        return done
+
     def _capture(self, g: _DecodeGraph) -> None:
         """Capture the step's graph.  Before a capture the libraries must have set themselves up,
         which takes one eager run of the same shapes: that run has every row on the cache's spare

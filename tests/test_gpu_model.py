@@ -598,6 +598,37 @@ def test_kernel_timing_reports_every_op(tmp_path_factory):
     assert "share" in t.table()
 
 
+def test_warm_up_captures_the_decode_graphs_beforehand(tmp_path):
+    """`Engine.warm_up` captures the graphs of the batch sizes named (their buckets, once each)
+    without touching a sequence: the steps that follow capture nothing more and give the same
+    bits as in an engine that was not warmed up; an engine without graphs has nothing to do."""
+    import inferllm_amd as I
+    from inferllm_amd import StepEntry
+    config = CONFIGS["B"]
+    d = make_model_dir(tmp_path, config, seed=31, dtype=torch.bfloat16, gain=4.0)
+    reqs = requests_for(config, [9, 14, 5, 11, 7], seed=4)
+
+    def run(warm):
+        eng = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=8, poison_freed=True)
+        if warm:
+            assert eng.warm_up([1, 5, 6, 8], longest=40) == 2           # graphs of 1 and of 8 rows
+            assert eng.warm_up([5]) == 0                               # there already
+            before = dict(eng.runner._graphs)
+        slots = [eng.alloc_slot() for _ in reqs]
+        eng.step([StepEntry(s, r[:-3], []) for s, r in zip(slots, reqs)])
+        outs = [eng.step([StepEntry(s, [r[len(r) - 3 + t]], [0]) for s, r in zip(slots, reqs)]).clone()
+                for t in range(3)]
+        if warm:
+            assert eng.runner._graphs.keys() == before.keys()
+        return outs
+
+    cold, warm = run(False), run(True)
+    for a, b in zip(cold, warm):
+        assert torch.equal(a, b)
+    eager = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=8, use_graphs=False)
+    assert eager.warm_up() == 0
+
+
 def test_head_size_80_in_bfloat16(tmp_path_factory):
     """A LLaMA of width 2560 with 32 heads of 80 (grouped in fours), a head size that is no
     multiple of 32: the matrix-core prompt kernel with its last block of dims half used, the
