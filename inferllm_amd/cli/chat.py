@@ -12,9 +12,10 @@ reference exits 0 silently, chat.cpp:98-100), and `-n/--n_predict` is honoured
 
 Prompts are token ids (`--prompt-ids "1,5,9"`, or `--prompt-ids-file` with one
 request per line: the lines form a batch), or text (`-p/--prompt`) when the model
-folder has a tokenizer.json.  Without a prompt the program reads requests from
-standard input, one per line, like the reference's interactive loop
-(chat.cpp:221-275), until end of input.
+folder has a tokenizer.json.  Without a prompt the program reads the turns of one
+conversation from standard input, one per line, like the reference's interactive
+loop (chat.cpp:221-275): every turn goes on from what was said before, until the
+context is full or the input ends.
 """
 from __future__ import annotations
 
@@ -168,15 +169,34 @@ def main(argv=None) -> int:
     if prompts:
         run(prompts)
         return 0
-    for line in sys.stdin:                       # one request per line until end of input
-        line = line.strip()
-        if not line:
-            continue
-        try:
-            ids = parse_ids(line)
-        except ValueError:
-            ids = text.encode(line, eng.spec.bos_token_id)
-        run([ids])
+    # No prompt: turns from standard input, one a line, in ONE context that goes on from turn to
+    # turn until it is full or the input ends, like the reference's loop (chat.cpp:221-275).
+    with eng.session(temperature=args.temp, top_k=args.top_k, top_p=args.top_p,
+                     repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n,
+                     seed=seed, stop_token_ids=stops) as talk:
+        eng.warm_up([1], args.ctx_size)
+        first = True
+        for line in sys.stdin:
+            line = line.strip()
+            if not line:
+                continue
+            try:
+                ids = parse_ids(line)
+            except ValueError:
+                ids = text.encode(line, eng.spec.bos_token_id if first else None)
+            if len(ids) + 1 > talk.remaining:
+                print(f"chat: the context is full ({talk.remaining} tokens left)", file=sys.stderr)
+                break
+            first = False
+            if text.tok is None:
+                out = talk.say(ids, args.n_predict, on_token=lambda t: print(t, end=" ", flush=True))
+                print(flush=True)
+            else:
+                print(text.show(talk.say(ids, args.n_predict)), flush=True)
+            if args.summary:
+                print(talk.last_stats.summary(), file=sys.stderr, flush=True)
+            if talk.remaining <= 0:
+                break
     return 0
 
 

@@ -175,6 +175,18 @@ class Engine:
         """See `StepRunner.step`.  The returned tensor is valid until the next step."""
         return self.runner.step(entries, device_tokens)
 
+    def session(self, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0,
+                repeat_penalty: float = 1.0, repeat_last_n: int = 64, seed: int = 0,
+                stop_token_ids: Optional[Sequence[int]] = None):
+        """A conversation in one slot of the cache: `say(tokens)` feeds a turn after everything
+        said so far and returns the answer, as the reference's chat keeps one context over its
+        turns (application/chat.cpp:221-275).  Close it (or use it in a `with`) to give the slot
+        back."""
+        from .session import Session
+        params = SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p,
+                                repeat_penalty=repeat_penalty, repeat_last_n=repeat_last_n, seed=seed)
+        return Session(self, params, stop_token_ids)
+
     def warm_up(self, batch_sizes: Optional[Sequence[int]] = None, longest: int = 1) -> int:
         """Capture the decode graphs for these numbers of sequences (default: every size up to
         `max_batch` that has a graph of its own) with contexts up to `longest` keys, so that the

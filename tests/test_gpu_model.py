@@ -464,6 +464,80 @@ def test_command_line_generates_like_the_plain_model(tmp_path):
     assert bad.returncode == 2 and "does not fit" in bad.stderr
 
 
+def test_a_session_keeps_one_context_over_its_turns(tmp_path):
+    """`Engine.session`: turns fed one after another into one slot give the tokens that the plain
+    model gives for the whole conversation; an answer cut by `max_new_tokens` leaves its last
+    token to be fed with the next turn, a stop token ends a turn and is never fed; the context's
+    end and the slot's return are kept track of."""
+    import inferllm_amd as I
+    config = CONFIGS["A"]
+    d = make_model_dir(tmp_path, config, seed=17, dtype=torch.float32, gain=4.0)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="float32", device=DEV, max_batch=2, max_seq_len=48, poison_freed=True)
+    turns = requests_for(config, [9, 4, 3], seed=6)
+    seen = []
+    with eng.session(stop_token_ids=[]) as talk:
+        said = list(turns[0])
+        a1 = talk.say(turns[0], max_new_tokens=5, on_token=seen.append)
+        assert a1 == plain_llama.generate_greedy(config, w, said, 5) and seen == a1
+        assert talk.length == len(said) + 4 and talk.remaining == 48 - len(said) - 5     # the fifth is not fed yet
+        said += a1 + list(turns[1])
+        a2 = talk.say(turns[1], max_new_tokens=3)
+        assert a2 == plain_llama.generate_greedy(config, w, said, 3)
+        said += a2
+        assert talk.last_stats.prompt_tokens == 1 + len(turns[1]) and talk.last_stats.generated_tokens == 3
+        with pytest.raises(ValueError, match="do not fit"):
+            talk.say([1] * 40)
+        assert talk.length == len(said) - 1                        # nothing was fed by the refused turn
+        slot = talk.slot
+    assert talk.slot is None
+    both = [eng.alloc_slot(), eng.alloc_slot()]                     # the slot is free again
+    assert slot in both
+    for s_ in both:
+        eng.free_slot(s_)
+    eng.cache.check()
+    with pytest.raises(ValueError, match="closed"):
+        talk.say([1])
+    # a stop token: a token of the first answer that none before it equals ends the turn; it is
+    # not returned and not fed
+    j = next(j for j in range(1, 5) if a1[j] not in a1[:j])
+    stop = a1[j]
+    with eng.session(stop_token_ids=[stop]) as talk:
+        b1 = talk.say(turns[0], max_new_tokens=5)
+        assert b1 == a1[:j] and talk.length == len(turns[0]) + j
+        said = list(turns[0]) + b1 + list(turns[2])
+        b2 = talk.say(turns[2], max_new_tokens=4, include_stop=True)
+        want = plain_llama.generate_greedy(config, w, said, 4, [stop])
+        assert b2[:len(want)] == want and (len(want) == 4 or b2[len(want)] == stop)
+    # the context's end: generation stops when nothing more fits, the rest of the answer is cut
+    with eng.session(stop_token_ids=[]) as talk:
+        out = talk.say(requests_for(config, [40], seed=8)[0], max_new_tokens=100)
+        assert len(out) == 9 and talk.length == 48 and talk.remaining == -1    # the ninth cannot be fed any more
+    eng.cache.check()
+
+
+def test_command_line_turns_from_standard_input_share_one_context(tmp_path):
+    """`bin/chat` without a prompt: the lines of standard input are turns of one conversation,
+    as in the reference's loop."""
+    import os
+    import subprocess
+    import sys
+    config = CONFIGS["A"]
+    d = make_model_dir(tmp_path, config, seed=7, dtype=torch.float32, gain=4.0)
+    w = read_weights(d)
+    turns = requests_for(config, [6, 3], seed=5)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "chat"), "-m", d, "-d", "float32", "--temp", "0",
+                        "-n", "4", "-c", "64", "--stop-ids", "100000"],
+                       input="\n".join(" ".join(map(str, t)) for t in turns) + "\n",
+                       capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0, r.stderr
+    got = [[int(t) for t in line.split()] for line in r.stdout.strip().splitlines()]
+    first = plain_llama.generate_greedy(config, w, turns[0], 4)
+    second = plain_llama.generate_greedy(config, w, list(turns[0]) + first + list(turns[1]), 4)
+    assert got == [first, second]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_prompt_then_decoding_at_head_size_128(tmp_path_factory, dtype):
     """1,500 tokens in one step (many query blocks, key tiles and pages), then 40 tokens one by
