@@ -159,7 +159,7 @@ class Bench:
         frac = self.step_bytes(batch, mean_ctx) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
         return batch * steps / dt, ms, frac
 
-    def prefill_run(self, T=2048, reps=3):
+    def prefill_run(self, T=2048, reps=6):
         from inferllm_amd import StepEntry
         from inferllm_amd.kernels import ops
         torch, eng = self.torch, self.eng
