@@ -7,10 +7,10 @@
 from . import models  # registers the architectures
 from .config import (ConfigError, config_from_dict, load_config, register_architecture,
                      registered_architectures)
-from .engine import Engine, StepEntry, StepError
+from .engine import Engine, Session, StepEntry, StepError
 from .sampling import SamplingParams
 from .weights import WeightsError, write_random_model
 
-__all__ = ["Engine", "StepEntry", "StepError", "SamplingParams", "ConfigError", "WeightsError",
+__all__ = ["Engine", "Session", "StepEntry", "StepError", "SamplingParams", "ConfigError", "WeightsError",
            "config_from_dict", "load_config", "register_architecture", "registered_architectures",
            "write_random_model"]
