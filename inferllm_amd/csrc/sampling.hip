@@ -69,8 +69,36 @@ __device__ __forceinline__ T block_exclusive_scan(T v, T* red, T* total) {
 
 // Walks of a row by one block wait for each load in turn unless several are asked for at once:
 // these bring eight values at a time, all loads issued before the first is used.
+typedef float sample_f32x4_t __attribute__((ext_vector_type(4)));
+
 template <typename F>
 __device__ __forceinline__ void each_strided8(const float* a, int n, int tid, F f) {
+    if ((((size_t)a) & 15) == 0) {
+        // 16 bytes a load where the row starts at a multiple of 16 bytes (the same for the whole
+        // block): four loads of four values in flight a thread, a quarter of the trips
+        const int n4 = n >> 2;
+        const sample_f32x4_t* a4 = (const sample_f32x4_t*)a;
+        for (int base = tid; base < n4; base += SB * 4) {
+            sample_f32x4_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i4 = base + u * SB;
+                v[u] = i4 < n4 ? a4[i4] : (sample_f32x4_t){0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i4 = base + u * SB;
+                if (i4 < n4) {
+                    f(4 * i4, v[u][0]);
+                    f(4 * i4 + 1, v[u][1]);
+                    f(4 * i4 + 2, v[u][2]);
+                    f(4 * i4 + 3, v[u][3]);
+                }
+            }
+        }
+        for (int i = 4 * n4 + tid; i < n; i += SB) f(i, a[i]);
+        return;
+    }
     for (int base = tid; base < n; base += SB * 8) {
         float v[8];
 #pragma unroll
@@ -503,29 +531,60 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
     mx = block_max(mx, red_f);
     // kept: key > prefix, and the first krem ids (ascending) with key == prefix
 
-    // 3. the kept ids and scores in id order into LDS
-    const int chunk = (V + SB - 1) / SB;
-    const int lo = min(V, tid * chunk), hi = min(V, lo + chunk);
-    int n_eq = 0, n_gt = 0;
-    each_in_order8(s, lo, hi, [&](int, float v) {
+    // 3. the kept ids and scores in id order into LDS.  A wave walks its own stretch of the row,
+    // 64 consecutive ids an instruction (a thread walking a stretch of its own would touch 64
+    // cache lines an instruction); within an instruction the lanes are in id order, so counts
+    // and places come from ballots.
+    const int lane = tid & (ILLM_WAVE - 1);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const int stretch = ((V + NW - 1) / NW + ILLM_WAVE - 1) / ILLM_WAVE * ILLM_WAVE;
+    const int lo = min(V, wave * stretch), hi = min(V, lo + stretch);
+    auto walk = [&](auto f) __attribute__((always_inline)) {
+        for (int base = lo; base < hi; base += 8 * ILLM_WAVE) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = base + u * ILLM_WAVE + lane;
+                v[u] = i < hi ? s[i] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = base + u * ILLM_WAVE + lane;
+                f(i, v[u], i < hi);
+            }
+        }
+    };
+    int n_eq = 0, n_gt = 0;                             // of the wave's stretch (the same in all its lanes)
+    walk([&](int, float v, bool in) {
         const uint32_t key = order_key(v);
-        n_gt += key > prefix ? 1 : 0;
-        n_eq += key == prefix ? 1 : 0;
+        n_gt += __popcll(__ballot(in && key > prefix));
+        n_eq += __popcll(__ballot(in && key == prefix));
     });
-    int total_i;
-    const int eq_before = block_exclusive_scan<int>(n_eq, red_i, &total_i);
-    const int eq_take = max(0, min(n_eq, krem - eq_before));
-    const int at0 = block_exclusive_scan<int>(n_gt + eq_take, red_i, &total_i);
-    const int n_kept = total_i;                        // == top_k
-    {
-        int at = at0, eq_left = eq_take;
-        each_in_order8(s, lo, hi, [&](int i, float v) {
-            const uint32_t key = order_key(v);
-            bool take = key > prefix;
-            if (key == prefix && eq_left > 0) { take = true; --eq_left; }
-            if (take && at < SB) { cand_id[at] = i; cand_s[at] = v; ++at; }
-        });
+    __syncthreads();
+    if (lane == 0) { red_i[wave] = n_eq; hist[0][wave] = n_gt; }
+    __syncthreads();
+    int eq_before = 0;
+    for (int w = 0; w < wave; ++w) eq_before += red_i[w];
+    int eq_left = max(0, min(n_eq, krem - eq_before));  // ids with the k-th key this wave still takes
+    int at = 0, n_kept = 0;                             // where the wave's first kept id goes; all kept (== top_k)
+    for (int w = 0, eb = 0; w < NW; ++w) {
+        const int took = hist[0][w] + max(0, min(red_i[w], krem - eb));
+        if (w < wave) at += took;
+        n_kept += took;
+        eb += red_i[w];
     }
+    __syncthreads();
+    walk([&](int i, float v, bool in) {
+        const uint32_t key = order_key(v);
+        const bool eq = in && key == prefix;
+        const unsigned long long eq_mask = __ballot(eq);
+        const bool take = (in && key > prefix) || (eq && __popcll(eq_mask & below) < eq_left);
+        const unsigned long long take_mask = __ballot(take);
+        const int to = at + __popcll(take_mask & below);
+        if (take && to < SB) { cand_id[to] = i; cand_s[to] = v; }
+        at += __popcll(take_mask);
+        eq_left -= min(eq_left, __popcll(eq_mask));
+    });
     __syncthreads();
 
     // 4. top_p: an id stays if the mass before it in descending order (ties: lower id first)
