@@ -749,19 +749,21 @@ def test_head_size_80_in_bfloat16(tmp_path_factory):
     eng.cache.check()
 
 
-def test_real_layer_sizes_with_many_sequences(tmp_path_factory, monkeypatch):
-    """Two layers of the LLaMA-2-7B sizes with 40, then 25 sequences decoding together: steps of
+@pytest.mark.parametrize("nkv,ffn", [(32, 11008), (8, 14336)])
+def test_real_layer_sizes_with_many_sequences(tmp_path_factory, monkeypatch, nkv, ffn):
+    """Two layers of the LLaMA-2-7B sizes (and of the LLaMA-3-8B ones: heads grouped in fours, a
+    q|k|v matrix of 6144 rows) with 40, then 25 sequences decoding together: steps of
     17 to 128 rows take the kernels that share X through LDS (fused q|k|v with rotation and
     store, gate|up with SiLU-multiply, o and down as planes, the head) from graphs of 48 and of
     32 rows, and no product of such a step goes to the vendor GEMM."""
     import inferllm_amd as I
     from inferllm_amd import StepEntry
-    config = {"architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "intermediate_size": 11008,
-              "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 32,
+    config = {"architectures": ["LlamaForCausalLM"], "hidden_size": 4096, "intermediate_size": ffn,
+              "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": nkv,
               "vocab_size": 32000, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
               "max_position_embeddings": 512, "tie_word_embeddings": False,
               "bos_token_id": 1, "eos_token_id": 2}
-    d = make_model_dir(tmp_path_factory.getbasetemp(), config, seed=12, dtype=torch.bfloat16, gain=2.0)
+    d = make_model_dir(tmp_path_factory.getbasetemp() / f"many{nkv}", config, seed=12, dtype=torch.bfloat16, gain=2.0)
     w = read_weights(d)
     eng = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=40, max_seq_len=64,
                                    poison_freed=True)
