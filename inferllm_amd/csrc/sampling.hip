@@ -448,9 +448,67 @@ sample_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
 // (4 passes of 8 bits, histograms per wave in LDS), the kept ids gathered in id order into LDS,
 // top_p decided per kept id from the mass that lies before it in descending order, the draw by
 // inverse CDF over what is left.  Ties at the k-th value and at the top_p cut go to the lower ids.
+// PART: the block takes one of gridDim.x stretches of the row (grid (parts, B)) and leaves its
+// top_k ids (global numbers, ascending) and their scores behind the rows' scores in `scratch`
+// for `sample_topk_merge_kernel`: a row is then the work of several compute units instead of
+// one, whose instruction issue bounds a block (top_k <= TOPK_PARTS_MAX_K, long rows).
+#define TOPK_PARTS_MAX_K 64
+#define TOPK_MAX_PARTS (SB / TOPK_PARTS_MAX_K)
+
+// What a row's parts leave for the merge, in the second plane of `scratch` (floats; B rows of V
+// before it): per part its count, then TOPK_PARTS_MAX_K scores, then as many ids.
+__device__ __forceinline__ float* topk_part_slot(float* scratch, int B, int V, int b, int part) {
+    return scratch + ((size_t)B + b) * V + (size_t)part * (1 + 2 * TOPK_PARTS_MAX_K);
+}
+
+// top_p over the n_kept candidates in cand_id / cand_s (ascending ids, one a thread), then the
+// draw: steps 4 and 5 of the kernel below.
+__device__ __forceinline__ void topk_finish(const int* cand_id, const float* cand_s, int n_kept,
+                                            float top_p, uint64_t seed, int counter, float* red_f,
+                                            int* sh_i, int32_t* out_b) {
+    const int tid = threadIdx.x;
+    const bool have = tid < n_kept;
+    const float my_s = have ? cand_s[tid] : -INFINITY;
+    const float mx = block_max(my_s, red_f);            // the largest score is among the kept
+    // 4. top_p: an id stays if the mass before it in descending order (ties: lower id first)
+    // does not yet reach top_p of the whole kept mass
+    const float my_p = have ? expf(my_s - mx) : 0.f;
+    bool stay = have;
+    if (top_p < 1.0f) {
+        const float z = block_sum_t<float>(my_p, red_f);
+        const float need = top_p * z;
+        if (have) {
+            float before = 0.f;
+            const uint32_t my_key = order_key(my_s);
+            for (int j = 0; j < n_kept; ++j) {
+                const uint32_t kj = order_key(cand_s[j]);
+                if (kj > my_key || (kj == my_key && j < tid)) before += expf(cand_s[j] - mx);
+            }
+            stay = before < need;
+        }
+    }
+    // 5. inverse CDF over what stays, in ascending id order (the order of the list)
+    const float mine = stay ? my_p : 0.f;
+    float total;
+    const float before = block_exclusive_scan<float>(mine, red_f, &total);
+    const float target = uniform_from(seed, counter) * total;
+    __syncthreads();
+    if (tid == 0) *sh_i = -1;
+    __syncthreads();
+    if (mine > 0.f && target >= before && target < before + mine) atomicMax(sh_i, cand_id[tid]);
+    __syncthreads();
+    if (*sh_i < 0) {
+        // rounding put the target past the last id that stays: take that id
+        if (stay) atomicMax(sh_i, cand_id[tid]);
+        __syncthreads();
+    }
+    if (tid == 0) *out_b = *sh_i < 0 ? 0 : *sh_i;
+}
+
+template <bool PART>
 __global__ void __launch_bounds__(SB)
 sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
-                   int32_t* __restrict__ out, int V, float temp, int top_k, float top_p,
+                   int32_t* __restrict__ out, int Vrow, float temp, int top_k, float top_p,
                    float repeat_penalty, const int32_t* __restrict__ last_tokens, int n_last,
                    const uint64_t* __restrict__ seeds, const int32_t* __restrict__ counters) {
     constexpr int NW = SB / ILLM_WAVE;
@@ -461,38 +519,45 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
     __shared__ int sh_d, sh_above, sh_i;
     __shared__ int cand_id[SB];
     __shared__ float cand_s[SB];
-    const int b = blockIdx.x, tid = threadIdx.x, wave = tid / ILLM_WAVE;
-    const float* row = logits + (size_t)b * V;
-    float* s = scratch + (size_t)b * V;
+    const int b = PART ? blockIdx.y : blockIdx.x, tid = threadIdx.x, wave = tid / ILLM_WAVE;
+    // the ids this block looks at: [first, first + V) of the row's Vrow
+    const int stretch_ids = PART ? ((Vrow + (int)gridDim.x - 1) / (int)gridDim.x + 3) / 4 * 4 : Vrow;
+    const int first = PART ? min(Vrow, (int)blockIdx.x * stretch_ids) : 0;
+    const int V = PART ? min(stretch_ids, Vrow - first) : Vrow;
+    const float* row = logits + (size_t)b * Vrow + first;
+    float* s = scratch + (size_t)b * Vrow + first;
     const int nl = last_tokens ? min(n_last, 256) : 0;
     if (tid < nl) last[tid] = last_tokens[(size_t)b * n_last + tid];
+    if (PART && V <= 0) {                               // (no ids left for this part)
+        if (tid == 0) *(int*)topk_part_slot(scratch, gridDim.y, Vrow, b, blockIdx.x) = 0;
+        return;
+    }
+    top_k = min(top_k, V);
 
     // 1. scaled scores; then the penalty, once for every id of the window
     const float inv_temp = 1.0f / temp;
     each_strided8(row, V, tid, [&](int i, float v) { s[i] = v * inv_temp; });
     __syncthreads();
     if (tid < nl) {
-        const int id = last[tid];
-        bool first = id >= 0 && id < V;
-        for (int j = 0; j < tid; ++j) first = first && last[j] != id;
-        if (first) {
+        const int id = last[tid] - first;
+        bool once = last[tid] >= 0 && id >= 0 && id < V;     // in this block's ids, and not named before
+        for (int j = 0; j < tid; ++j) once = once && last[j] != last[tid];
+        if (once) {
             const float l = row[id], v = l * inv_temp;
             s[id] = l < 0.f ? v * repeat_penalty : v / repeat_penalty;
         }
     }
     __syncthreads();
 
-    // 2. the key of the top_k-th largest score, 8 bits a pass; the largest score on the way
+    // 2. the key of the top_k-th largest score, 8 bits a pass
     uint32_t prefix = 0;
     int krem = top_k;
-    float mx = -INFINITY;
     for (int pass = 0; pass < 4; ++pass) {
         const int shift = 24 - 8 * pass;
         const uint32_t hi_mask = pass ? (0xffffffffu << (shift + 8)) : 0u;
         for (int i = tid; i < NW * 256; i += SB) (&hist[0][0])[i] = 0;
         __syncthreads();
         each_strided8(s, V, tid, [&](int, float v) {
-            if (pass == 0) mx = fmaxf(mx, v);
             const uint32_t key = order_key(v);
             if ((key & hi_mask) == prefix) atomicAdd(&hist[wave][(key >> shift) & 255u], 1);
         });
@@ -528,7 +593,6 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
         krem -= sh_above;
         __syncthreads();
     }
-    mx = block_max(mx, red_f);
     // kept: key > prefix, and the first krem ids (ascending) with key == prefix
 
     // 3. the kept ids and scores in id order into LDS.  A wave walks its own stretch of the row,
@@ -587,42 +651,71 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
     });
     __syncthreads();
 
-    // 4. top_p: an id stays if the mass before it in descending order (ties: lower id first)
-    // does not yet reach top_p of the whole kept mass
-    const bool have = tid < n_kept;
-    const float my_s = have ? cand_s[tid] : -INFINITY;
-    const float my_p = have ? expf(my_s - mx) : 0.f;
-    bool stay = have;
-    if (top_p < 1.0f) {
-        const float z = block_sum_t<float>(my_p, red_f);
-        const float need = top_p * z;
-        if (have) {
-            float before = 0.f;
-            const uint32_t my_key = order_key(my_s);
-            for (int j = 0; j < n_kept; ++j) {
-                const uint32_t kj = order_key(cand_s[j]);
-                if (kj > my_key || (kj == my_key && j < tid)) before += expf(cand_s[j] - mx);
-            }
-            stay = before < need;
+    if (PART) {
+        // the part's kept ids (global numbers) and scores for the merge
+        float* slot = topk_part_slot(scratch, gridDim.y, Vrow, b, blockIdx.x);
+        if (tid == 0) *(int*)slot = n_kept;
+        if (tid < n_kept) {
+            slot[1 + tid] = cand_s[tid];
+            ((int*)slot)[1 + TOPK_PARTS_MAX_K + tid] = first + cand_id[tid];
+        }
+        return;
+    }
+    topk_finish(cand_id, cand_s, n_kept, top_p, seeds[b], counters[b], red_f, &sh_i, out + b);
+}
+
+// The parts' kept ids of a row (at most SB together, in ascending id order part after part):
+// the top_k of them by score (ties: the lower id), then top_p and the draw as above.
+__global__ void __launch_bounds__(SB)
+sample_topk_merge_kernel(float* __restrict__ scratch, int32_t* __restrict__ out, int V, int parts,
+                         int top_k, float top_p, const uint64_t* __restrict__ seeds,
+                         const int32_t* __restrict__ counters) {
+    constexpr int NW = SB / ILLM_WAVE;
+    __shared__ float red_f[NW];
+    __shared__ int red_i[NW];
+    __shared__ int sh_i;
+    __shared__ int cand_id[SB];
+    __shared__ float cand_s[SB];
+    __shared__ int part_at[TOPK_MAX_PARTS + 1];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    if (tid == 0) {
+        int at = 0;
+        for (int p = 0; p < parts; ++p) {
+            part_at[p] = at;
+            at += *(const int*)topk_part_slot(scratch, gridDim.x, V, b, p);
+        }
+        part_at[parts] = at;
+    }
+    __syncthreads();
+    const int n_all = part_at[parts];
+    {
+        const int p = tid / TOPK_PARTS_MAX_K, j = tid % TOPK_PARTS_MAX_K;
+        if (p < parts && j < part_at[p + 1] - part_at[p]) {
+            const float* slot = topk_part_slot(scratch, gridDim.x, V, b, p);
+            cand_s[part_at[p] + j] = slot[1 + j];
+            cand_id[part_at[p] + j] = ((const int*)slot)[1 + TOPK_PARTS_MAX_K + j];
         }
     }
-
-    // 5. inverse CDF over what stays, in ascending id order (the order of the list)
-    const float mine = stay ? my_p : 0.f;
-    float total;
-    const float before = block_exclusive_scan<float>(mine, red_f, &total);
-    const float target = uniform_from(seeds[b], counters[b]) * total;
     __syncthreads();
-    if (tid == 0) sh_i = -1;
-    __syncthreads();
-    if (mine > 0.f && target >= before && target < before + mine) atomicMax(&sh_i, cand_id[tid]);
-    __syncthreads();
-    if (sh_i < 0) {
-        // rounding put the target past the last id that stays: take that id
-        if (stay) atomicMax(&sh_i, cand_id[tid]);
-        __syncthreads();
+    // a candidate's place in descending order of score, the lower id first among equals
+    const bool have = tid < n_all;
+    const float my_s = have ? cand_s[tid] : 0.f;
+    const int my_id = have ? cand_id[tid] : 0;
+    int rank = 0;
+    if (have) {
+        const uint32_t my_key = order_key(my_s);
+        for (int j = 0; j < n_all; ++j) {
+            const uint32_t kj = order_key(cand_s[j]);
+            rank += (kj > my_key || (kj == my_key && j < tid)) ? 1 : 0;
+        }
     }
-    if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
+    const bool keep = have && rank < top_k;
+    int n_kept;
+    const int to = block_exclusive_scan<int>(keep ? 1 : 0, red_i, &n_kept);
+    __syncthreads();
+    if (keep) { cand_id[to] = my_id; cand_s[to] = my_s; }
+    __syncthreads();
+    topk_finish(cand_id, cand_s, n_kept, top_p, seeds[b], counters[b], red_f, &sh_i, out + b);
 }
 
 extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V,
@@ -633,8 +726,19 @@ extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, in
         n_last < 0 || n_last > 256 || !seeds || !counters || !scratch)
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;
-    if (top_k > 0 && top_k <= SB && top_k < V)
-        hipLaunchKernelGGL(sample_topk_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
+    if (top_k > 0 && top_k <= TOPK_PARTS_MAX_K && V >= 65536 && B <= 65535) {
+        // a row in parts of 4,096 ids or more, about 512 blocks in all, then the merge (at 32,000
+        // ids the second launch costs what the parts save: 60 us against 52)
+        int parts = V / 4096;
+        parts = parts > TOPK_MAX_PARTS ? TOPK_MAX_PARTS : parts;
+        while (parts > 2 && parts * B > 512) parts /= 2;
+        hipLaunchKernelGGL(sample_topk_kernel<true>, dim3(parts, B), dim3(SB), 0, (hipStream_t)stream,
+                           logits, scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens,
+                           n_last, seeds, counters);
+        hipLaunchKernelGGL(sample_topk_merge_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, scratch,
+                           out, V, parts, top_k, top_p, seeds, counters);
+    } else if (top_k > 0 && top_k <= SB && top_k < V)
+        hipLaunchKernelGGL(sample_topk_kernel<false>, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
                            scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
                            seeds, counters);
     else if (V <= SAMPLE_REG_IDS * SB)

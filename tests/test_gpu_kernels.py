@@ -847,7 +847,10 @@ def test_the_uniform_numbers_of_the_tests_and_of_the_host_side_agree():
     (32000, 1.0, 0, 0.9, 1.0), (300, 0.7, 1, 1.0, 1.0), (128256, 0.9, 50, 0.8, 1.2),
     (2000, 0.9, 1024, 0.7, 1.1), (2000, 0.9, 1025, 0.7, 1.0), (50, 1.0, 49, 0.5, 1.0), (32000, 0.1, 40, 0.95, 1.1),
     # rows too long for a thread's registers: top_p alone, with a large top_k, temperature alone
-    (128256, 0.9, 0, 0.8, 1.2), (40000, 1.0, 2000, 0.6, 1.0), (33000, 0.7, 0, 0.999, 1.0), (50000, 1.3, 0, 1.0, 1.0)])
+    (128256, 0.9, 0, 0.8, 1.2), (40000, 1.0, 2000, 0.6, 1.0), (33000, 0.7, 0, 0.999, 1.0), (50000, 1.3, 0, 1.0, 1.0),
+    # long rows with a small top_k are cut into parts that blocks of their own take: a length that
+    # no part divides, the largest top_k of that way and the first beyond it
+    (70001, 0.1, 40, 0.95, 1.1), (65536, 1.0, 64, 0.5, 1.0), (65536, 1.0, 65, 0.5, 1.3), (200003, 0.8, 3, 1.0, 1.3)])
 def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top_p, penalty):
     uniform = R.uniform                                      # the tests' own statement of the hash
     B = 6
@@ -865,6 +868,26 @@ def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top
                            last[b] if penalty != 1.0 else None), (b, got[b], u)
     if top_k == 1:
         assert got == torch.argmax(logits, -1).tolist() or penalty != 1.0
+
+
+def test_sample_of_a_long_row_in_parts_keeps_what_one_block_would():
+    """A long row with a small top_k is the work of several blocks, each with a stretch of the ids.
+    Equal scores at the k-th place go to the lower ids, wherever the stretches' edges lie: of 90 equal
+    scores spread over the whole row, the 40 with the lowest ids are kept, and every draw is one of them."""
+    V, B, top_k = 131072, 64, 40
+    logits = rnd(B, V, seed=21, std=1.0).clamp_(max=3.0)
+    high = torch.arange(90) * 1451 + 7                        # up to id 129,146: in every stretch
+    logits[:, high] = 9.0
+    logits[1, high[:5]] = 12.0                                # row 1: five above, then 35 of the 85 equal ones
+    seeds = torch.arange(B, dtype=torch.int64) * 104729 + 3
+    counters = torch.arange(B, dtype=torch.int32)
+    got = ops().sample(logits.to(DEV), 1.0, top_k, 1.0, 1.0, None, seeds.to(DEV), counters.to(DEV)).cpu()
+    kept = set(high[:top_k].tolist())
+    assert all(int(t) in kept for t in got), [int(t) for t in got if int(t) not in kept]
+    assert len({int(t) for t in got}) > 20                    # and not always the same few
+    for b in range(B):
+        u = R.uniform(int(seeds[b]), int(counters[b]))
+        assert interval_ok(logits[b], int(got[b]), u, 1.0, top_k, 1.0, 1.0, None), (b, int(got[b]), u)
 
 
 def test_sample_frequencies_match_probabilities():
