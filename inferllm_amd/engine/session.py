@@ -56,7 +56,7 @@ class Session:
     @property
     def remaining(self) -> int:
         """Tokens that still fit into the context (fed or generated)."""
-        return self.engine.max_seq_len - self.length - (1 if self._unfed is not None else 0)
+        return max(0, self.engine.max_seq_len - self.length - (1 if self._unfed is not None else 0))
 
     def _open(self) -> None:
         if self.slot is None:
@@ -100,12 +100,14 @@ class Session:
                              f"the context are left")
         stats = self.last_stats = GenerationStats(prompt_tokens=len(feed), batches=1)
         sync = lambda: torch.cuda.synchronize(self.engine.device)
-        self.history.extend(turn)
-        self._unfed = None
         out: List[int] = []
         sync()
         start = time.perf_counter()
+        # (a step that the cache has no room for raises before it changes anything: the session
+        # stays as it was)
         logits = self.engine.step([StepEntry(self.slot, feed, [len(feed) - 1])])
+        self.history.extend(turn)
+        self._unfed = None
         token = self._draw(logits)
         sync()
         stats.prefill_seconds = time.perf_counter() - start

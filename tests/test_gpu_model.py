@@ -512,8 +512,22 @@ def test_a_session_keeps_one_context_over_its_turns(tmp_path):
     # the context's end: generation stops when nothing more fits, the rest of the answer is cut
     with eng.session(stop_token_ids=[]) as talk:
         out = talk.say(requests_for(config, [40], seed=8)[0], max_new_tokens=100)
-        assert len(out) == 9 and talk.length == 48 and talk.remaining == -1    # the ninth cannot be fed any more
+        assert len(out) == 9 and talk.length == 48 and talk.remaining == 0     # the ninth cannot be fed any more
     eng.cache.check()
+    # no pages left for a turn: the error leaves the session as it was, and the turn goes
+    # through once another session has given its pages back
+    from inferllm_amd.cache import CacheFull
+    eng = I.Engine.from_pretrained(d, dtype="float32", device=DEV, max_batch=2, max_tokens=128, poison_freed=True)
+    first, second = eng.session(stop_token_ids=[]), eng.session(stop_token_ids=[])
+    first.say(requests_for(config, [70], seed=3)[0], max_new_tokens=2)       # both pages
+    with pytest.raises(CacheFull):
+        second.say(turns[0], max_new_tokens=5)
+    assert second.length == 0 and second.history == [] and second.remaining == eng.max_seq_len
+    first.close()
+    assert second.say(turns[0], max_new_tokens=5) == a1
+    second.close()
+    eng.cache.check()
+    assert eng.cache.slots.n_held() == 0
 
 
 def test_command_line_turns_from_standard_input_share_one_context(tmp_path):
