@@ -12,8 +12,8 @@ reference exits 0 silently, chat.cpp:98-100), and `-n/--n_predict` is honoured
 
 Prompts are token ids (`--prompt-ids "1,5,9"`, or `--prompt-ids-file` with one
 request per line: the lines form a batch), or text (`-p/--prompt`) when the model
-folder has a tokenizer.json.  Without a prompt the program reads the turns of one
-conversation from standard input, one per line, like the reference's interactive
+folder has a tokenizer.json or a tokenizer.model.  Without a prompt the program reads the
+turns of one conversation from standard input, one per line, like the reference's interactive
 loop (chat.cpp:221-275): every turn goes on from what was said before, until the
 context is full or the input ends.
 """
@@ -49,7 +49,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--mmap", action="store_true",
                     help="accepted for compatibility; safetensors files are always memory-mapped")
     ap.add_argument("-n", "--n_predict", type=int, default=128, help="new tokens to predict (default: 128)")
-    ap.add_argument("-p", "--prompt", default=None, help="text prompt (needs tokenizer.json in the model folder)")
+    ap.add_argument("-p", "--prompt", default=None, help="text prompt (needs tokenizer.json or tokenizer.model in the model folder)")
     ap.add_argument("--prompt-ids", default=None, help='prompt as token ids, e.g. "1,5,9"')
     ap.add_argument("--prompt-ids-file", default=None, help="file with one request (token ids) per line")
     ap.add_argument("--stop-ids", default=None, help="stop token ids (default: the model's eos ids)")
@@ -72,24 +72,35 @@ def parse_ids(text: str) -> List[int]:
 
 
 class _Text:
-    """Text in and out through the folder's tokenizer.json, if there is one."""
+    """Text in and out through the folder's tokenizer.json or, without one, its tokenizer.model
+    (a SentencePiece model, as LLaMA-2 checkpoints bring it), if there is either."""
 
     def __init__(self, model_dir: Optional[str]):
-        self.tok = None
+        self.tok = self.pieces = None
         path = os.path.join(model_dir, "tokenizer.json") if model_dir else None
+        spm = os.path.join(model_dir, "tokenizer.model") if model_dir else None
         if path and os.path.isfile(path):
             from tokenizers import Tokenizer
             self.tok = Tokenizer.from_file(path)
+        elif spm and os.path.isfile(spm):
+            from sentencepiece import SentencePieceProcessor
+            self.pieces = SentencePieceProcessor(model_file=spm)
 
     def encode(self, text: str, bos: Optional[int]) -> List[int]:
-        if self.tok is None:
-            raise SystemExit("text prompts need a tokenizer.json in the model folder; use --prompt-ids")
-        ids = self.tok.encode(text, add_special_tokens=False).ids
+        if self.tok is not None:
+            ids = self.tok.encode(text, add_special_tokens=False).ids
+        elif self.pieces is not None:
+            ids = list(self.pieces.encode(text))
+        else:
+            raise SystemExit("text prompts need a tokenizer.json or a tokenizer.model in the model "
+                             "folder; use --prompt-ids")
         return ([bos] if bos is not None else []) + ids      # the reference prepends BOS (model_imp.cpp:123-125)
 
     def show(self, ids: List[int]) -> str:
         if self.tok is not None:
             return self.tok.decode(ids)
+        if self.pieces is not None:
+            return self.pieces.decode(list(ids))
         return " ".join(str(i) for i in ids)
 
 

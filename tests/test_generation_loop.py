@@ -291,3 +291,29 @@ def test_rows_of_the_decode_graphs():
         b = _bucket(n)
         assert n <= b and (b < 2 * n or n == 1) and (n < 17 or 2 * b < 3 * n)
         assert b == _bucket(b)
+
+
+def test_command_line_text_through_a_sentencepiece_model(tmp_path):
+    """`bin/chat -p` takes text through the folder's tokenizer.json or, without one, through its
+    tokenizer.model (SentencePiece, as LLaMA-2 checkpoints bring it): a small model trained here
+    encodes and decodes a sentence, BOS in front as the reference puts it (model_imp.cpp:123-125);
+    a folder with neither refuses text with a clear message."""
+    spm = pytest.importorskip("sentencepiece")
+    from inferllm_amd.cli.chat import _Text
+    corpus = tmp_path / "corpus.txt"
+    corpus.write_text("\n".join(["the quick brown fox jumps over the lazy dog",
+                                 "a model of language reads tokens and writes tokens",
+                                 "one two three four five six seven eight nine ten"] * 20))
+    folder = tmp_path / "model"
+    folder.mkdir()
+    spm.SentencePieceTrainer.train(input=str(corpus), model_prefix=str(folder / "tokenizer"), vocab_size=60,
+                                   model_type="bpe", minloglevel=2)
+    text = _Text(str(folder))
+    ids = text.encode("the quick fox", bos=1)
+    assert ids[0] == 1 and len(ids) > 1 and all(isinstance(i, int) and 0 <= i < 60 for i in ids)
+    assert text.show(ids[1:]) == "the quick fox"
+    empty = tmp_path / "empty"
+    empty.mkdir()
+    with pytest.raises(SystemExit, match="tokenizer"):
+        _Text(str(empty)).encode("x", bos=None)
+    assert _Text(str(empty)).show([3, 4]) == "3 4"
