@@ -86,6 +86,11 @@ class _Text:
             from sentencepiece import SentencePieceProcessor
             self.pieces = SentencePieceProcessor(model_file=spm)
 
+    @property
+    def known(self) -> bool:
+        """Whether the folder brought a tokenizer (else ids are shown as numbers)."""
+        return self.tok is not None or self.pieces is not None
+
     def encode(self, text: str, bos: Optional[int]) -> List[int]:
         if self.tok is not None:
             ids = self.tok.encode(text, add_special_tokens=False).ids
@@ -102,6 +107,26 @@ class _Text:
         if self.pieces is not None:
             return self.pieces.decode(list(ids))
         return " ".join(str(i) for i in ids)
+
+    def printer(self):
+        """`put(token)` prints an answer as its tokens come (the reference prints every token as it
+        is generated, application/chat.cpp:232-236): ids as numbers, text as what the answer so
+        far decodes to beyond what is already out (a token that ends inside a character waits
+        for the rest of it)."""
+        ids: List[int] = []
+        out = [""]
+
+        def put(token: int) -> None:
+            if not self.known:
+                print(token, end=" ", flush=True)
+                return
+            ids.append(token)
+            now = self.show(ids)
+            if now.endswith("\ufffd"):
+                return
+            print(now[len(os.path.commonprefix([out[0], now])):], end="", flush=True)
+            out[0] = now
+        return put
 
 
 def main(argv=None) -> int:
@@ -143,12 +168,14 @@ def main(argv=None) -> int:
     stops = parse_ids(args.stop_ids) if args.stop_ids else None
 
     def run(prompts: List[List[int]]) -> None:
-        stream = len(prompts) == 1 and text.tok is None     # one request of ids: print as they come
+        stream = len(prompts) == 1                        # one request: printed as it comes
+        put = text.printer()
 
         def show(i: int, tok: int) -> None:
-            print(tok, end=" ", flush=True)
+            put(tok)
         # the decode graph of this batch before its first token is timed or awaited
-        eng.warm_up([min(len(prompts), args.max_batch)], max(len(p) for p in prompts) + args.n_predict)
+        eng.warm_up([min(len(prompts), args.max_batch)], max(len(p) for p in prompts) + args.n_predict,
+                    prompt_tokens=max(len(p) for p in prompts))
         outs = eng.generate(prompts, temperature=args.temp, top_k=args.top_k, top_p=args.top_p,
                             repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n,
                             seed=seed, max_new_tokens=args.n_predict, stop_token_ids=stops,
@@ -199,11 +226,8 @@ def main(argv=None) -> int:
                 print(f"chat: the context is full ({talk.remaining} tokens left)", file=sys.stderr)
                 break
             first = False
-            if text.tok is None:
-                out = talk.say(ids, args.n_predict, on_token=lambda t: print(t, end=" ", flush=True))
-                print(flush=True)
-            else:
-                print(text.show(talk.say(ids, args.n_predict)), flush=True)
+            talk.say(ids, args.n_predict, on_token=text.printer())
+            print(flush=True)
             if args.summary:
                 print(talk.last_stats.summary(), file=sys.stderr, flush=True)
             if talk.remaining <= 0:

@@ -293,7 +293,7 @@ def test_rows_of_the_decode_graphs():
         assert b == _bucket(b)
 
 
-def test_command_line_text_through_a_sentencepiece_model(tmp_path):
+def test_command_line_text_through_a_sentencepiece_model(tmp_path, capsys):
     """`bin/chat -p` takes text through the folder's tokenizer.json or, without one, through its
     tokenizer.model (SentencePiece, as LLaMA-2 checkpoints bring it): a small model trained here
     encodes and decodes a sentence, BOS in front as the reference puts it (model_imp.cpp:123-125);
@@ -312,8 +312,16 @@ def test_command_line_text_through_a_sentencepiece_model(tmp_path):
     ids = text.encode("the quick fox", bos=1)
     assert ids[0] == 1 and len(ids) > 1 and all(isinstance(i, int) and 0 <= i < 60 for i in ids)
     assert text.show(ids[1:]) == "the quick fox"
+    put = text.printer()                                   # an answer printed as its tokens come
+    capsys.readouterr()
+    for t in ids[1:]:
+        put(t)
+    assert capsys.readouterr().out == "the quick fox"
     empty = tmp_path / "empty"
     empty.mkdir()
     with pytest.raises(SystemExit, match="tokenizer"):
         _Text(str(empty)).encode("x", bos=None)
     assert _Text(str(empty)).show([3, 4]) == "3 4"
+    put = _Text(str(empty)).printer()
+    put(3); put(4)
+    assert capsys.readouterr().out == "3 4 "

@@ -688,8 +688,9 @@ def test_kernel_timing_reports_every_op(tmp_path_factory):
 
 def test_warm_up_captures_the_decode_graphs_beforehand(tmp_path):
     """`Engine.warm_up` captures the graphs of the batch sizes named (their buckets, once each)
-    without touching a sequence: the steps that follow capture nothing more and give the same
-    bits as in an engine that was not warmed up; an engine without graphs has nothing to do."""
+    without touching a sequence, and runs a throwaway prompt if asked to: the steps that follow
+    capture nothing more and give the same bits as in an engine that was not warmed up; an engine
+    without graphs has nothing to do."""
     import inferllm_amd as I
     from inferllm_amd import StepEntry
     config = CONFIGS["B"]
@@ -700,7 +701,9 @@ def test_warm_up_captures_the_decode_graphs_beforehand(tmp_path):
         eng = I.Engine.from_pretrained(d, dtype="bfloat16", device=DEV, max_batch=8, poison_freed=True)
         if warm:
             assert eng.warm_up([1, 5, 6, 8], longest=40) == 2           # graphs of 1 and of 8 rows
-            assert eng.warm_up([5]) == 0                               # there already
+            assert eng.warm_up([5], prompt_tokens=70) == 0             # there already; a throwaway prompt
+            assert eng.cache.slots.n_held() == 0                       # whose slot and pages came back
+            eng.cache.check()
             before = dict(eng.runner._graphs)
         slots = [eng.alloc_slot() for _ in reqs]
         eng.step([StepEntry(s, r[:-3], []) for s, r in zip(slots, reqs)])
