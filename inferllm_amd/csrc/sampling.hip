@@ -718,6 +718,355 @@ sample_topk_merge_kernel(float* __restrict__ scratch, int32_t* __restrict__ out,
     topk_finish(cand_id, cand_s, n_kept, top_p, seeds[b], counters[b], red_f, &sh_i, out + b);
 }
 
+// ---------------------------------------------------------------- sampler, long rows without top_k
+// The same choice as `sample_kernel` makes for top_k == 0 (temperature, repeat penalty, top_p),
+// for rows of 65,536 ids and more, by several blocks a row: one block walks 128,256 ids in 30 to
+// 50 us a pass and needs three passes for temperature alone and nine with top_p, bound by one
+// compute unit's instruction issue.  Here a row is cut into up to 16 parts with blocks of their
+// own and every pass is a kernel; what a pass hands to the next lies in the row's `SpRow`.
+// Masses are integers (p * 2^40), so no sum depends on the order of its terms:
+//   scale   scaled and penalised scores; the parts' largest
+//   mass    p = exp(s - max); the parts' masses; (top_p) the mass per top digit of the key
+//   digit   x3 (top_p) every block finds the threshold's next digit from the last pass's masses
+//           per digit, then adds up the masses per next digit among the keys with that prefix
+//   edge    (top_p) the last digit; per part the mass above the threshold key and the ids at it
+//   draw    one block a row: how many ids at the threshold key stay (the lowest ids), the part
+//           that holds the target of the draw, and the id in it
+#define SP_MAX_PARTS 16
+typedef unsigned long long sp_u64;
+
+struct SpRow {
+    float pmax[SP_MAX_PARTS];
+    sp_u64 ptotal[SP_MAX_PARTS];
+    sp_u64 mass_gt[SP_MAX_PARTS];
+    sp_u64 one_fx[SP_MAX_PARTS];              // the mass of an id at the threshold key (0: none in the part)
+    int n_eq[SP_MAX_PARTS];
+    uint32_t t[5];                            // the threshold's key after 0 .. 4 digits
+    uint32_t pad;
+    sp_u64 above[5];                          // mass of the keys above that prefix
+    sp_u64 hist[2][SP_MAX_PARTS][256];        // mass per digit, two passes alternating
+};
+static_assert(sizeof(SpRow) <= ILLM_SAMPLE_LONG_ROW_BYTES, "SpRow must fit what callers allocate");
+
+__device__ __forceinline__ sp_u64 sp_fixed(float p) { return (sp_u64)(p * 1099511627776.0f); }
+
+struct SpPart {
+    int first, n;                             // the ids [first, first + n) of the row
+};
+__device__ __forceinline__ SpPart sp_part(int V, int parts, int p) {
+    const int stretch = ((V + parts - 1) / parts + 3) / 4 * 4;
+    const int first = min(V, p * stretch);
+    return {first, min(stretch, V - first)};
+}
+
+__global__ void __launch_bounds__(SB)
+sp_scale_kernel(const float* __restrict__ logits, float* __restrict__ scratch, SpRow* __restrict__ rows,
+                int V, float temp, float repeat_penalty, const int32_t* __restrict__ last_tokens,
+                int n_last) {
+    __shared__ float red_f[SB / ILLM_WAVE];
+    __shared__ int last[256];
+    const int p = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const SpPart part = sp_part(V, gridDim.x, p);
+    const float* row = logits + (size_t)b * V + part.first;
+    float* s = scratch + (size_t)b * V + part.first;
+    const int nl = last_tokens ? min(n_last, 256) : 0;
+    if (tid < nl) last[tid] = last_tokens[(size_t)b * n_last + tid];
+    const float inv_temp = 1.0f / temp;
+    each_strided8(row, part.n, tid, [&](int i, float v) { s[i] = v * inv_temp; });
+    __syncthreads();
+    // the penalty, once for every id of the window that lies in this part
+    if (tid < nl) {
+        const int id = last[tid] - part.first;
+        bool once = last[tid] >= 0 && id >= 0 && id < part.n;
+        for (int j = 0; j < tid; ++j) once = once && last[j] != last[tid];
+        if (once) {
+            const float l = row[id], v = l * inv_temp;
+            s[id] = l < 0.f ? v * repeat_penalty : v / repeat_penalty;
+        }
+    }
+    __syncthreads();
+    float mx = -INFINITY;
+    each_strided8(s, part.n, tid, [&](int, float v) { mx = fmaxf(mx, v); });
+    mx = block_max(mx, red_f);
+    if (tid == 0) rows[b].pmax[p] = mx;
+}
+
+// The mass per digit `(key >> shift) & 255` of the part's ids whose key has the prefix `t` above
+// those bits (hi_mask == 0: all ids), into out[256]; by the waves into LDS, then added up.
+template <typename F>
+__device__ __forceinline__ void sp_histogram(sp_u64 (*mhist)[256], sp_u64* out, F walk, uint32_t t,
+                                             uint32_t hi_mask, int shift) {
+    const int tid = threadIdx.x, wave = tid / ILLM_WAVE;
+    for (int i = tid; i < (SB / ILLM_WAVE) * 256; i += SB) (&mhist[0][0])[i] = 0;
+    __syncthreads();
+    walk([&](uint32_t key, sp_u64 fx) {
+        if ((key & hi_mask) == t) atomicAdd(&mhist[wave][(key >> shift) & 255u], fx);
+    });
+    __syncthreads();
+    if (tid < 256) {
+        sp_u64 m = 0;
+        for (int w = 0; w < SB / ILLM_WAVE; ++w) m += mhist[w][tid];
+        out[tid] = m;
+    }
+}
+
+__global__ void __launch_bounds__(SB)
+sp_mass_kernel(float* __restrict__ scratch, SpRow* __restrict__ rows, int V, int n_rows, float top_p) {
+    __shared__ sp_u64 mhist[SB / ILLM_WAVE][256];
+    __shared__ sp_u64 sh_total;
+    const int p = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, parts = gridDim.x;
+    const SpPart part = sp_part(V, parts, p);
+    SpRow& R = rows[b];
+    float mx = R.pmax[0];
+    for (int q = 1; q < parts; ++q) mx = fmaxf(mx, R.pmax[q]);
+    const float* s = scratch + (size_t)b * V + part.first;
+    float* pr = scratch + ((size_t)n_rows + b) * V + part.first;
+    sp_u64 mine = 0;
+    each_strided8(s, part.n, tid, [&](int i, float v) {
+        const float e = expf(v - mx);
+        pr[i] = e;
+        mine += sp_fixed(e);
+    });
+    if (tid == 0) sh_total = 0;
+    __syncthreads();
+    atomicAdd(&sh_total, mine);
+    __syncthreads();
+    if (tid == 0) {
+        R.ptotal[p] = sh_total;
+        if (p == 0) { R.t[0] = 0u; R.above[0] = 0; }
+    }
+    if (top_p < 1.0f) {
+        // (a thread reads back the probabilities that it wrote itself)
+        auto walk = [&](auto f) __attribute__((always_inline)) {
+            each_strided8(s, part.n, tid, [&](int i, float v) { f(order_key(v), sp_fixed(pr[i])); });
+        };
+        sp_histogram(mhist, R.hist[0][p], walk, 0u, 0u, 24);
+    }
+}
+
+// The threshold after `level` + 1 digits, from the masses per digit that pass `level` left: the
+// largest digit at which the mass from the top reaches what top_p needs.  Every block of the next
+// pass finds it for itself; the first of a row writes it down for the passes after.
+__device__ __forceinline__ void sp_decide(SpRow& R, int parts, int level, float top_p, sp_u64* digit_mass,
+                                          uint32_t* t_out, sp_u64* above_out, bool write) {
+    __shared__ int sh_digit;
+    __shared__ sp_u64 sh_above;
+    const int tid = threadIdx.x, shift = 24 - 8 * level;
+    sp_u64 total = 0;
+    for (int q = 0; q < parts; ++q) total += R.ptotal[q];
+    sp_u64 need = (sp_u64)((double)top_p * (double)total);
+    need = need > 0 ? need : 1;
+    if (tid < 256) {
+        sp_u64 m = 0;
+        for (int q = 0; q < parts; ++q) m += R.hist[level & 1][q][tid];
+        digit_mass[tid] = m;
+    }
+    if (tid == 0) { sh_digit = 0; sh_above = R.above[level]; }
+    __syncthreads();
+    if (tid < 256) {
+        sp_u64 over = R.above[level];
+        for (int d = tid + 1; d < 256; ++d) over += digit_mass[d];
+        if (over < need && over + digit_mass[tid] >= need) { sh_digit = tid; sh_above = over; }
+    }
+    __syncthreads();
+    *t_out = R.t[level] | ((uint32_t)sh_digit << shift);
+    *above_out = sh_above;
+    if (write && tid == 0) { R.t[level + 1] = *t_out; R.above[level + 1] = sh_above; }
+    __syncthreads();
+}
+
+// level 1 .. 3: decide digit `level - 1`, then the masses per digit `level` under the new prefix
+__global__ void __launch_bounds__(SB)
+sp_digit_kernel(const float* __restrict__ scratch, SpRow* __restrict__ rows, int V, int n_rows,
+                float top_p, int level) {
+    __shared__ sp_u64 mhist[SB / ILLM_WAVE][256];
+    __shared__ sp_u64 digit_mass[256];
+    const int p = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, parts = gridDim.x;
+    const SpPart part = sp_part(V, parts, p);
+    SpRow& R = rows[b];
+    uint32_t t;
+    sp_u64 above;
+    sp_decide(R, parts, level - 1, top_p, digit_mass, &t, &above, p == 0);
+    const float* s = scratch + (size_t)b * V + part.first;
+    const float* pr = scratch + ((size_t)n_rows + b) * V + part.first;
+    auto walk = [&](auto f) __attribute__((always_inline)) {
+        each_strided8(s, part.n, tid, [&](int i, float v) { f(order_key(v), sp_fixed(pr[i])); });
+    };
+    const int shift = 24 - 8 * level;
+    sp_histogram(mhist, R.hist[level & 1][p], walk, t, 0xffffffffu << (shift + 8), shift);
+}
+
+// the last digit; the part's mass above the threshold key, its ids at that key and their mass
+__global__ void __launch_bounds__(SB)
+sp_edge_kernel(const float* __restrict__ scratch, SpRow* __restrict__ rows, int V, int n_rows,
+               float top_p) {
+    __shared__ sp_u64 digit_mass[256];
+    __shared__ sp_u64 sh_gt, sh_one;
+    __shared__ int sh_eq;
+    const int p = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, parts = gridDim.x;
+    const SpPart part = sp_part(V, parts, p);
+    SpRow& R = rows[b];
+    uint32_t t;
+    sp_u64 above;
+    sp_decide(R, parts, 3, top_p, digit_mass, &t, &above, p == 0);
+    const float* s = scratch + (size_t)b * V + part.first;
+    const float* pr = scratch + ((size_t)n_rows + b) * V + part.first;
+    sp_u64 gt = 0, one = 0;
+    int eq = 0;
+    each_strided8(s, part.n, tid, [&](int i, float v) {
+        const uint32_t key = order_key(v);
+        if (key > t) gt += sp_fixed(pr[i]);
+        else if (key == t) { eq += 1; one = sp_fixed(pr[i]); }
+    });
+    if (tid == 0) { sh_gt = 0; sh_one = 0; sh_eq = 0; }
+    __syncthreads();
+    atomicAdd(&sh_gt, gt);
+    atomicAdd(&sh_eq, eq);
+    if (eq) atomicMax(&sh_one, one);
+    __syncthreads();
+    if (tid == 0) { R.mass_gt[p] = sh_gt; R.n_eq[p] = sh_eq; R.one_fx[p] = sh_one; }
+}
+
+__global__ void __launch_bounds__(SB)
+sp_draw_kernel(const float* __restrict__ scratch, const SpRow* __restrict__ rows, int32_t* __restrict__ out,
+               int V, int n_rows, int parts, float top_p, const uint64_t* __restrict__ seeds,
+               const int32_t* __restrict__ counters) {
+    __shared__ sp_u64 red_u[SB / ILLM_WAVE];
+    __shared__ int red_i[SB / ILLM_WAVE];
+    __shared__ int sh_i;
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const SpRow& R = rows[b];
+    const float* s = scratch + (size_t)b * V;
+    const float* pr = scratch + ((size_t)n_rows + b) * V;
+    const bool all = !(top_p < 1.0f);                    // every id stays
+    // (every thread works these few numbers out for itself)
+    sp_u64 total = 0;
+    for (int q = 0; q < parts; ++q) total += R.ptotal[q];
+    uint32_t t = 0;
+    int cut = V, part_of_cut = parts, eq_in_cut_part = 0;
+    sp_u64 one = 0, kept_total = total;
+    if (!all) {
+        sp_u64 need = (sp_u64)((double)top_p * (double)total);
+        need = need > 0 ? need : 1;
+        t = R.t[4];
+        const sp_u64 above = R.above[4];
+        int n_eq = 0;
+        for (int q = 0; q < parts; ++q) { n_eq += R.n_eq[q]; one = one ? one : R.one_fx[q]; }
+        // ids at the threshold key that stay: as many as still needed to reach top_p, the lowest ids
+        long long m = one > 0 ? (long long)((need - above + one - 1) / one) : n_eq;
+        m = m < 1 ? 1 : (m > n_eq ? n_eq : m);
+        kept_total = above + (sp_u64)m * one;
+        int before = 0;
+        for (int q = 0; q < parts; ++q) {
+            if (m > before && m <= before + R.n_eq[q]) { part_of_cut = q; eq_in_cut_part = (int)m - before; }
+            before += R.n_eq[q];
+        }
+        // the id of that last one: the eq_in_cut_part-th id at the key in its part
+        const SpPart part = sp_part(V, parts, part_of_cut);
+        const int chunk = (part.n + SB - 1) / SB;
+        const int lo = part.first + min(part.n, tid * chunk), hi = min(part.first + part.n, lo + chunk);
+        int mine = 0;
+        for (int i = lo; i < hi; ++i) mine += order_key(s[i]) == t ? 1 : 0;
+        int all_eq;
+        const int bef = block_exclusive_scan<int>(mine, red_i, &all_eq);
+        __syncthreads();
+        if (tid == 0) sh_i = part.first + part.n - 1;
+        __syncthreads();
+        if (eq_in_cut_part > bef && eq_in_cut_part <= bef + mine) {
+            int c = bef;
+            for (int i = lo; i < hi; ++i)
+                if (order_key(s[i]) == t && ++c == eq_in_cut_part) { sh_i = i; break; }
+        }
+        __syncthreads();
+        cut = sh_i;
+        __syncthreads();
+    }
+    auto stays = [&](int i) {
+        if (all) return true;
+        const uint32_t key = order_key(s[i]);
+        return key > t || (key == t && i <= cut);
+    };
+    // the part that holds the target, by the parts' kept masses in id order
+    const float u = uniform_from(seeds[b], counters[b]);
+    sp_u64 target = (sp_u64)((double)u * (double)kept_total);
+    target = target < kept_total ? target : (kept_total ? kept_total - 1 : 0);
+    int pt = parts - 1;
+    sp_u64 before_part = 0;
+    {
+        sp_u64 acc = 0;
+        bool found = false;
+        for (int q = 0; q < parts; ++q) {
+            const sp_u64 km = all ? R.ptotal[q]
+                                  : R.mass_gt[q] + one * (sp_u64)(q < part_of_cut ? R.n_eq[q]
+                                                                  : (q == part_of_cut ? eq_in_cut_part : 0));
+            if (!found && target < acc + km) { pt = q; before_part = acc; found = true; }
+            acc += km;
+        }
+    }
+    const sp_u64 rem = target - before_part;
+    const SpPart part = sp_part(V, parts, pt);
+    const int chunk = (part.n + SB - 1) / SB;
+    const int lo = part.first + min(part.n, tid * chunk), hi = min(part.first + part.n, lo + chunk);
+    sp_u64 mine = 0;
+    for (int i = lo; i < hi; ++i)
+        if (stays(i)) mine += sp_fixed(pr[i]);
+    sp_u64 part_total;
+    const sp_u64 bef = block_exclusive_scan<sp_u64>(mine, red_u, &part_total);
+    __syncthreads();
+    if (tid == 0) sh_i = -1;
+    __syncthreads();
+    if (mine > 0 && rem >= bef && rem < bef + mine) {
+        sp_u64 c = bef;
+        int pick = -1;
+        for (int i = lo; i < hi; ++i) {
+            if (!stays(i)) continue;
+            pick = i;
+            c += sp_fixed(pr[i]);
+            if (rem < c) break;
+        }
+        atomicMax(&sh_i, pick);
+    }
+    __syncthreads();
+    if (sh_i < 0) {
+        // (the target lies past the part's last kept id only if the sums disagree: take that id)
+        int lastk = -1;
+        for (int i = lo; i < hi; ++i)
+            if (stays(i) && sp_fixed(pr[i]) > 0) lastk = i;
+        atomicMax(&sh_i, lastk);
+        __syncthreads();
+    }
+    if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
+}
+
+extern "C" int illm_sample_long(const float* logits, float* scratch, void* rows, int32_t* out, int B,
+                                int V, float temp, float top_p, float repeat_penalty,
+                                const int32_t* last_tokens, int n_last, const uint64_t* seeds,
+                                const int32_t* counters, void* stream) {
+    if (B < 0 || B > 65535 || V < 65536 || !(temp > 0.f) || !(top_p > 0.f) || !(repeat_penalty > 0.f) ||
+        n_last < 0 || n_last > 256 || !seeds || !counters || !scratch || !rows)
+        return ILLM_ERR_ARG;
+    if (B == 0) return ILLM_OK;
+    // parts of 4,096 ids or more, about 512 blocks in all
+    int parts = V / 4096;
+    parts = parts > SP_MAX_PARTS ? SP_MAX_PARTS : parts;
+    while (parts > 2 && parts * B > 512) parts /= 2;
+    hipStream_t st = (hipStream_t)stream;
+    SpRow* R = (SpRow*)rows;
+    const dim3 grid(parts, B);
+    hipLaunchKernelGGL(sp_scale_kernel, grid, dim3(SB), 0, st, logits, scratch, R, V, temp,
+                       repeat_penalty, last_tokens, n_last);
+    hipLaunchKernelGGL(sp_mass_kernel, grid, dim3(SB), 0, st, scratch, R, V, B, top_p);
+    if (top_p < 1.0f) {
+        for (int level = 1; level <= 3; ++level)
+            hipLaunchKernelGGL(sp_digit_kernel, grid, dim3(SB), 0, st, (const float*)scratch, R, V, B,
+                               top_p, level);
+        hipLaunchKernelGGL(sp_edge_kernel, grid, dim3(SB), 0, st, (const float*)scratch, R, V, B, top_p);
+    }
+    hipLaunchKernelGGL(sp_draw_kernel, dim3(B), dim3(SB), 0, st, (const float*)scratch, (const SpRow*)R,
+                       out, V, B, parts, top_p, seeds, counters);
+    return illm_launch_status();
+}
+
 extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V,
                            float temp, int top_k, float top_p, float repeat_penalty,
                            const int32_t* last_tokens, int n_last, const uint64_t* seeds,

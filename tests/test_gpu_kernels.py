@@ -850,7 +850,10 @@ def test_the_uniform_numbers_of_the_tests_and_of_the_host_side_agree():
     (128256, 0.9, 0, 0.8, 1.2), (40000, 1.0, 2000, 0.6, 1.0), (33000, 0.7, 0, 0.999, 1.0), (50000, 1.3, 0, 1.0, 1.0),
     # long rows with a small top_k are cut into parts that blocks of their own take: a length that
     # no part divides, the largest top_k of that way and the first beyond it
-    (70001, 0.1, 40, 0.95, 1.1), (65536, 1.0, 64, 0.5, 1.0), (65536, 1.0, 65, 0.5, 1.3), (200003, 0.8, 3, 1.0, 1.3)])
+    (70001, 0.1, 40, 0.95, 1.1), (65536, 1.0, 64, 0.5, 1.0), (65536, 1.0, 65, 0.5, 1.3), (200003, 0.8, 3, 1.0, 1.3),
+    # long rows without top_k: several blocks a row and a kernel a pass
+    (70001, 0.7, 0, 0.9, 1.0), (131072, 1.0, 0, 1.0, 1.1), (200003, 0.5, 0, 0.5, 1.3), (65536, 2.0, 0, 0.999, 1.0),
+    (65537, 0.3, 0, 0.05, 1.0)])
 def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top_p, penalty):
     uniform = R.uniform                                      # the tests' own statement of the hash
     B = 6
