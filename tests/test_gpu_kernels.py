@@ -893,6 +893,27 @@ def test_sample_of_a_long_row_in_parts_keeps_what_one_block_would():
         assert interval_ok(logits[b], int(got[b]), u, 1.0, top_k, 1.0, 1.0, None), (b, int(got[b]), u)
 
 
+@pytest.mark.parametrize("top_p", [1.0, 0.9, 0.3])
+def test_sample_of_a_long_row_does_not_depend_on_its_company(top_p):
+    """Rows of 65,536 ids and more without top_k are cut into more or fewer parts depending on how
+    many rows there are; the masses are added as integers, so a row draws the same id alone and
+    among 69 others, draw after draw."""
+    V = 100003
+    rows = rnd(70, V, seed=33, std=3.0)
+    seeds = torch.arange(70, dtype=torch.int64) * 7919 + 5
+    last = torch.randint(0, V, (70, 16), generator=torch.Generator().manual_seed(2), dtype=torch.int32)
+    for counter in (0, 1, 2):
+        counters = torch.full((70,), counter, dtype=torch.int32)
+        together = ops().sample(rows.to(DEV), 0.8, 0, top_p, 1.2, last.to(DEV), seeds.to(DEV), counters.to(DEV)).cpu()
+        for b in (0, 13, 69):
+            alone = ops().sample(rows[b:b + 1].to(DEV), 0.8, 0, top_p, 1.2, last[b:b + 1].to(DEV),
+                                 seeds[b:b + 1].to(DEV), counters[b:b + 1].to(DEV)).cpu()
+            assert int(alone[0]) == int(together[b]), (b, counter)
+        few = ops().sample(rows[:9].to(DEV), 0.8, 0, top_p, 1.2, last[:9].to(DEV), seeds[:9].to(DEV),
+                           counters[:9].to(DEV)).cpu()
+        assert few.tolist() == together[:9].tolist()
+
+
 def test_sample_frequencies_match_probabilities():
     V, n = 7, 4000
     row = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, 1.5, -3.0])
