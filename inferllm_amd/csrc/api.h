@@ -225,7 +225,7 @@ int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V,
                 int top_k, float top_p, float repeat_penalty, const int32_t* last_tokens,
                 int n_last, const uint64_t* seeds, const int32_t* counters, void* stream);
 
-// The same without top_k for rows of 65,536 ids and more, several blocks a row and a kernel a
+// The same without top_k for rows of 16,384 ids and more, several blocks a row and a kernel a
 // pass (illm_sample walks such a row with one block).  rows: B x ILLM_SAMPLE_LONG_ROW_BYTES bytes
 // of device memory, 8-byte aligned, that the passes hand their results on through; nothing in it
 // needs clearing.  Shorter rows: ILLM_ERR_ARG.

@@ -720,7 +720,7 @@ sample_topk_merge_kernel(float* __restrict__ scratch, int32_t* __restrict__ out,
 
 // ---------------------------------------------------------------- sampler, long rows without top_k
 // The same choice as `sample_kernel` makes for top_k == 0 (temperature, repeat penalty, top_p),
-// for rows of 65,536 ids and more, by several blocks a row: one block walks 128,256 ids in 30 to
+// for rows of 16,384 ids and more, by several blocks a row: one block walks 128,256 ids in 30 to
 // 50 us a pass and needs three passes for temperature alone and nine with top_p, bound by one
 // compute unit's instruction issue.  Here a row is cut into up to 16 parts with blocks of their
 // own and every pass is a kernel; what a pass hands to the next lies in the row's `SpRow`.
@@ -1042,7 +1042,7 @@ extern "C" int illm_sample_long(const float* logits, float* scratch, void* rows,
                                 int V, float temp, float top_p, float repeat_penalty,
                                 const int32_t* last_tokens, int n_last, const uint64_t* seeds,
                                 const int32_t* counters, void* stream) {
-    if (B < 0 || B > 65535 || V < 65536 || !(temp > 0.f) || !(top_p > 0.f) || !(repeat_penalty > 0.f) ||
+    if (B < 0 || B > 65535 || V < 16384 || !(temp > 0.f) || !(top_p > 0.f) || !(repeat_penalty > 0.f) ||
         n_last < 0 || n_last > 256 || !seeds || !counters || !scratch || !rows)
         return ILLM_ERR_ARG;
     if (B == 0) return ILLM_OK;

@@ -853,7 +853,7 @@ def test_the_uniform_numbers_of_the_tests_and_of_the_host_side_agree():
     (70001, 0.1, 40, 0.95, 1.1), (65536, 1.0, 64, 0.5, 1.0), (65536, 1.0, 65, 0.5, 1.3), (200003, 0.8, 3, 1.0, 1.3),
     # long rows without top_k: several blocks a row and a kernel a pass
     (70001, 0.7, 0, 0.9, 1.0), (131072, 1.0, 0, 1.0, 1.1), (200003, 0.5, 0, 0.5, 1.3), (65536, 2.0, 0, 0.999, 1.0),
-    (65537, 0.3, 0, 0.05, 1.0)])
+    (65537, 0.3, 0, 0.05, 1.0), (16384, 0.9, 0, 0.7, 1.2), (16387, 1.1, 0, 1.0, 1.0)])
 def test_sample_draws_from_the_reference_distribution(V, temperature, top_k, top_p, penalty):
     uniform = R.uniform                                      # the tests' own statement of the hash
     B = 6
@@ -895,7 +895,7 @@ def test_sample_of_a_long_row_in_parts_keeps_what_one_block_would():
 
 @pytest.mark.parametrize("top_p", [1.0, 0.9, 0.3])
 def test_sample_of_a_long_row_does_not_depend_on_its_company(top_p):
-    """Rows of 65,536 ids and more without top_k are cut into more or fewer parts depending on how
+    """Rows of 16,384 ids and more without top_k are cut into more or fewer parts depending on how
     many rows there are; the masses are added as integers, so a row draws the same id alone and
     among 69 others, draw after draw."""
     V = 100003
