@@ -505,7 +505,9 @@ __device__ __forceinline__ void topk_finish(const int* cand_id, const float* can
     if (tid == 0) *out_b = *sh_i < 0 ? 0 : *sh_i;
 }
 
-template <bool PART>
+// NR > 0: the block's ids fit NR registers a thread (a wave's stretch of the row in 64 * NR ids) and
+// every pass after the first reads them from there instead of from the scratch.
+template <bool PART, int NR>
 __global__ void __launch_bounds__(SB)
 sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch,
                    int32_t* __restrict__ out, int Vrow, float temp, int top_k, float top_p,
@@ -549,6 +551,44 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
     }
     __syncthreads();
 
+    // A wave walks its own stretch of the row, 64 consecutive ids an instruction (a thread walking
+    // a stretch of its own would touch 64 cache lines an instruction); within an instruction the
+    // lanes are in id order, so the gather below gets counts and places from ballots.
+    const int lane = tid & (ILLM_WAVE - 1);
+    const int stretch = ((V + NW - 1) / NW + ILLM_WAVE - 1) / ILLM_WAVE * ILLM_WAVE;
+    const int lo = min(V, wave * stretch), hi = min(V, lo + stretch);
+    float rv[NR > 0 ? NR : 1];
+    if constexpr (NR > 0) {
+#pragma unroll
+        for (int u = 0; u < NR; ++u) {
+            const int i = lo + u * ILLM_WAVE + lane;
+            rv[u] = i < hi ? s[i] : 0.f;
+        }
+    }
+    auto walk = [&](auto f) __attribute__((always_inline)) {
+        if constexpr (NR > 0) {
+#pragma unroll
+            for (int u = 0; u < NR; ++u) {
+                const int i = lo + u * ILLM_WAVE + lane;
+                f(i, rv[u], i < hi);
+            }
+        } else {
+            for (int base = lo; base < hi; base += 8 * ILLM_WAVE) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int i = base + u * ILLM_WAVE + lane;
+                    v[u] = i < hi ? s[i] : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int i = base + u * ILLM_WAVE + lane;
+                    f(i, v[u], i < hi);
+                }
+            }
+        }
+    };
+
     // 2. the key of the top_k-th largest score, 8 bits a pass
     uint32_t prefix = 0;
     int krem = top_k;
@@ -557,9 +597,9 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
         const uint32_t hi_mask = pass ? (0xffffffffu << (shift + 8)) : 0u;
         for (int i = tid; i < NW * 256; i += SB) (&hist[0][0])[i] = 0;
         __syncthreads();
-        each_strided8(s, V, tid, [&](int, float v) {
+        walk([&](int, float v, bool in) {
             const uint32_t key = order_key(v);
-            if ((key & hi_mask) == prefix) atomicAdd(&hist[wave][(key >> shift) & 255u], 1);
+            if (in && (key & hi_mask) == prefix) atomicAdd(&hist[wave][(key >> shift) & 255u], 1);
         });
         __syncthreads();
         if (tid < 256) {
@@ -595,29 +635,8 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
     }
     // kept: key > prefix, and the first krem ids (ascending) with key == prefix
 
-    // 3. the kept ids and scores in id order into LDS.  A wave walks its own stretch of the row,
-    // 64 consecutive ids an instruction (a thread walking a stretch of its own would touch 64
-    // cache lines an instruction); within an instruction the lanes are in id order, so counts
-    // and places come from ballots.
-    const int lane = tid & (ILLM_WAVE - 1);
+    // 3. the kept ids and scores in id order into LDS: counts and places from ballots
     const unsigned long long below = (1ull << lane) - 1ull;
-    const int stretch = ((V + NW - 1) / NW + ILLM_WAVE - 1) / ILLM_WAVE * ILLM_WAVE;
-    const int lo = min(V, wave * stretch), hi = min(V, lo + stretch);
-    auto walk = [&](auto f) __attribute__((always_inline)) {
-        for (int base = lo; base < hi; base += 8 * ILLM_WAVE) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int i = base + u * ILLM_WAVE + lane;
-                v[u] = i < hi ? s[i] : 0.f;
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int i = base + u * ILLM_WAVE + lane;
-                f(i, v[u], i < hi);
-            }
-        }
-    };
     int n_eq = 0, n_gt = 0;                             // of the wave's stretch (the same in all its lanes)
     walk([&](int, float v, bool in) {
         const uint32_t key = order_key(v);
@@ -1081,13 +1100,24 @@ extern "C" int illm_sample(const float* logits, float* scratch, int32_t* out, in
         int parts = V / 4096;
         parts = parts > TOPK_MAX_PARTS ? TOPK_MAX_PARTS : parts;
         while (parts > 2 && parts * B > 512) parts /= 2;
-        hipLaunchKernelGGL(sample_topk_kernel<true>, dim3(parts, B), dim3(SB), 0, (hipStream_t)stream,
-                           logits, scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens,
-                           n_last, seeds, counters);
+        // (a part's ids: as sample_topk_kernel cuts the row)
+        const int part_ids = ((V + parts - 1) / parts + 3) / 4 * 4;
+        if (part_ids <= 8 * ILLM_WAVE * (SB / ILLM_WAVE))
+            hipLaunchKernelGGL((sample_topk_kernel<true, 8>), dim3(parts, B), dim3(SB), 0, (hipStream_t)stream,
+                               logits, scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens,
+                               n_last, seeds, counters);
+        else
+            hipLaunchKernelGGL((sample_topk_kernel<true, 0>), dim3(parts, B), dim3(SB), 0, (hipStream_t)stream,
+                               logits, scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens,
+                               n_last, seeds, counters);
         hipLaunchKernelGGL(sample_topk_merge_kernel, dim3(B), dim3(SB), 0, (hipStream_t)stream, scratch,
                            out, V, parts, top_k, top_p, seeds, counters);
-    } else if (top_k > 0 && top_k <= SB && top_k < V)
-        hipLaunchKernelGGL(sample_topk_kernel<false>, dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
+    } else if (top_k > 0 && top_k <= SB && top_k < V && V <= 32 * ILLM_WAVE * (SB / ILLM_WAVE))
+        hipLaunchKernelGGL((sample_topk_kernel<false, 32>), dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
+                           scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
+                           seeds, counters);
+    else if (top_k > 0 && top_k <= SB && top_k < V)
+        hipLaunchKernelGGL((sample_topk_kernel<false, 0>), dim3(B), dim3(SB), 0, (hipStream_t)stream, logits,
                            scratch, out, V, temp, top_k, top_p, repeat_penalty, last_tokens, n_last,
                            seeds, counters);
     else if (V <= SAMPLE_REG_IDS * SB)
