@@ -230,6 +230,7 @@ int illm_sample(const float* logits, float* scratch, int32_t* out, int B, int V,
 // of device memory, 8-byte aligned, that the passes hand their results on through; nothing in it
 // needs clearing.  Shorter rows: ILLM_ERR_ARG.
 #define ILLM_SAMPLE_LONG_ROW_BYTES 73728
+int illm_sample_long_row_bytes(void);          // ILLM_SAMPLE_LONG_ROW_BYTES, for callers that cannot read this file
 int illm_sample_long(const float* logits, float* scratch, void* rows, int32_t* out, int B, int V,
                      float temp, float top_p, float repeat_penalty, const int32_t* last_tokens,
                      int n_last, const uint64_t* seeds, const int32_t* counters, void* stream);

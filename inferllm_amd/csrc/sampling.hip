@@ -1057,6 +1057,8 @@ sp_draw_kernel(const float* __restrict__ scratch, const SpRow* __restrict__ rows
     if (tid == 0) out[b] = sh_i < 0 ? 0 : sh_i;
 }
 
+extern "C" int illm_sample_long_row_bytes(void) { return ILLM_SAMPLE_LONG_ROW_BYTES; }
+
 extern "C" int illm_sample_long(const float* logits, float* scratch, void* rows, int32_t* out, int B,
                                 int V, float temp, float top_p, float repeat_penalty,
                                 const int32_t* last_tokens, int n_last, const uint64_t* seeds,

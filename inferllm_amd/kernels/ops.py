@@ -996,7 +996,7 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 
 
 SAMPLE_LONG_FROM = 16384          # ids from which a row without top_k is sampled by several blocks
-SAMPLE_LONG_ROW_BYTES = 73728     # ILLM_SAMPLE_LONG_ROW_BYTES of csrc/api.h
+_sample_long_row_bytes = 0        # ILLM_SAMPLE_LONG_ROW_BYTES of csrc/api.h, asked of the library at first use
 
 
 def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float,
@@ -1019,7 +1019,10 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float,
     if (top_k <= 0 or top_k >= V) and V >= SAMPLE_LONG_FROM and B <= 65535:
         # a long row without top_k: several blocks a row (one block walks 32,000 ids in 54 us for
         # temperature alone and 109 us with top_p, 128,256 in 134 and 395 us)
-        rows = torch.empty((B, SAMPLE_LONG_ROW_BYTES // 8), dtype=torch.int64, device=logits.device)
+        global _sample_long_row_bytes
+        if not _sample_long_row_bytes:
+            _sample_long_row_bytes = int(_lib().illm_sample_long_row_bytes())
+        rows = torch.empty((B, (_sample_long_row_bytes + 7) // 8), dtype=torch.int64, device=logits.device)
         _check(_lib().illm_sample_long(
             _p(logits), _p(scratch), _p(rows), _p(out), B, V, ctypes.c_float(temperature),
             ctypes.c_float(top_p), ctypes.c_float(repeat_penalty), _p(last_tokens), n_last, _p(seeds),
