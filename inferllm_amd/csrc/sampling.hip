@@ -466,6 +466,7 @@ __device__ __forceinline__ float* topk_part_slot(float* scratch, int B, int V, i
 __device__ __forceinline__ void topk_finish(const int* cand_id, const float* cand_s, int n_kept,
                                             float top_p, uint64_t seed, int counter, float* red_f,
                                             int* sh_i, int32_t* out_b) {
+    __shared__ float cand_p[SB];                        // exp(score - max), computed once
     const int tid = threadIdx.x;
     const bool have = tid < n_kept;
     const float my_s = have ? cand_s[tid] : -INFINITY;
@@ -475,14 +476,15 @@ __device__ __forceinline__ void topk_finish(const int* cand_id, const float* can
     const float my_p = have ? expf(my_s - mx) : 0.f;
     bool stay = have;
     if (top_p < 1.0f) {
-        const float z = block_sum_t<float>(my_p, red_f);
+        cand_p[tid] = my_p;
+        const float z = block_sum_t<float>(my_p, red_f);        // (its barriers publish cand_p)
         const float need = top_p * z;
         if (have) {
             float before = 0.f;
             const uint32_t my_key = order_key(my_s);
             for (int j = 0; j < n_kept; ++j) {
                 const uint32_t kj = order_key(cand_s[j]);
-                if (kj > my_key || (kj == my_key && j < tid)) before += expf(cand_s[j] - mx);
+                if (kj > my_key || (kj == my_key && j < tid)) before += cand_p[j];
             }
             stay = before < need;
         }
