@@ -604,17 +604,11 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
             if (in && (key & hi_mask) == prefix) atomicAdd(&hist[wave][(key >> shift) & 255u], 1);
         });
         __syncthreads();
-        if (tid < 256) {
-            int t = 0;
-            for (int w = 0; w < NW; ++w) t += hist[w][tid];
-            hist[0][tid] = t;
-        }
-        __syncthreads();
         // how many keys have a larger digit: a suffix sum over the 256 digits, within each of
         // the first four waves by shuffles, across them through LDS
         int cnt = 0, suffix = 0;
         if (tid < 256) {
-            cnt = hist[0][tid];
+            for (int w = 0; w < NW; ++w) cnt += hist[w][tid];
             suffix = cnt;
             const int ln = tid & (ILLM_WAVE - 1);
 #pragma unroll
@@ -631,9 +625,9 @@ sample_topk_kernel(const float* __restrict__ logits, float* __restrict__ scratch
             if (above < krem && above + cnt >= krem) { sh_d = tid; sh_above = above; }
         }
         __syncthreads();
+        // (sh_d and sh_above are written again only after the next pass's barriers)
         prefix |= (uint32_t)sh_d << shift;
         krem -= sh_above;
-        __syncthreads();
     }
     // kept: key > prefix, and the first krem ids (ascending) with key == prefix
 
