@@ -1,5 +1,5 @@
-from .manager import PAGE_SIZE, CacheManager, KVGroup, KVSpec, StateSpec, round_up
+from .manager import PAGE_SIZE, CacheManager, KVGroup, KVSpec, StateSpec, TokenTensor, round_up
 from .slots import CacheError, CacheFull, FreeList
 
-__all__ = ["PAGE_SIZE", "CacheManager", "KVGroup", "KVSpec", "StateSpec", "round_up",
+__all__ = ["PAGE_SIZE", "CacheManager", "KVGroup", "KVSpec", "StateSpec", "TokenTensor", "round_up",
            "CacheError", "CacheFull", "FreeList"]

@@ -8,8 +8,11 @@ names it).  Lines with the same needs form a *group* with storage of its own:
 * kind "window": only the last `window` keys are ever read, so a sequence keeps a
   ring of pages and its storage stops growing.
 
-A group holds K and V as [line][page][kv head][row in page][head_dim]; a page has
-`page_size` (64) rows, so one kv head's part of a page is contiguous.  Each group
+What a line keeps per token is a list of named tensors (`TokenTensor`: name, per-token shape,
+dtype), which its mixer states: attention keeps "k" and "v" of [kv heads, head_dim]; another
+mixer may keep one latent row, keys and values of different widths, or a dtype of its own.  A
+tensor of per-token shape (*lead, d) is stored as [line][page][*lead][row in page][d]; a page has
+`page_size` (64) rows, so for keys one kv head's part of a page is contiguous.  Each group
 has its own page pool and its own page table [slot][logical page] -> page.  The
 last slot and the last page of every group are spare: rows that only pad a batch
 point there.  Sequence lengths live in `slot_len`, one int per slot, on the host
@@ -39,11 +42,24 @@ def round_up(n: int, m: int) -> int:
 
 
 @dataclass(frozen=True)
+class TokenTensor:
+    """One tensor a cache line keeps per token: its name, its per-token shape, and its dtype
+    (None: the engine's)."""
+    name: str
+    shape: Tuple[int, ...]
+    dtype: Optional[torch.dtype] = None
+
+    def __post_init__(self):
+        if not self.shape or any(int(n) <= 0 for n in self.shape):
+            raise CacheError(f"per-token tensor {self.name!r} needs a shape of positive sizes")
+
+
+@dataclass(frozen=True)
 class KVSpec:
-    """What one cache line needs: kept keys ("full" or "window"), kv heads, head size."""
+    """What one cache line needs: which tokens are kept ("full": all, "window": the last
+    `window`) and the tensors kept of each."""
     kind: str
-    num_kv_heads: int
-    head_dim: int
+    tensors: Tuple[TokenTensor, ...]
     window: Optional[int] = None
 
     def __post_init__(self):
@@ -51,6 +67,16 @@ class KVSpec:
             raise CacheError(f"unknown cache kind {self.kind!r}")
         if self.kind == "window" and not (self.window and self.window > 0):
             raise CacheError("a window cache needs a positive window")
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise CacheError(f"a cache line needs per-token tensors with distinct names, got {names}")
+
+    @classmethod
+    def keys_values(cls, num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> "KVSpec":
+        """Attention's needs: "k" and "v" of [kv heads, head_dim] in the engine's dtype."""
+        shape = (int(num_kv_heads), int(head_dim))
+        return cls("window" if window else "full",
+                   (TokenTensor("k", shape), TokenTensor("v", shape)), window or None)
 
 
 @dataclass(frozen=True)
@@ -64,15 +90,18 @@ class KVGroup:
     """Storage, page pool and page table of the lines that share one `KVSpec`."""
 
     def __init__(self, spec: KVSpec, lines: Sequence[int], n_slots: int, max_tokens: int,
-                 max_seq_len: int, dtype: torch.dtype, device, page_size: int = PAGE_SIZE):
+                 max_seq_len: int, dtype: torch.dtype, device, page_size: int = PAGE_SIZE,
+                 step_rows: int = 0):
         self.spec = spec
         self.lines = list(lines)
         self.page_size = page_size
         pages_full = max(1, max_tokens // page_size)
         seq_pages = max(1, round_up(max_seq_len, page_size) // page_size)
         if spec.kind == "window":
-            # pages that the last `window` keys of any position can touch
-            self.ring = (spec.window + page_size - 2) // page_size + 1
+            # pages that the last `window` keys of any position can touch, and `step_rows` more
+            # rows: a step stores all its keys before its rows read, so the keys of a step of n
+            # tokens must not reach round the ring into the window of the step's first row
+            self.ring = (spec.window + max(0, step_rows - 1) + page_size - 2) // page_size + 1
             if self.ring >= seq_pages:
                 self.ring = 0           # the window never wraps: same as "full"
         else:
@@ -81,17 +110,37 @@ class KVGroup:
         self.n_pages = min(pages_full, n_slots * self.pages_per_seq)
         self.pool = FreeList(self.n_pages, "page", scatter=True)
         self.spare_page = self.n_pages
-        shape = (len(self.lines), self.n_pages + 1, spec.num_kv_heads, page_size, spec.head_dim)
-        self.k = torch.zeros(shape, dtype=dtype, device=device)
-        self.v = torch.zeros(shape, dtype=dtype, device=device)
+        self.tensors: Dict[str, torch.Tensor] = {}
+        for t in spec.tensors:
+            shape = (len(self.lines), self.n_pages + 1) + tuple(t.shape[:-1]) + (page_size, t.shape[-1])
+            self.tensors[t.name] = torch.zeros(shape, dtype=t.dtype or dtype, device=device)
         self.table_host = torch.full((n_slots + 1, self.pages_per_seq), self.spare_page,
                                      dtype=torch.int32)
         self.table = self.table_host.to(device)
         self.held: Dict[int, List[int]] = {}     # slot -> pages in logical order
         self._dirty = set()
 
+    @property
+    def k(self) -> torch.Tensor:
+        return self.tensors["k"]
+
+    @property
+    def v(self) -> torch.Tensor:
+        return self.tensors["v"]
+
+    @property
+    def step_limit(self) -> Optional[int]:
+        """Most tokens a sequence may go on by in one step so that none of the step's keys lands
+        on a key that a row of the step still reads (None: no limit, nothing wraps)."""
+        return self.ring * self.page_size - self.spec.window + 1 if self.ring else None
+
     def line_index(self, line: int) -> int:
         return self.lines.index(line)
+
+    def _poison(self, pages: Sequence[int]) -> None:
+        for t in self.tensors.values():
+            if pages and t.dtype.is_floating_point:
+                t[:, torch.tensor(list(pages), dtype=torch.long, device=t.device)] = float("nan")
 
     def pages_needed(self, length: int) -> int:
         n = (length + self.page_size - 1) // self.page_size
@@ -112,12 +161,25 @@ class KVGroup:
             pages.append(p)
             self._dirty.add(slot)
 
+    def shrink(self, slot: int, length: int, poison: bool = False) -> None:
+        """Give back the pages that a sequence of only `length` tokens does not need."""
+        pages = self.held.get(slot, [])
+        need = self.pages_needed(length)
+        gone = pages[need:]
+        if not gone:
+            return
+        del pages[need:]
+        if poison:
+            self._poison(gone)
+        for p in gone:
+            self.pool.free(p)
+        self.table_host[slot, need:need + len(gone)] = self.spare_page
+        self._dirty.add(slot)
+
     def release(self, slot: int, poison: bool = False) -> None:
         pages = self.held.pop(slot, [])
-        if poison and pages and self.k.dtype.is_floating_point:
-            idx = torch.tensor(pages, dtype=torch.long, device=self.k.device)
-            self.k[:, idx] = float("nan")
-            self.v[:, idx] = float("nan")
+        if poison:
+            self._poison(pages)
         for p in pages:
             self.pool.free(p)
         self.table_host[slot].fill_(self.spare_page)
@@ -139,7 +201,10 @@ class CacheManager:
 
     def __init__(self, kv_lines: Dict[int, KVSpec], state_lines: Dict[int, StateSpec],
                  max_tokens: int, max_slots: int, max_seq_len: int, dtype: torch.dtype, device,
-                 page_size: int = PAGE_SIZE, poison_freed: bool = False):
+                 page_size: int = PAGE_SIZE, poison_freed: bool = False, step_rows: int = 0):
+        """`step_rows`: the most tokens by which a sequence that already holds tokens goes on in
+        one step without the step being cut (`step_limit`); it sizes the rings of window groups
+        and costs nothing where nothing is a ring."""
         if max_slots <= 0 or max_tokens <= 0 or max_seq_len <= 0:
             raise CacheError("max_slots, max_tokens and max_seq_len must be positive")
         self.page_size = page_size
@@ -155,8 +220,12 @@ class CacheManager:
         for line in sorted(kv_lines):
             by_spec.setdefault(kv_lines[line], []).append(line)
         self.groups: List[KVGroup] = [
-            KVGroup(spec, lines, max_slots, self.max_tokens, max_seq_len, dtype, device, page_size)
+            KVGroup(spec, lines, max_slots, self.max_tokens, max_seq_len, dtype, device, page_size,
+                    step_rows)
             for spec, lines in by_spec.items()]
+        limits = [g.step_limit for g in self.groups if g.step_limit is not None]
+        # most tokens a sequence may bring to a step that reads the cache (None: any number)
+        self.step_limit: Optional[int] = min(limits) if limits else None
         self._group_of: Dict[int, KVGroup] = {l: g for g in self.groups for l in g.lines}
         self.states: Dict[int, torch.Tensor] = {
             line: torch.zeros((max_slots + 1,) + tuple(s.shape), dtype=s.dtype, device=device)
@@ -203,9 +272,29 @@ class CacheManager:
         self._len[slot] = new_len
         self._len_dirty = True
 
-    def extend_all(self, items: Sequence[Tuple[int, int, int]]) -> None:
-        """`extend` for every (slot, start_pos, n_tokens) of a step, or for none of them: if the
-        step as a whole does not fit, CacheFull is raised and the cache is as it was."""
+    def rewind(self, slot: int, n_tokens: int) -> None:
+        """Take the last `n_tokens` of `slot` back: the next step goes on from the shorter
+        sequence and writes over what they left.  Only keys and values can be taken back (a
+        window's ring keeps everything the shorter sequence still sees as long as no more tokens
+        are taken back than a step may bring); fixed-size state cannot, so a cache with state
+        refuses."""
+        if not self.slots.holds(slot):
+            raise CacheError(f"slot {slot} is not held")
+        if self.states:
+            raise CacheError("per-sequence state cannot be taken back by tokens")
+        have = int(self._len[slot])
+        if not 0 <= n_tokens <= have:
+            raise CacheError(f"slot {slot} holds {have} tokens; {n_tokens} cannot be taken back")
+        for g in self.groups:
+            if g.ring and n_tokens > g.step_limit:
+                raise CacheError(f"a window's ring does not keep what {n_tokens} tokens wrote over")
+            g.shrink(slot, have - n_tokens, self.poison_freed)
+        self._len[slot] = have - n_tokens
+        self._len_dirty = True
+
+    def check_room(self, items: Sequence[Tuple[int, int, int]]) -> None:
+        """Raise unless every (slot, start_pos, n_tokens) of a step follows its slot and the step
+        as a whole fits; nothing is changed."""
         for g in self.groups:
             more = 0
             for slot, start, n in items:
@@ -222,6 +311,11 @@ class CacheManager:
             if start + n > self.max_seq_len:
                 raise CacheFull(f"sequence would reach {start + n} tokens; the limit is "
                                 f"{self.max_seq_len}")
+
+    def extend_all(self, items: Sequence[Tuple[int, int, int]]) -> None:
+        """`extend` for every (slot, start_pos, n_tokens) of a step, or for none of them: if the
+        step as a whole does not fit, CacheFull is raised and the cache is as it was."""
+        self.check_room(items)
         for slot, start, n in items:
             self.extend(slot, start, n)
 
@@ -237,10 +331,18 @@ class CacheManager:
 
     # ------------------------------------------------------------ views for parts
     def kv_line(self, line: int):
-        """(K, V, group) of a cache line; K and V are [page, kv head, row, head_dim]."""
+        """(K, V, group) of a cache line that keeps "k" and "v"; K and V are
+        [page, kv head, row, head_dim]."""
         g = self._group_of[line]
         i = g.line_index(line)
         return g.k[i], g.v[i], g
+
+    def token_line(self, line: int):
+        """(name -> tensor [page, *lead, row, d], group) of a cache line: everything it keeps per
+        token."""
+        g = self._group_of[line]
+        i = g.line_index(line)
+        return {name: t[i] for name, t in g.tensors.items()}, g
 
     def state_line(self, line: int) -> Optional[torch.Tensor]:
         return self.states.get(line)

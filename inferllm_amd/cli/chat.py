@@ -173,9 +173,10 @@ def main(argv=None) -> int:
 
         def show(i: int, tok: int) -> None:
             put(tok)
-        # the decode graph of this batch before its first token is timed or awaited
-        eng.warm_up([min(len(prompts), args.max_batch)], max(len(p) for p in prompts) + args.n_predict,
-                    prompt_tokens=max(len(p) for p in prompts))
+        # the decode graph of this batch is captured before the request starts, so that its first
+        # decoded tokens do not wait for the capture; no throwaway prompt is run: for a one-shot
+        # command that would be the whole prompt twice, and `--summary` shows what the user waited
+        eng.warm_up([min(len(prompts), args.max_batch)], max(len(p) for p in prompts) + args.n_predict)
         outs = eng.generate(prompts, temperature=args.temp, top_k=args.top_k, top_p=args.top_p,
                             repeat_penalty=args.repeat_penalty, repeat_last_n=args.repeat_last_n,
                             seed=seed, max_new_tokens=args.n_predict, stop_token_ids=stops,

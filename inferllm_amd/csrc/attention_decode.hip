@@ -1018,14 +1018,27 @@ static __device__ __align__(256) float scratch[ILLM_DECODE_SCRATCH_BYTES / sizeo
 static float* scratch_of_device[ILLM_MAX_DEVICES];     // null until the device's first call
 static std::mutex scratch_lock;
 
-// The address of `scratch` on the current device, looked up at the device's first call.
-static int scratch_here(float** p) {
+// The address of `scratch` on the device that holds `out` (the device the kernels will run on,
+// whichever is current for the calling thread), looked up at that device's first call with that
+// device current.
+static int scratch_of(const void* out, float** p) {
     int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ILLM_MAX_DEVICES) return ILLM_ERR_LAUNCH;
+    hipPointerAttribute_t attr;
+    if (out && hipPointerGetAttributes(&attr, out) == hipSuccess) dev = attr.device;
+    else {
+        (void)hipGetLastError();                        // not a pointer the runtime knows: fall back
+        if (hipGetDevice(&dev) != hipSuccess) return ILLM_ERR_LAUNCH;
+    }
+    if (dev < 0 || dev >= ILLM_MAX_DEVICES) return ILLM_ERR_LAUNCH;
     std::lock_guard<std::mutex> hold(scratch_lock);
     if (!scratch_of_device[dev]) {
+        int current = -1;
+        if (hipGetDevice(&current) != hipSuccess) return ILLM_ERR_LAUNCH;
+        if (current != dev && hipSetDevice(dev) != hipSuccess) return ILLM_ERR_LAUNCH;
         void* q = nullptr;
-        if (hipGetSymbolAddress(&q, HIP_SYMBOL(scratch)) != hipSuccess || !q) return ILLM_ERR_LAUNCH;
+        const hipError_t rc = hipGetSymbolAddress(&q, HIP_SYMBOL(scratch));
+        if (current != dev && hipSetDevice(current) != hipSuccess) return ILLM_ERR_LAUNCH;
+        if (rc != hipSuccess || !q) return ILLM_ERR_LAUNCH;
         scratch_of_device[dev] = (float*)q;
     }
     *p = scratch_of_device[dev];
@@ -1043,7 +1056,7 @@ extern "C" int illm_attn_decode_bf16_static(const void* qkv, void* out, const vo
     if (nsplit > 1) {
         const size_t need = (size_t)B * nh * nsplit * (size_t)(hd + 2) * sizeof(float);
         if (need > ILLM_DECODE_SCRATCH_BYTES) return ILLM_ERR_SCRATCH;
-        const int rc = scratch_here(&partial);
+        const int rc = scratch_of(out, &partial);
         if (rc != ILLM_OK) return rc;
     }
     // every (sequence, head, split) entry that the merge reads is written by the first kernel of

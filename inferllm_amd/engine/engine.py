@@ -15,6 +15,7 @@ import torch
 from ..kernels import ops
 from ..kernels.plan import Plan
 from ..cache.manager import PAGE_SIZE, CacheManager, round_up
+from ..cache.slots import CacheError, CacheFull
 from ..config.registry import config_from_dict, load_config
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
@@ -53,6 +54,10 @@ class Engine:
     the ways for shapes the tables lack (thin matrices now, many-row products at first use) and
     keeps the winners in `engine.plan`; `plan=` (a `Plan` or what its `to_dict()` gave) pins them.
 
+    `step_rows`: a cache line that keeps a window of keys is a ring of pages with room for the
+    window and this many rows more; a sequence that goes on from earlier tokens by more than
+    that in one step has the step run in pieces.  Models without windows ignore it.
+
     Cache size: `max_tokens` is the most tokens live sequences hold together (each
     rounded up to 64), `max_batch` the most live sequences, `max_seq_len` the longest
     sequence (default: the model's max positions).
@@ -61,7 +66,8 @@ class Engine:
     def __init__(self, config, tensors: Dict[str, torch.Tensor], dtype, device="cuda:0",
                  max_batch: int = 8, max_seq_len: Optional[int] = None,
                  max_tokens: Optional[int] = None, use_graphs: bool = True,
-                 poison_freed: bool = False, decode_copies=None, tune: bool = False, plan=None):
+                 poison_freed: bool = False, decode_copies=None, tune: bool = False, plan=None,
+                 step_rows: int = 512):
         self.config = config
         self.dtype = parse_dtype(dtype)
         self.device = torch.device(device)
@@ -93,27 +99,11 @@ class Engine:
             plan = Plan.from_dict(plan)
         self.plan: Plan = plan if plan is not None else Plan.fixed(measure=bool(tune))
         if self.plan.measure and self.dtype == torch.bfloat16:
-            ops.use_plan(self.plan)
+            # what each part lists as having several ways (`Part.tunables`); the engine knows no
+            # part's fields
             for part in self.model.every_part():
-                for w in vars(part).values():
-                    if (isinstance(w, ops.Weight) and w.tiled is not None and w.mode == "plain"
-                            and tuple(w.shape) not in self.plan.planes_from
-                            and w.shape[1] >= 2 * w.shape[0] and w.shape[0] <= ops.MID_MAX_COLS
-                            and w.shape[0] % 4 == 0):
-                        self.plan.planes_from[tuple(w.shape)] = ops.measure_planes_from(w)
-                # a mixer that keeps a fused q|k|v matrix in its fused kernel's tile order
-                w = getattr(part, "w_qkv", None)
-                if (isinstance(w, ops.Weight) and w.mode == "qkv" and w.tiled is not None
-                        and w.shape[1] % 64 == 0
-                        and ("qkv",) + tuple(w.shape) not in self.plan.rows_from):
-                    self.plan.rows_from[("qkv",) + tuple(w.shape)] = ops.measure_rows_from_qkv(
-                        w, part.nh, part.nkv, part.hd)
-                # a feed-forward that keeps a fused gate|up matrix likewise
-                w = getattr(part, "w_gate_up", None)
-                if (isinstance(w, ops.Weight) and w.mode == "gate_up" and w.tiled is not None
-                        and w.shape[1] % 64 == 0
-                        and ("gate_up",) + tuple(w.shape) not in self.plan.rows_from):
-                    self.plan.rows_from[("gate_up",) + tuple(w.shape)] = ops.measure_rows_from_gate_up(w)
+                for kind, w, geometry in part.tunables():
+                    ops.tune_product(self.plan, kind, w, **geometry)
         limit = self.spec.max_positions
         self.max_seq_len = min(int(max_seq_len), limit) if max_seq_len else limit
         self.max_batch = int(max_batch)
@@ -122,7 +112,8 @@ class Engine:
         self.cache = CacheManager(self.model.kv_lines(), self.model.state_lines(),
                                   max_tokens=int(max_tokens), max_slots=self.max_batch,
                                   max_seq_len=self.max_seq_len, dtype=self.dtype,
-                                  device=self.device, poison_freed=poison_freed)
+                                  device=self.device, poison_freed=poison_freed,
+                                  step_rows=int(step_rows))
         self.runner = StepRunner(self.model, self.cache, self.dtype, self.device, use_graphs,
                                  plan=self.plan)
         self.last_stats: Optional[GenerationStats] = None
@@ -170,10 +161,24 @@ class Engine:
     def free_slot(self, slot: int) -> None:
         self.cache.free_slot(slot)
 
-    def step(self, entries: Sequence[StepEntry],
-             device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-        """See `StepRunner.step`.  The returned tensor is valid until the next step."""
-        return self.runner.step(entries, device_tokens)
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None,
+             borrow: bool = False) -> Optional[torch.Tensor]:
+        """See `StepRunner.step`.  The returned tensor is the caller's; with `borrow` it may be
+        memory that the next step writes again."""
+        return self.runner.step(entries, device_tokens, borrow)
+
+    def generation_loop(self, sampler: Sampler, on_token=None, max_step_tokens: Optional[int] = None,
+                        ahead: bool = True) -> GenerationLoop:
+        """The generation loop over this engine's step function, cache and `sampler`.  `ahead`:
+        every step is started before the tokens of the step before it have been read."""
+        step = lambda entries, device_tokens=None: self.runner.step(entries, device_tokens, borrow=True)
+        return GenerationLoop(step, sampler, self.alloc_slot, self.free_slot,
+                              max_batch=self.max_batch, max_tokens=self.cache.max_tokens,
+                              max_seq_len=self.max_seq_len, page_size=self.cache.page_size,
+                              sync=lambda: torch.cuda.synchronize(self.device), on_token=on_token,
+                              draw=sampler.draw if ahead else None, max_step_tokens=max_step_tokens,
+                              keep=lambda logits, row: logits[row].clone(), join=torch.stack,
+                              rewind_slot=self.cache.rewind)
 
     def session(self, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0,
                 repeat_penalty: float = 1.0, repeat_last_n: int = 64, seed: int = 0,
@@ -200,9 +205,14 @@ class Engine:
         captured = self.runner.warm_up(batch_sizes, min(int(longest), self.max_seq_len))
         n = min(int(prompt_tokens), self.max_seq_len)
         if n > 0:
-            slot = self.alloc_slot()
+            try:
+                slot = self.alloc_slot()
+            except CacheError:
+                return captured                  # every slot is in use: nothing to warm up with
             try:
                 self.step([StepEntry(slot, [0] * n, [n - 1])])
+            except CacheFull:
+                pass                             # no room for a throwaway prompt now: skipped
             finally:
                 self.free_slot(slot)
         return captured
@@ -236,12 +246,7 @@ class Engine:
         if max_step_tokens is not None and self.model.one_token_mixers:
             raise ValueError("max_step_tokens: this model's " + ", ".join(self.model.one_token_mixers)
                              + " cannot go on from the cache by several tokens")
-        loop = GenerationLoop(self.step, sampler, self.alloc_slot, self.free_slot,
-                              max_batch=self.max_batch, max_tokens=self.cache.max_tokens,
-                              max_seq_len=self.max_seq_len, page_size=self.cache.page_size,
-                              sync=lambda: torch.cuda.synchronize(self.device), on_token=on_token,
-                              draw=sampler.draw, max_step_tokens=max_step_tokens,
-                              join=lambda pieces: torch.stack([lg[row] for lg, row in pieces]))
+        loop = self.generation_loop(sampler, on_token, max_step_tokens)
         out = loop.run(prompts, params, max_new_tokens, stops, include_stop)
         self.last_stats = loop.stats
         return out

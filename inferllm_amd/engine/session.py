@@ -6,19 +6,17 @@ tokens at `m_past`, src/core/model_imp.cpp:38-52), then tokens are decoded one b
 the end token (`decode_iter`, :55-65; the loop is application/chat.cpp:221-275), and the token
 that ended a turn is never run through the model.  A `Session` does the same with one slot of
 the cache: the tokens of a turn are one step that goes on from the slot's length, the answer
-is decoded from there, and the slot is given back when the session is closed.
+is decoded from there, and the slot is given back when the session is closed.  The decoding is
+the generation loop's, with a batch of one in a slot that the session owns, so a conversation
+runs one step ahead of the host like any other batch.
 """
 from __future__ import annotations
 
-import time
 from typing import Callable, List, Optional, Sequence
-
-import torch
 
 from ..sampling.params import SamplingParams, request_seed
 from ..sampling.sampler import Sampler
 from .generate import GenerationStats
-from .step import StepEntry
 
 
 class Session:
@@ -74,20 +72,20 @@ class Session:
         self.close()
 
     # ------------------------------------------------------------ a turn
-    def _draw(self, logits: torch.Tensor) -> int:
-        hist = [self.history] if self.sampler.needs_histories() else None
-        token = self.sampler(logits, [self.seed], [self.drawn], hist)[0]
-        self.drawn += 1
-        self.history.append(token)
-        return token
-
     def say(self, tokens: Sequence[int], max_new_tokens: int = 128,
             on_token: Optional[Callable[[int], None]] = None, include_stop: bool = False) -> List[int]:
         """Feed `tokens` after what was said so far and generate until a stop token, until
         `max_new_tokens` are drawn or until the context is full.  `on_token(token)` is called for
-        every token as it comes.  Raises ValueError if the turn does not fit into the context."""
+        every token as it comes.  Raises ValueError if the turn does not fit into the context.
+
+        A step that the cache has no room for raises (`CacheFull`; the page pool is shared with
+        other sessions and batches).  The session then stands where the last step that ran left
+        it: a turn whose first step found no room has not happened; an answer that broke off
+        keeps the tokens shown so far (the exception carries them as `generated`), and the next
+        turn goes on behind them."""
         self._open()
-        vocab = self.engine.spec.vocab_size
+        engine = self.engine
+        vocab = engine.spec.vocab_size
         turn = [int(t) for t in tokens]
         for t in turn:
             if not 0 <= t < vocab:
@@ -95,38 +93,43 @@ class Session:
         feed = ([self._unfed] if self._unfed is not None else []) + turn
         if not feed:
             raise ValueError("a turn needs at least one token")
-        if len(feed) > self.engine.max_seq_len - self.length:
+        held = self.length
+        if len(feed) > engine.max_seq_len - held:
             raise ValueError(f"the turn's {len(turn)} tokens do not fit: {self.remaining} tokens of "
                              f"the context are left")
-        stats = self.last_stats = GenerationStats(prompt_tokens=len(feed), batches=1)
-        sync = lambda: torch.cuda.synchronize(self.engine.device)
-        out: List[int] = []
-        sync()
-        start = time.perf_counter()
-        # (a step that the cache has no room for raises before it changes anything: the session
-        # stays as it was)
-        logits = self.engine.step([StepEntry(self.slot, feed, [len(feed) - 1])])
-        self.history.extend(turn)
-        self._unfed = None
-        token = self._draw(logits)
-        sync()
-        stats.prefill_seconds = time.perf_counter() - start
-        start = time.perf_counter()
-        while True:
-            stop = token in self.stops
-            if not stop or include_stop:
-                out.append(token)
-                stats.generated_tokens += 1
-                if on_token is not None:
-                    on_token(token)
-            if stop:
-                break                                   # (the token that ends a turn is not run)
-            if len(out) >= max_new_tokens or self.engine.max_seq_len - self.length < 1:
-                self._unfed = token                     # shown, to be run with the next turn
-                break
-            logits = self.engine.step([StepEntry(self.slot, [token], [0])])
-            token = self._draw(logits)
-            stats.decode_steps += 1
-        sync()
-        stats.decode_seconds = time.perf_counter() - start
-        return out
+        # a void step (the one the loop has started when a stop token turns up) can be taken back
+        # from keys and values, not from a mixer's own state: such a model is decoded in step
+        loop = engine.generation_loop(self.sampler, ahead=not engine.cache.states,
+                                      on_token=(lambda _i, tok: on_token(tok)) if on_token else None)
+        self.last_stats = loop.stats
+        history = self.history + turn
+        record = None
+        try:
+            record = loop.run_turn(self.slot, held, feed, history, self.seed, self.drawn,
+                                   max_new_tokens, self.stops, include_stop)
+        except Exception as e:
+            now = engine.cache.length(self.slot)
+            if now == held:
+                raise                                   # the turn's first step did not run
+            if now < held + len(feed):
+                self.close()                            # a part of the turn ran: nothing to go on from
+                raise
+            # the turn ran and `history` holds every token that was read since; all of them
+            # were run except, when the loop decodes in step, the newest
+            answer = history[len(self.history) + len(turn):]
+            self._settle(history, held + len(feed), len(answer))
+            self.history = history
+            e.generated = list(answer)
+            raise
+        self._settle(history, held + len(feed), record.drawn)
+        self.history = history
+        if record.why == "stop":
+            self._unfed = None                          # the token that ends a turn is never run
+        return record.out
+
+    def _settle(self, history: List[int], fed_len: int, drawn: int) -> None:
+        """After a turn (or what ran of it): count the draws and find the token that was shown
+        but not run, from what the cache holds."""
+        self.drawn += drawn
+        missing = fed_len + drawn - self.engine.cache.length(self.slot)
+        self._unfed = history[-1] if drawn > 0 and missing >= 1 else None

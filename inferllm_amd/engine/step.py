@@ -1,8 +1,8 @@
 """The step function: one batch of sequences, either all at their first token
 (whole prompts of unequal lengths) or all going on by one token; if every mixer of
-the model says it can go on from what it kept by several tokens (attention without a
-window does: its rows then attend over the paged cache), also any mix of starting
-sequences and sequences that go on by any number of tokens (a prompt cut into steps).
+the model says it can go on from what it kept by several tokens (attention does: its rows
+then attend over the paged cache), also any mix of starting sequences and sequences that
+go on by any number of tokens (a prompt cut into steps, a conversation's next turn).
 
 It runs only the tokens it is given, packed as one batch, against the cache that
 earlier steps left, and returns float32 logits at the places asked for.  Steps
@@ -134,15 +134,19 @@ class StepRunner:
 
     # ------------------------------------------------------------ the step
     @torch.no_grad()
-    def step(self, entries: Sequence[StepEntry],
-             device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None,
+             borrow: bool = False) -> Optional[torch.Tensor]:
         """Run one step; float32 logits [wanted, vocab] in the order of the entries
         and of their `want`, or None when nothing is wanted.
 
         `device_tokens` (a step of single tokens only): int32 [len(entries)] on the device, the
         token of every entry in order, in place of the entries' own (which are placeholders
         then).  It lets a caller start the next step from tokens that were chosen on the device
-        before it has read them back."""
+        before it has read them back.
+
+        `borrow`: the result may be a view of memory that the next step writes again (a decode
+        graph's output); a caller that has used it up by then saves a copy.  Without it the
+        result is the caller's to keep."""
         prefill = self._phase(entries)          # True: a step of several tokens per sequence
         if self.plan is not None:
             ops.use_plan(self.plan)
@@ -153,11 +157,42 @@ class StepRunner:
                     or device_tokens.shape != (len(entries),)):
                 raise StepError(f"device_tokens must be int32 [{len(entries)}] on {self.device}")
         starts = [self.cache.length(e.slot) for e in entries]
+        limit = self.cache.step_limit
+        if (prefill and limit is not None and any(starts)
+                and max(len(e.tokens) for e in entries) > limit):
+            return self._in_pieces(entries, starts, limit)
         self.cache.extend_all([(e.slot, s, len(e.tokens)) for e, s in zip(entries, starts)])
         self.cache.upload(lengths=prefill)
         if prefill:
             return self._prefill(entries, starts)
-        return self._decode(entries, starts, device_tokens)
+        return self._decode(entries, starts, device_tokens, borrow)
+
+    def _in_pieces(self, entries: Sequence[StepEntry], starts: Sequence[int],
+                   limit: int) -> Optional[torch.Tensor]:
+        """A step that reads the cache and brings some sequence more tokens than a window's ring
+        of pages keeps apart, as several steps of at most `limit` tokens a sequence: a step
+        stores all its keys before its rows read, and a longer one would write round the ring
+        onto keys that its first rows still see.  The logits come out in the whole step's order."""
+        self.cache.check_room([(e.slot, s, len(e.tokens)) for e, s in zip(entries, starts)])
+        pieces, keys = [], []
+        for lo in range(0, max(len(e.tokens) for e in entries), limit):
+            part = []
+            for i, e in enumerate(entries):
+                if lo >= len(e.tokens):
+                    continue
+                want = [(j, int(w) - lo) for j, w in enumerate(e.want) if lo <= int(w) < lo + limit]
+                part.append(StepEntry(e.slot, e.tokens[lo:lo + limit], [w for _, w in want]))
+                keys.extend((i, j) for j, _ in want)
+            out = self.step(part)
+            if out is not None:
+                pieces.append(out)
+        if not pieces:
+            return None
+        logits = pieces[0] if len(pieces) == 1 else torch.cat(pieces, dim=0)
+        order = sorted(range(len(keys)), key=keys.__getitem__)
+        if order != list(range(len(keys))):
+            logits = logits[torch.tensor(order, dtype=torch.long, device=self.device)]
+        return logits
 
     def _prefill(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> Optional[torch.Tensor]:
         tokens: List[int] = []
@@ -192,7 +227,8 @@ class StepRunner:
         return self.model.forward(ctx, parts[7] if want else None)
 
     def _decode(self, entries: Sequence[StepEntry], starts: Sequence[int],
-                device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                device_tokens: Optional[torch.Tensor] = None,
+                borrow: bool = False) -> Optional[torch.Tensor]:
         B = len(entries)
         size = _bucket(B) if self.use_graphs else B
         pad = size - B
@@ -232,7 +268,8 @@ class StepRunner:
         if not wanted:
             return None
         if wanted == list(range(B)):
-            return g.logits[:B]
+            # the graph's own output, which its next replay writes again
+            return g.logits[:B] if borrow else g.logits[:B].clone()
         return g.logits[torch.tensor(wanted, dtype=torch.long, device=self.device)]
 
     @torch.no_grad()

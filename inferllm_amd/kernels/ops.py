@@ -506,6 +506,41 @@ def measure_planes_from(w: "Weight") -> int:
     return first
 
 
+def tune_product(plan: Plan, kind: str, w, votes: int = 1, **geometry) -> Optional[tuple]:
+    """Time what the plan's tables lack for one product a part lists (`Part.tunables`) and enter
+    it: for a thin "plain" matrix from how few rows the planes pay, for a fused "qkv" or
+    "gate_up" matrix from how few rows the kernels that share X do.  The median of `votes`
+    measurements.  Returns (table, key, value) of the new entry, or None if nothing was timed
+    (no decode copy, a shape the kernels do not take, an entry that is there)."""
+    if not (isinstance(w, Weight) and w.tiled is not None and w.mode == kind):
+        return None
+    N, K = w.shape
+    if kind == "plain":
+        key, table = (N, K), plan.planes_from
+        fits = K >= 2 * N and N <= MID_MAX_COLS and N % 4 == 0
+        measure = lambda: measure_planes_from(w)
+    elif kind == "qkv":
+        key, table = ("qkv", N, K), plan.rows_from
+        fits = K % 64 == 0
+        measure = lambda: measure_rows_from_qkv(w, geometry["nh"], geometry["nkv"], geometry["hd"])
+    elif kind == "gate_up":
+        key, table = ("gate_up", N, K), plan.rows_from
+        fits = K % 64 == 0
+        measure = lambda: measure_rows_from_gate_up(w)
+    else:
+        raise ValueError(f"unknown kind of product {kind!r}")
+    if not fits or key in table:
+        return None
+    saved, current = _plan, plan
+    use_plan(current)
+    try:
+        runs = sorted(measure() for _ in range(max(1, votes)))
+    finally:
+        use_plan(saved)
+    table[key] = runs[len(runs) // 2]
+    return ("planes_from" if kind == "plain" else "rows_from"), key, table[key]
+
+
 def linear_planes_pays(x, w) -> bool:
     """Whether the planes are the faster way for these operands (which `linear_planes_fits`).
     From 17 to 64 rows always.  Up to 16 rows `linear_add` reads X once per

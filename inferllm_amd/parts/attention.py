@@ -35,12 +35,11 @@ class Attention(Mixer):
     adds_residual = True
     takes_normed_rows = True
 
-    @property
-    def takes_continuations(self) -> bool:
-        """A step of several tokens may go on from keys the cache holds (a prompt cut into
-        steps): its rows then attend over the paged cache.  Not with a window, whose ring of
-        pages a long step overwrites while it is still read."""
-        return self.window is None
+    # A step of several tokens may go on from keys the cache holds (a prompt cut into steps, a
+    # conversation's next turn): its rows then attend over the paged cache.  With a window the
+    # cache keeps a ring of pages; the step function cuts a step that would write round the ring
+    # into what its own first rows still read (`CacheManager.step_limit`).
+    takes_continuations = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: Optional[int] = None, softmax_scale: Optional[float] = None, tensors=None):
@@ -62,7 +61,7 @@ class Attention(Mixer):
                 "o": TensorWant((self.E, self.nh * self.hd))}
 
     def kv_spec(self) -> KVSpec:
-        return KVSpec("window" if self.window else "full", self.nkv, self.hd, self.window)
+        return KVSpec.keys_values(self.nkv, self.hd, self.window)
 
     def load(self, tensors) -> None:
         # the decode copy of q|k|v follows the tiles of the position encoding's fused kernel, if it
@@ -73,6 +72,10 @@ class Attention(Mixer):
                                        mode, self.decode_copies, **geometry)
         self.w_o = ops.decode_weight(self._take(tensors, "o").contiguous(), "plain",
                                      self.decode_copies)
+
+    def tunables(self):
+        return (("qkv", self.w_qkv, dict(nh=self.nh, nkv=self.nkv, hd=self.hd)),
+                ("plain", self.w_o, {}))
 
     def forward(self, h, ctx: StepContext, line, writes_cache, position, residual=None,
                 next_norm=None):

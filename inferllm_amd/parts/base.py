@@ -90,6 +90,14 @@ class Part:
     def _take(self, tensors: Dict[str, torch.Tensor], param: str) -> torch.Tensor:
         return tensors[self.tensors[param]]
 
+    def tunables(self):
+        """The part's products that have several equivalent ways, for whoever times them (an
+        engine built with `tune=True`, `kernels.tune`): tuples (kind, weight, geometry), kind
+        "plain" (a matrix of ordinary products), "gate_up" (a fused gate|up matrix in its fused
+        kernel's tile order) or "qkv" (a fused q|k|v matrix likewise; geometry `nh`, `nkv`, `hd`).
+        A part that lists nothing is never timed and takes the rule for unlisted shapes."""
+        return ()
+
 
 class Mixer(Part):
     # The position encoding of the mixer's block, set by the block before `load` (None: none).

@@ -39,6 +39,9 @@ class SwiGLU(FeedForward):
         self.w_down = ops.decode_weight(self._take(tensors, "down").contiguous(), "plain",
                                         self.decode_copies)
 
+    def tunables(self):
+        return (("gate_up", self.w_gate_up, {}), ("plain", self.w_down, {}))
+
     def forward(self, h, ctx: StepContext, residual=None, next_norm=None):
         a = ops.gate_up_silu(h, self.w_gate_up)
         if (next_norm is not None and getattr(next_norm, "adds_planes", False)

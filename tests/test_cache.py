@@ -9,7 +9,7 @@ from inferllm_amd.cache import (CacheError, CacheFull, CacheManager, FreeList, K
 
 
 def manager(max_tokens=64 * 8, max_slots=4, max_seq_len=256, lines=None, states=None):
-    lines = lines if lines is not None else {0: KVSpec("full", 2, 16), 1: KVSpec("full", 2, 16)}
+    lines = lines if lines is not None else {0: KVSpec.keys_values(2, 16), 1: KVSpec.keys_values(2, 16)}
     return CacheManager(lines, states or {}, max_tokens, max_slots, max_seq_len,
                         torch.float32, "cpu")
 
@@ -112,8 +112,8 @@ def test_a_step_that_does_not_fit_leaves_the_cache_as_it_was():
 
 
 def test_groups_with_different_needs_have_their_own_storage():
-    lines = {0: KVSpec("full", 2, 16), 1: KVSpec("window", 2, 16, window=70), 2: KVSpec("full", 4, 8),
-             3: KVSpec("window", 2, 16, window=70)}
+    lines = {0: KVSpec.keys_values(2, 16), 1: KVSpec.keys_values(2, 16, window=70), 2: KVSpec.keys_values(4, 8),
+             3: KVSpec.keys_values(2, 16, window=70)}
     m = CacheManager(lines, {}, 64 * 32, 2, 1024, torch.bfloat16, "cpu")
     assert len(m.groups) == 3
     k0, v0, g0 = m.kv_line(0)
@@ -157,9 +157,72 @@ def test_fixed_size_state_is_zeroed_when_a_slot_is_handed_out():
 
 
 def test_freed_pages_can_be_poisoned():
-    m = CacheManager({0: KVSpec("full", 1, 8)}, {}, 128, 2, 128, torch.float32, "cpu", poison_freed=True)
+    m = CacheManager({0: KVSpec.keys_values(1, 8)}, {}, 128, 2, 128, torch.float32, "cpu", poison_freed=True)
     s = m.alloc_slot()
     m.extend(s, 0, 3)
     page = m.groups[0].held[s][0]
     m.free_slot(s)
     assert torch.isnan(m.kv_line(0)[0][page]).all()
+
+
+def test_tokens_can_be_taken_back():
+    """`rewind`: the last tokens of a sequence are given up (the void step behind a stop token);
+    pages that the shorter sequence does not need go back to the pool, a window's ring keeps its
+    pages, and state of fixed size refuses."""
+    m = CacheManager({0: KVSpec.keys_values(2, 16), 1: KVSpec.keys_values(2, 16, window=70)}, {}, 64 * 8, 2, 512,
+                     torch.float32, "cpu", poison_freed=True)
+    full, ring = m.groups
+    s = m.alloc_slot()
+    m.extend(s, 0, 129)
+    assert len(full.held[s]) == 3 and len(ring.held[s]) == 3
+    third = full.held[s][2]
+    m.rewind(s, 1)
+    assert m.length(s) == 128 and len(full.held[s]) == 2 and len(ring.held[s]) == 2
+    assert torch.isnan(m.kv_line(0)[0][third]).all() and int(full.table_host[s, 2]) == full.spare_page
+    m.check()
+    m.extend(s, 128, 200)                                   # the next step goes on from the shorter sequence
+    assert m.length(s) == 328 and len(ring.held[s]) == 3 and len(full.held[s]) == 6
+    assert ring.step_limit == 3 * 64 - 70 + 1 and m.step_limit == ring.step_limit
+    with pytest.raises(CacheError, match="ring"):
+        m.rewind(s, ring.step_limit + 1)                    # the ring has written over what that needs
+    with pytest.raises(CacheError, match="cannot be taken back"):
+        m.rewind(s, 329)
+    m.rewind(s, 0)
+    m.free_slot(s)
+    m.check()
+    with_state = CacheManager({0: KVSpec.keys_values(1, 8)}, {0: StateSpec((4,))}, 128, 2, 128, torch.float32, "cpu")
+    s = with_state.alloc_slot()
+    with_state.extend(s, 0, 5)
+    with pytest.raises(CacheError, match="state"):
+        with_state.rewind(s, 1)
+
+
+def test_a_line_keeps_the_per_token_tensors_its_mixer_names():
+    """Keys and values are one case: a line may keep one latent row a token, tensors of different
+    widths, or a dtype of its own; lines with the same needs share a group."""
+    from inferllm_amd.cache import TokenTensor
+    latent = KVSpec("full", (TokenTensor("latent", (24,), torch.float32),))
+    uneven = KVSpec("window", (TokenTensor("k", (2, 32)), TokenTensor("v", (2, 8), torch.float16)), window=100)
+    m = CacheManager({0: latent, 1: KVSpec.keys_values(2, 16), 2: latent, 3: uneven}, {}, 64 * 8, 2, 1024,
+                     torch.bfloat16, "cpu", step_rows=300)
+    assert len(m.groups) == 3
+    kept, g = m.token_line(2)
+    assert set(kept) == {"latent"} and kept["latent"].shape == (g.n_pages + 1, 64, 24)
+    assert kept["latent"].dtype == torch.float32 and g.lines == [0, 2]
+    kept, g = m.token_line(3)
+    assert kept["k"].shape[1:] == (2, 64, 32) and kept["k"].dtype == torch.bfloat16
+    assert kept["v"].shape[1:] == (2, 64, 8) and kept["v"].dtype == torch.float16
+    assert g.ring == 8 and m.step_limit == 8 * 64 - 100 + 1 >= 300   # ceil((100 - 1 + 299) / 64) + 1 pages
+    k, v, _ = m.kv_line(1)
+    assert k.shape[1:] == (2, 64, 16) and v.dtype == torch.bfloat16
+    with pytest.raises(KeyError):
+        m.kv_line(0)                                        # that line keeps no keys and values
+    with pytest.raises(CacheError, match="distinct names"):
+        KVSpec("full", (TokenTensor("a", (4,)), TokenTensor("a", (4,))))
+    with pytest.raises(CacheError, match="positive"):
+        TokenTensor("a", ())
+    s = m.alloc_slot()
+    m.extend(s, 0, 70)
+    assert all(len(g.held[s]) == 2 for g in m.groups)
+    m.free_slot(s)
+    m.check()

@@ -325,3 +325,92 @@ def test_command_line_text_through_a_sentencepiece_model(tmp_path, capsys):
     put = _Text(str(empty)).printer()
     put(3); put(4)
     assert capsys.readouterr().out == "3 4 "
+
+
+class TurnModel(FakeModel):
+    """A fake model whose slots the caller owns, with `rewind`."""
+
+    def rewind(self, slot, n):
+        assert 0 < n <= len(self.seq[slot])
+        del self.seq[slot][-n:]
+        self.rewound = getattr(self, "rewound", 0) + n
+
+
+@AHEAD
+def test_a_turn_in_a_slot_that_the_caller_owns(ahead):
+    """`run_turn`: one sequence goes on, in a slot that is not given back, from what it holds;
+    the loop leaves in it everything that was run.  A stop token is never run: when the loop
+    runs ahead its void step is taken back from the slot."""
+    m = TurnModel(2, takes_cut_prompts=True)
+    loop = GenerationLoop(m.step, m.sample, m.alloc, m.release, 2, 6400, 256, draw=m.draw if ahead else None,
+                          rewind_slot=m.rewind)
+    slot = m.alloc()
+    first = [4, 4, 9]
+    history = list(first)
+    r = loop.run_turn(slot, 0, first, history, seed=1, draws_before=0, max_new_tokens=4)
+    want = expected(first, 4)
+    assert r.out == want and r.why == "length" and history == first + want
+    assert m.seq[slot] == first + want[:3]                   # the last drawn token is still to be run
+    # the next turn brings that token in front of its own; a stop token ends it
+    turn = [want[3], 7, 1]
+    said = first + want + [7, 1]
+    ans = expected(said, 6)
+    stop = ans[2]
+    history += [7, 1]
+    r = loop.run_turn(slot, len(m.seq[slot]), turn, history, seed=1, draws_before=4, max_new_tokens=6,
+                      stop_token_ids=[stop])
+    j = ans.index(stop)
+    assert r.out == ans[:j] and r.why == "stop" and r.drawn == j + 1
+    assert m.seq[slot] == said + ans[:j]                    # the stop token is not in the slot
+    assert getattr(m, "rewound", 0) == (1 if ahead else 0)
+    assert slot in m.seq and len(m.free) == 1               # the slot is still the caller's
+    assert loop.stats.prompt_tokens == 6 and loop.stats.batches == 2    # the loop's stats add up over its calls
+    with pytest.raises(ValueError, match="at least one token"):
+        loop.run_turn(slot, len(m.seq[slot]), [], history, 1, 0, 3)
+    if ahead:
+        with pytest.raises(ValueError, match="rewind_slot"):
+            GenerationLoop(m.step, m.sample, m.alloc, m.release, 2, 6400, 256, draw=m.draw).run_turn(
+                slot, len(m.seq[slot]), [1], history, 1, 0, 3)
+
+
+def test_a_turn_counts_draws_and_lengths_from_what_the_slot_holds():
+    """The sampler's counter goes on from the draws before, and the context's end is counted
+    with the tokens the slot held before the turn."""
+    calls = []
+
+    def draw(logits, seeds, counters, histories, latest=None):
+        calls.append(list(counters))
+        return FakeDraw(list(logits))
+    m = TurnModel(1, takes_cut_prompts=True)
+    loop = GenerationLoop(m.step, m.sample, m.alloc, m.release, 1, 6400, max_seq_len=10, draw=draw,
+                          rewind_slot=m.rewind)
+    slot = m.alloc()
+    m.seq[slot] = [1, 2, 3, 4, 5, 6]
+    history = [1, 2, 3, 4, 5, 6, 7, 8]
+    r = loop.run_turn(slot, 6, [7, 8], history, seed=0, draws_before=11, max_new_tokens=50)
+    assert calls[0] == [11] and calls[1] == [12]
+    assert r.why == "context" and len(m.seq[slot]) == 10 and len(r.out) == 3   # the third cannot be run any more
+    assert r.out == expected([1, 2, 3, 4, 5, 6, 7, 8], 50, limit=10)
+
+
+def test_logits_of_a_prompt_that_ended_are_taken_out_at_once():
+    """A step's logits may be memory that the next step writes again (a decode graph's output):
+    when prompts are fed in several steps, the loop keeps a prompt's last-token row through
+    `keep` before the next step runs."""
+    buffer = [None]                                          # the one place every step writes to
+
+    class Reusing(FakeModel):
+        def step(self, entries, device_tokens=None):
+            rows = super().step(entries, device_tokens)
+            if rows is None:
+                return None
+            buffer[0] = list(rows)
+            return buffer                                    # a view: logits[0] is the live list
+
+    m = Reusing(3, takes_cut_prompts=True)
+    loop = GenerationLoop(m.step, lambda lg, *a: [row[0] if isinstance(row, list) else row for row in lg],
+                          m.alloc, m.release, 3, 6400, 256, max_step_tokens=1,
+                          keep=lambda logits, row: list(logits[0])[row], join=list)
+    prompts = [[1, 2, 3], [7, 5], [4, 4]]
+    out = loop.run(prompts, SamplingParams(), 1)
+    assert out == [expected(p, 1) for p in prompts]

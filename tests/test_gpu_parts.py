@@ -906,3 +906,253 @@ def test_toy_embedding_and_toy_head(tmp_path):
         if float(top2[0] - top2[1]) > 1e-4:                      # a near tie may go either way
             assert t == int(torch.argmax(logits))
         seq.append(t)
+
+
+# ---------------------------------------------------------------- windows and steps that go on
+def _windowed_architecture(name, E, V, nh, nkv, hd, F, eps, theta, windows, max_pos=1024):
+    """A toy architecture whose layer i is attention with window windows[i] (None: all keys)."""
+    from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+
+    @register_architecture(name)
+    class Cfg:
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": [name]}
+
+        def to_spec(self):
+            norm = lambda n: PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": n})
+            layers = [LayerSpec("pre_norm",
+                                PartSpec("attention", {"hidden_size": E, "num_heads": nh, "num_kv_heads": nkv,
+                                                       "head_dim": hd, "window": win},
+                                         {k: f"l{i}.{k}" for k in "qkvo"}),
+                                PartSpec("swiglu", {"hidden_size": E, "intermediate_size": F},
+                                         {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+                                norm(f"l{i}.n1"), norm(f"l{i}.n2"),
+                                PartSpec("rotary", {"head_dim": hd, "rotary_dim": hd, "theta": theta,
+                                                    "pairing": "half", "max_positions": max_pos}))
+                      for i, win in enumerate(windows)]
+            return ModelSpec(name, V, E, max_pos,
+                             PartSpec("token_embedding", {"vocab_size": V, "hidden_size": E}, {"weight": "emb"}),
+                             layers, [ScheduleEntry(i, i) for i in range(len(windows))], norm("nf"),
+                             PartSpec("lm_head", {"hidden_size": E, "vocab_size": V}, {"weight": "head"}))
+
+    def plain(w, ids):
+        S = len(ids)
+        pos = list(range(S))
+        x = P.embedding(w["emb"], ids)
+        for i, win in enumerate(windows):
+            h = P.rms_norm(x, w[f"l{i}.n1"], eps)
+            q = P.rope_rotate_half(P.linear(h, w[f"l{i}.q"]).reshape(S, nh, hd), pos, theta)
+            k = P.rope_rotate_half(P.linear(h, w[f"l{i}.k"]).reshape(S, nkv, hd), pos, theta)
+            v = P.linear(h, w[f"l{i}.v"]).reshape(S, nkv, hd)
+            x = x + P.linear(P.causal_attention(q, k, v, window=win), w[f"l{i}.o"])
+            x = x + P.swiglu_ffn(P.rms_norm(x, w[f"l{i}.n2"], eps), w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+        return P.linear(P.rms_norm(x, w["nf"], eps), w["head"])
+    return Cfg, plain
+
+
+def _scaled(d, gain):
+    """The folder's matrices (not the embedding or the head) times `gain`, so that attention is
+    far from uniform and a wrong or missing key moves the logits by their own size."""
+    import os
+    from inferllm_amd.weights import open_model_files, write_safetensors
+    tensors = []
+    for f in open_model_files(d):
+        for n in f.names():
+            t = f.read(n)
+            tensors.append((n, t * gain if t.dim() == 2 and n not in ("emb", "head") else t))
+        f.close()
+    write_safetensors(os.path.join(d, "model.safetensors"), tensors, metadata={"format": "pt"})
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("step_rows", [0, 512])
+def test_a_window_model_goes_on_by_many_tokens(tmp_path, dtype, step_rows):
+    """Attention with a window keeps a ring of pages.  A step stores all its keys before its rows
+    read, so a sequence that goes on by more tokens than the ring holds beyond the window would
+    write over keys that the step's first rows still see: the step function runs such a step in
+    pieces (`step_rows=0`: a ring with 64 to 127 rows to spare), or the ring is made longer
+    (`step_rows=512`).  Either way a prompt cut into steps of any lengths, a session's turns and
+    `max_step_tokens` give what the whole prompt gives: layer 0 sees 70 keys, layer 1 all."""
+    import inferllm_amd as I
+    from tiny import random_ids, read_weights
+    E, V, nh, nkv, hd, F, eps, theta, win = 64, 120, 4, 2, 16, 100, 1e-5, 10000.0, 70
+    name = f"ToyWindowForTests_{dtype}_{step_rows}"
+    Cfg, plain = _windowed_architecture(name, E, V, nh, nkv, hd, F, eps, theta, [win, None])
+    d = I.write_random_model(str(tmp_path / "win"), Cfg(), seed=21)
+    _scaled(d, 5.0)
+    w = read_weights(d)
+    if dtype == "bfloat16":
+        w = {n: (t.to(torch.bfloat16) if t.dim() == 2 else t) for n, t in w.items()}
+    tol = TOL[torch.float32 if dtype == "float32" else torch.bfloat16]
+    eng = I.Engine.from_pretrained(d, dtype=dtype, max_batch=3, max_seq_len=1024, step_rows=step_rows,
+                                   poison_freed=True)
+    ring = next(g for g in eng.cache.groups if g.ring)
+    assert ring.spec.window == win and eng.model.one_token_mixers == []
+    limit = eng.cache.step_limit
+    assert (64 <= limit <= 127) if step_rows == 0 else limit >= 512
+    ids = random_ids(600, V, 5)
+    want = plain(w, ids)
+    # whole, then cut into steps: the second and third are longer than the spare rows of a short
+    # ring, the fourth crosses from one piece into the next with wanted places in both
+    s = eng.alloc_slot()
+    got = eng.step([I.StepEntry(s, ids, list(range(len(ids))))])
+    assert rel(got, want) < tol
+    eng.free_slot(s)
+    s, t = eng.alloc_slot(), eng.alloc_slot()
+    other = random_ids(150, V, 9)
+    want_other = plain(w, other)
+    at = 0
+    for n, picks in ((40, [39]), (200, [0, 199, 100]), (300, [299, 3]), (59, list(range(59))), (1, [0])):
+        entries = [I.StepEntry(s, ids[at:at + n], picks)]
+        if at == 40:
+            entries.append(I.StepEntry(t, other, [149, 0]))        # a sequence that starts beside it
+        out = eng.step(entries)
+        for j, p in enumerate(picks):
+            assert rel(out[j], want[at + p]) < tol, (at, p)
+        if at == 40:
+            assert rel(out[len(picks)], want_other[149]) < tol and rel(out[len(picks) + 1], want_other[0]) < tol
+        at += n
+    assert at == 600 and eng.cache.length(s) == 600
+    eng.free_slot(s)
+    eng.free_slot(t)
+    eng.cache.check()
+    if dtype != "float32":
+        return
+    # the generation loop feeds prompts in steps of 90 tokens, and a conversation goes on turn
+    # after turn, with a stop token whose void step is taken back from the ring
+    prompts = [ids[:230], other[:100], ids[300:420]]
+    greedy = lambda p, n: [int(x) for x in _greedy(plain, w, p, n)]
+    assert eng.generate(prompts, max_new_tokens=4, stop_token_ids=[], max_step_tokens=90) == \
+        [greedy(p, 4) for p in prompts]
+    first = greedy(ids[:150], 6)
+    j = next(j for j in range(1, 6) if first[j] not in first[:j])
+    with eng.session(stop_token_ids=[first[j]]) as talk:
+        assert talk.say(ids[:150], max_new_tokens=6) == first[:j]
+        assert talk.length == 150 + j                      # the stop token's void step was taken back
+        said = list(ids[:150]) + first[:j] + list(other[:130])
+        want2 = greedy(said, 3)
+        if first[j] in want2:
+            want2 = want2[:want2.index(first[j])]
+        assert talk.say(other[:130], max_new_tokens=3) == want2
+    eng.cache.check()
+    assert eng.cache.slots.n_held() == 0
+
+
+def _greedy(plain, w, prompt, n):
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(int(torch.argmax(plain(w, seq)[-1])))
+    return seq[len(prompt):]
+
+
+def test_a_toy_mixer_keeps_one_latent_row_per_token(tmp_path):
+    """What a cache line keeps per token is the mixer's to say: this one keeps a single row of 12
+    numbers in float32 (in a bfloat16 engine too) instead of keys and values, in the same paged
+    storage with the same slots, page tables and lengths; its output is a projection of the mean
+    of the rows kept so far.  Registered, built and stepped without a change to the library."""
+    import inferllm_amd as I
+    from inferllm_amd.cache import KVSpec, TokenTensor
+    from inferllm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from inferllm_amd.parts import Mixer, register_part
+    from inferllm_amd.weights import TensorWant
+    from tiny import random_ids, read_weights
+    E, R, V, eps = 40, 12, 90, 1e-5
+
+    @register_part("mixer", "toy_latent_rows")
+    class LatentRows(Mixer):
+        graph_safe = False                    # reads the step's lengths on the host
+        takes_continuations = True
+
+        def __init__(self, hidden_size, rank, tensors=None):
+            super().__init__(tensors)
+            self.E, self.R = hidden_size, rank
+
+        def shapes(self):
+            return {"down": TensorWant((self.R, self.E)), "up": TensorWant((self.E, self.R))}
+
+        def kv_spec(self):
+            return KVSpec("full", (TokenTensor("latent", (self.R,), torch.float32),))
+
+        def load(self, tensors):
+            self.down, self.up = self._take(tensors, "down").float(), self._take(tensors, "up").float()
+
+        def forward(self, h, ctx, line, writes_cache, position):
+            kept, group = ctx.cache.token_line(line)
+            rows = kept["latent"]                             # [page, row in page, R]
+            c = h.float() @ self.down.t()
+            pos, slot = ctx.row_pos.long(), ctx.row_slot.long()
+            page = group.table[slot, pos // group.page_size].long()
+            if writes_cache:
+                rows[page, pos % group.page_size] = c
+            out = torch.empty((h.shape[0], self.R), dtype=torch.float32, device=h.device)
+            for r, (p, s) in enumerate(zip(pos.tolist(), slot.tolist())):
+                js = torch.arange(p + 1, device=h.device)
+                pages = group.table[s, js // group.page_size].long()
+                out[r] = rows[pages, js % group.page_size].mean(dim=0)
+            return (out @ self.up.t()).to(h.dtype)
+
+    @register_architecture("ToyLatentForTests")
+    class Cfg:
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return {"architectures": ["ToyLatentForTests"]}
+
+        def to_spec(self):
+            norm = lambda n: PartSpec("rms_norm", {"size": E, "eps": eps}, {"weight": n})
+            layers = [LayerSpec("pre_norm", PartSpec("toy_latent_rows", {"hidden_size": E, "rank": R},
+                                                     {"down": f"l{i}.dn", "up": f"l{i}.up"}),
+                                PartSpec("swiglu", {"hidden_size": E, "intermediate_size": 64},
+                                         {"gate": f"l{i}.g", "up": f"l{i}.u", "down": f"l{i}.d"}),
+                                norm(f"l{i}.n1"), norm(f"l{i}.n2"), None) for i in range(2)]
+            return ModelSpec("ToyLatentForTests", V, E, 512,
+                             PartSpec("token_embedding", {"vocab_size": V, "hidden_size": E}, {"weight": "emb"}),
+                             layers, [ScheduleEntry(0, 0), ScheduleEntry(1, 1)], norm("nf"),
+                             PartSpec("lm_head", {"hidden_size": E, "vocab_size": V}, {"weight": "head"}))
+
+    def plain(w, ids):
+        x = P.embedding(w["emb"], ids)
+        for i in range(2):
+            c = P.linear(P.rms_norm(x, w[f"l{i}.n1"], eps), w[f"l{i}.dn"])
+            mean = torch.cumsum(c, 0) / torch.arange(1, len(ids) + 1, dtype=torch.float64)[:, None]
+            x = x + P.linear(mean, w[f"l{i}.up"])
+            x = x + P.swiglu_ffn(P.rms_norm(x, w[f"l{i}.n2"], eps), w[f"l{i}.g"], w[f"l{i}.u"], w[f"l{i}.d"])
+        return P.linear(P.rms_norm(x, w["nf"], eps), w["head"])
+
+    d = I.write_random_model(str(tmp_path / "latent"), Cfg(), seed=3)
+    w = read_weights(d)
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 3e-2)):
+        wd = w if dtype == "float32" else {n: (t.to(torch.bfloat16) if t.dim() == 2 else t) for n, t in w.items()}
+        eng = I.Engine.from_pretrained(d, dtype=dtype, max_batch=2, max_seq_len=256, poison_freed=True)
+        (group,) = eng.cache.groups
+        assert set(group.tensors) == {"latent"} and group.tensors["latent"].dtype == torch.float32
+        assert group.tensors["latent"].shape[2:] == (64, R)
+        reqs = [random_ids(n, V, n) for n in (90, 7, 70)]
+        want = [plain(wd, r) for r in reqs]
+        for order in ([0, 1], [2, 1]):                       # slots and pages are used again
+            slots = {i: eng.alloc_slot() for i in order}
+            head = {i: len(reqs[i]) - 3 for i in order}
+            out = eng.step([I.StepEntry(slots[i], reqs[i][:head[i]], [head[i] - 1]) for i in order])
+            for j, i in enumerate(order):
+                assert rel(out[j], want[i][head[i] - 1]) < tol
+            for t in range(3):
+                out = eng.step([I.StepEntry(slots[i], [reqs[i][head[i] + t]], [0]) for i in order])
+                for j, i in enumerate(order):
+                    assert rel(out[j], want[i][head[i] + t]) < tol
+            for i in order:
+                eng.free_slot(slots[i])
+            eng.cache.check()
+        # it says it goes on by several tokens: a prompt in two steps, and generation
+        s = eng.alloc_slot()
+        eng.step([I.StepEntry(s, reqs[0][:50], [])])
+        out = eng.step([I.StepEntry(s, reqs[0][50:], [39])])
+        assert rel(out[0], want[0][89]) < tol
+        eng.free_slot(s)
+        if dtype == "float32":
+            assert eng.generate([reqs[1]], max_new_tokens=3, stop_token_ids=[]) == [_greedy(plain, w, reqs[1], 3)]

@@ -39,13 +39,14 @@ def _both(lib, B, nh, nkv, hd, lens, nsplit, waves, seed):
     assert rc == 0
     got = torch.zeros_like(want)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(DEV)
+    # free memory as the driver counts it: torch's own counters would not see a hipMalloc
+    before = torch.cuda.mem_get_info(DEV)[0]
     rc = lib.illm_attn_decode_bf16_static(p(qkv), p(got), p(kc), p(vc), p(pt), pt.shape[1], PAGE, 0,
                                           p(slots), p(seq_len), nsplit, waves, B, nh, nkv, hd,
                                           scale, 0, stream)
     assert rc == 0
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated(DEV) == before
+    assert torch.cuda.mem_get_info(DEV)[0] == before
     assert torch.isfinite(got.float()).all()
     assert torch.equal(got, want), (B, nh, nkv, hd, nsplit)
     return got
@@ -63,6 +64,32 @@ def test_two_calls_in_a_row_share_the_scratch_array():
     _both(lib, 3, 32, 8, 128, [650, 90, 3000], 4, 4, seed=1)
     # a single range per sequence uses no scratch at all
     _both(lib, 2, 8, 2, 32, [100, 63], 1, 1, seed=4)
+
+
+def test_the_entry_point_can_be_captured_into_a_graph():
+    """An allocation (or any other call that a capture forbids) inside the entry point would end
+    the capture with an error; the replays, with eager work between them, must give what the
+    eager call gave."""
+    from inferllm_amd.kernels import build
+    lib = build.library()
+    B, nh, nkv, hd, nsplit, waves = 2, 16, 4, 128, 4, 4
+    want = _both(lib, B, nh, nkv, hd, [900, 130], nsplit, waves, seed=6)   # the device's first call is eager
+    qkv, kc, vc, pt, slots, seq_len = _case(B, nh, nkv, hd, [900, 130], seed=6)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    got = torch.zeros_like(want)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.illm_attn_decode_bf16_static(
+            p(qkv), p(got), p(kc), p(vc), p(pt), pt.shape[1], PAGE, 0, p(slots), p(seq_len), nsplit,
+            waves, B, nh, nkv, hd, ctypes.c_float(1.0 / math.sqrt(hd)), 0,
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    for _ in range(3):
+        got.fill_(0)
+        _both(lib, 1, 4, 4, 64, [200], 2, 2, seed=2)        # eager work that uses the array between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
 
 
 def test_what_does_not_fit_the_array_is_refused():
