@@ -89,8 +89,76 @@ class _DecodeGraph:
             max_len=self.max_len, cache=runner.cache)
 
 
+PROMPT_GRAPH_ROWS = (16, 32, 64, 96, 128, 192, 256)   # rows of the graphs that short prompt steps are replayed from
+PROMPT_GRAPH_SEQS = (2, 4, 8, 16, 32)                 # and their sequences (one of them takes the padding rows)
+
+
+class _PromptGraph:
+    """Static buffers and the captured graph for steps of several tokens a sequence with at most
+    `rows` rows in at most `seqs` - 1 sequences, of which at most 2 `seqs` rows are wanted.  Rows
+    that only fill the graph up are a sequence of their own on the cache's spare slot; sequences
+    that only fill it up have no rows."""
+
+    def __init__(self, runner: "StepRunner", rows: int, seqs: int, continues: bool):
+        self.rows, self.seqs, self.continues = rows, seqs, continues
+        dev = runner.device
+        # tokens | pos | slot (rows each) | cu (seqs + 1) | seq slot | seq len | seq start (seqs each) | wanted
+        self.sizes = (rows, rows, rows, seqs + 1, seqs, seqs, seqs, 2 * seqs)
+        n = sum(self.sizes)
+        self.meta = torch.zeros(n, dtype=torch.int32, device=dev)
+        self.stage = torch.zeros(n, dtype=torch.int32, pin_memory=True)
+        self.stage_np = self.stage.numpy()
+        self.copied = torch.cuda.Event()
+        self.in_flight = False
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+
+    def parts(self) -> List[torch.Tensor]:
+        out, o = [], 0
+        for n in self.sizes:
+            out.append(self.meta[o:o + n])
+            o += n
+        return out
+
+    def context(self, runner: "StepRunner") -> StepContext:
+        p = self.parts()
+        limit = runner.cache.max_seq_len
+        return StepContext(
+            device=runner.device, act_dtype=runner.act_dtype, prefill=True, n_rows=self.rows,
+            n_seqs=self.seqs, tokens=p[0], row_pos=p[1], row_slot=p[2], cu_seqlens=p[3], seq_slot=p[4],
+            seq_len=p[5], max_len=limit if self.continues else self.rows, cache=runner.cache,
+            seq_start=p[6], max_rows=self.rows, continues=self.continues)
+
+    def fill(self, runner: "StepRunner", entries: Sequence[StepEntry], starts: Sequence[int]) -> int:
+        """Write the step's numbers into the pinned stage; returns the number of wanted rows."""
+        spare = runner.cache.spare_slot
+        wrap = max(1, min(64, runner.cache.max_seq_len))       # positions of the padding rows
+        tokens: List[int] = []
+        pos: List[int] = []
+        slot: List[int] = []
+        cu = [0]
+        want: List[int] = []
+        for e, start in zip(entries, starts):
+            n = len(e.tokens)
+            want.extend(cu[-1] + int(w) for w in e.want)
+            tokens.extend(int(t) for t in e.tokens)
+            pos.extend(range(start, start + n))
+            slot.extend([e.slot] * n)
+            cu.append(cu[-1] + n)
+        pad = self.rows - len(tokens)
+        idle = self.seqs - len(entries)                         # >= 1: the first takes the padding rows
+        host = (tokens + [0] * pad + pos + [i % wrap for i in range(pad)] + slot + [spare] * pad
+                + cu + [self.rows] * idle
+                + [e.slot for e in entries] + [spare] * idle
+                + [s + len(e.tokens) for e, s in zip(entries, starts)] + [max(pad, 1)] + [1] * (idle - 1)
+                + [int(s) for s in starts] + [0] * idle
+                + want + [0] * (2 * self.seqs - len(want)))
+        self.stage_np[:] = host
+        return len(want)
+
+
 class StepRunner:
-    """Owns the model, the cache and the decode graphs; `step` is the one entry."""
+    """Owns the model, the cache and the step graphs; `step` is the one entry."""
 
     def __init__(self, model: DecoderModel, cache: CacheManager, act_dtype: torch.dtype,
                  device: torch.device, use_graphs: bool = True, plan=None):
@@ -101,6 +169,11 @@ class StepRunner:
         self.use_graphs = (use_graphs and model.graph_safe
                            and os.environ.get("INFERLLM_NO_GRAPH", "0") != "1")
         self._graphs: Dict[tuple, _DecodeGraph] = {}
+        # steps of few rows with several tokens a sequence (short prompts, a conversation's turns):
+        # replayed from a graph from the second step of a shape on (the first runs eagerly: one
+        # prompt does not pay for a capture)
+        self._prompt_graphs: Dict[tuple, _PromptGraph] = {}
+        self._prompt_uses: Dict[tuple, int] = {}
 
     # ------------------------------------------------------------ checks
     def _phase(self, entries: Sequence[StepEntry]) -> bool:
@@ -164,8 +237,65 @@ class StepRunner:
         self.cache.extend_all([(e.slot, s, len(e.tokens)) for e, s in zip(entries, starts)])
         self.cache.upload(lengths=prefill)
         if prefill:
+            g = self._prompt_graph_for(entries, starts)
+            if g is not None:
+                return self._replay_prompt(g, entries, starts, borrow)
             return self._prefill(entries, starts)
         return self._decode(entries, starts, device_tokens, borrow)
+
+    def _prompt_graph_for(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> Optional[_PromptGraph]:
+        """The graph that this step of several tokens a sequence is replayed from, or None if it
+        runs eagerly: more rows, sequences or wanted rows than the graphs hold, or a shape seen
+        for the first time."""
+        if not self.use_graphs:
+            return None
+        rows = sum(len(e.tokens) for e in entries)
+        wanted = sum(len(e.want) for e in entries)
+        if rows > PROMPT_GRAPH_ROWS[-1] or len(entries) + 1 > PROMPT_GRAPH_SEQS[-1] or wanted == 0:
+            return None
+        if next(b for b in PROMPT_GRAPH_ROWS if b >= rows) > self.cache.max_seq_len:
+            return None         # the padding rows are a sequence too, and no sequence is that long here
+        seqs = next(b for b in PROMPT_GRAPH_SEQS if b >= len(entries) + 1)
+        if wanted > 2 * seqs:
+            return None
+        key = (next(b for b in PROMPT_GRAPH_ROWS if b >= rows), seqs, any(int(s) > 0 for s in starts))
+        self._prompt_uses[key] = self._prompt_uses.get(key, 0) + 1
+        g = self._prompt_graphs.get(key)
+        if g is None:
+            if self._prompt_uses[key] < 2:
+                return None
+            g = self._prompt_graphs[key] = _PromptGraph(self, *key)
+        return g
+
+    def _replay_prompt(self, g: _PromptGraph, entries: Sequence[StepEntry], starts: Sequence[int],
+                       borrow: bool) -> torch.Tensor:
+        if g.graph is None:
+            self._capture_prompt(g)
+        if g.in_flight:
+            g.copied.synchronize()          # the last step's copy has left the pinned buffer
+        wanted = g.fill(self, entries, starts)
+        g.meta.copy_(g.stage, non_blocking=True)
+        g.copied.record()
+        g.in_flight = True
+        g.graph.replay()
+        return g.logits[:wanted] if borrow else g.logits[:wanted].clone()
+
+    def _capture_prompt(self, g: _PromptGraph) -> None:
+        """As `_capture`: one eager run of the same shapes with every row on the spare slot (one
+        sequence of padding rows, the other sequences empty), then the capture."""
+        g.fill(self, [], [])
+        g.meta.copy_(g.stage)
+        rows = g.parts()[7]
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            self.model.forward(g.context(self), rows)
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            g.logits = self.model.forward(g.context(self), rows)
+        g.graph = graph
 
     def _in_pieces(self, entries: Sequence[StepEntry], starts: Sequence[int],
                    limit: int) -> Optional[torch.Tensor]:

@@ -142,7 +142,8 @@ def test_few_rows_through_the_planes_where_they_pay(tmp_path_factory, monkeypatc
     and 9 tokens and six sequences decoding together must come out as the plain model's in each."""
     from inferllm_amd import StepEntry
     from inferllm_amd.kernels import ops
-    eng, plain, config = setup(tmp_path_factory, "B", "bfloat16", max_batch=8, decode_copies=True)
+    # (without graphs: a graph's step has its bucket's rows, and the way is chosen by the rows)
+    eng, plain, config = setup(tmp_path_factory, "B", "bfloat16", max_batch=8, decode_copies=True, use_graphs=False)
     shape = (config["hidden_size"], config["intermediate_size"])
     eng.plan.planes_from[shape] = first
     calls = []
@@ -987,3 +988,53 @@ def test_bfloat16_error_grows_with_the_square_root_of_depth(tmp_path_factory, la
     assert float(per_pos.max()) < depth_budget(layers), per_pos.tolist()
     # and the budget is no empty promise: the error is of the budget's order, not far below it
     assert float(per_pos.max()) > depth_budget(layers) / 30
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_short_prompt_steps_are_replayed_from_graphs(tmp_path_factory, name, dtype):
+    """Steps of several tokens a sequence with few rows (short prompts, a conversation's turns)
+    run eagerly the first time a shape comes and from a HIP graph from the second time on: rows
+    that only fill the graph up are a sequence of their own on the spare slot, sequences that
+    only fill it up are empty.  Whole prompts, ragged batches, steps that go on from the cache,
+    wanted rows anywhere; and the cache they leave serves the decode steps that follow."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, name, dtype, max_batch=6)
+    assert eng.runner.use_graphs
+    budget = BUDGET[dtype]
+    for round_ in range(3):                                  # eager, capture + replay, replay
+        for batch in ([9], [3, 30, 1], [40, 41, 17, 70, 2]):
+            reqs = requests_for(config, [n + 4 for n in batch], seed=50 + 7 * round_ + len(batch))
+            slots = [eng.alloc_slot() for _ in reqs]
+            want = [plain(r) for r in reqs]
+            # the prompts but their last four tokens, logits wanted at the first and the last row
+            out = eng.step([StepEntry(s, r[:n], [0, n - 1] if n > 1 else [0]) for s, r, n in zip(slots, reqs, batch)])
+            at = 0
+            for i, n in enumerate(batch):
+                for p_ in ([0, n - 1] if n > 1 else [0]):
+                    assert err(out[at], want[i][p_]) < budget, (round_, batch, i, p_)
+                    at += 1
+            assert at == out.shape[0]
+            # two more tokens in a step that goes on from the cache (rows over the paged cache)
+            out = eng.step([StepEntry(s, r[n:n + 2], [1]) for s, r, n in zip(slots, reqs, batch)])
+            for i, n in enumerate(batch):
+                assert err(out[i], want[i][n + 1]) < budget, (round_, batch, i)
+            # and single tokens: the cache holds what the graphs' steps stored
+            for t in (2, 3):
+                out = eng.step([StepEntry(s, [r[n + t]], [0]) for s, r, n in zip(slots, reqs, batch)])
+                for i, n in enumerate(batch):
+                    assert err(out[i], want[i][n + t]) < budget, (round_, batch, i, t)
+            for s in slots:
+                eng.free_slot(s)
+            eng.cache.check()
+    keys = set(eng.runner._prompt_graphs)
+    # (rows, sequences, goes on): 9 and 2 rows in 16, 34 and 6 in 64 and 16, 170 and 10 in 192 and 16
+    assert keys == {(16, 2, False), (16, 2, True), (64, 4, False), (16, 4, True), (192, 8, False), (16, 8, True)}
+    assert all(g.graph is not None for g in eng.runner._prompt_graphs.values())
+    # more rows or more wanted rows than a graph holds, and a step that wants nothing: eagerly
+    s = eng.alloc_slot()
+    ids = requests_for(config, [60], seed=77)[0]
+    before = dict(eng.runner._prompt_uses)
+    out = eng.step([StepEntry(s, ids, list(range(60)))])
+    assert err(out, plain(ids)) < budget and eng.runner._prompt_uses == before
+    eng.free_slot(s)
