@@ -7,12 +7,15 @@ Default: the LLaMA-2-7B layer sizes (32 layers, hidden 4096, 32/32 heads of 128,
 feed-forward 11008, vocabulary 32000) with seeded random bfloat16 weights, a batch
 of 8 sequences with 512-token prompts that decode 256 tokens (8 more to warm up),
 cache context 4096.  A step is one decode step of the whole batch: step function, greedy choice on the device, the tokens
-back on the host.  One JSON line is printed: decoded tokens per second, the
+back on the host, as `Engine.generate` runs it.  One JSON line is printed: decoded tokens per second, the
 prefill of 2,048 tokens, the decode step against the HBM roofline, and under
 `points` decoding at batch 1 and 64, decoding from 3,800-token contexts at batch
-8 and 64, and the LLaMA-3-8B shape with 16 prompts of 64 to 4,096 tokens through the
-generation loop (`--with-70b` adds the LLaMA-2-70B shape: prefill of 2,048 tokens,
-decode at batch 1 and 32 from 1,024-token prompts).  Every decode point has a
+8 and 64, milliseconds to the first token of prompts of 16, 64 and 160 tokens, prefills of
+64 x 128, 8,192 and 16,384 tokens (and of 16,384 in steps of 2,048 that go on from the paged
+cache), the LLaMA-3-8B shape with 16 prompts of 64 to 4,096 tokens and with 8 sequences at
+8,000-token contexts, and the LLaMA-2-70B shape (prefill of 2,048 tokens, decode at batch 1 and
+32 from 1,024-token prompts; `--no-70b` leaves it out).  Every decode run goes through the
+engine's generation loop, whose stopwatch starts after the warm-up steps.  Every decode point has a
 `..._hbm_frac` beside it: the bytes its step has to read (every weight once, the
 cache of its live sequences) / its time / the HBM peak.  Peaks are the published ones
 of MI355X (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, float32 157.3 TFLOP/s).
@@ -103,90 +106,73 @@ class Bench:
 
     def decode_run(self, batch, steps, warmup, prompt):
         """(tokens/s, ms/step, fraction of the HBM peak) of `steps` timed decode steps of `batch`
-        sequences that start from prompts of `prompt` tokens."""
-        from inferllm_amd import StepEntry
-        from inferllm_amd.kernels import ops
+        sequences that start from prompts of `prompt` tokens, through the engine's generation
+        loop (greedy, no stop token): the loop runs `warmup` decode steps, waits for the device,
+        and its stopwatch runs from there to the end of the batch."""
         from inferllm_amd.sampling import Sampler, SamplingParams
         torch, eng = self.torch, self.eng
         prompts = [self.ids(prompt) for _ in range(batch)]
-        slots = [eng.alloc_slot() for _ in range(batch)]
-        # prompts go in pieces of at most 16,384 tokens to bound the prefill's activations
-        per = max(1, 16384 // prompt)
-        toks = [0] * batch
-        for i in range(0, batch, per):
-            part = list(range(i, min(batch, i + per)))
-            logits = eng.step([StepEntry(slots[j], prompts[j], [prompt - 1]) for j in part])
-            for j, t in zip(part, ops.argmax(logits.contiguous()).tolist()):
-                toks[j] = t
-
-        # as the generation loop runs greedy requests: a step starts from the tokens the last
-        # one chose on the device, and the host reads every step's tokens while the next runs
-        sampler = Sampler(SamplingParams(), eng.device)             # greedy
-        draw = sampler.draw(eng.step([StepEntry(s, [t], [0]) for s, t in zip(slots, toks)]),
-                            [0] * batch, [0] * batch)
-        seen = []
-
-        def one():
-            nonlocal draw
-            logits = eng.step([StepEntry(s, [0], [0]) for s in slots], device_tokens=draw.device)
-            following = sampler.draw(logits, [0] * batch, [0] * batch)
-            seen.append(draw.tokens())
-            draw = following
-            return logits
-
-        for _ in range(warmup):
-            one()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(steps):
-            logits = one()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t
-        # what was timed must have computed something: finite logits, and greedy tokens that
-        # are not one and the same everywhere (a run on NaN or constant logits would be as fast)
-        if not bool(torch.isfinite(logits).all()):
-            raise SystemExit(f"bench: non-finite logits in the decode run at batch {batch}")
-        distinct = {int(t) for row in seen for t in row}
+        params = SamplingParams()                                   # greedy
+        # (prompts go in steps of at most 16,384 tokens to bound the prefill's activations)
+        loop = eng.generation_loop(Sampler(params, eng.device), max_step_tokens=16384)
+        loop.time_after = warmup
+        out = loop.run(prompts, params, warmup + steps + 1, [])
+        st = loop.stats
+        if st.timed_steps != steps or st.batches != 1 or any(len(o) != warmup + steps + 1 for o in out):
+            raise SystemExit(f"bench: the loop timed {st.timed_steps} steps of {st.batches} batches at "
+                             f"batch {batch}, not {steps} of one")
+        dt = st.timed_seconds
+        # what was timed must have computed something: greedy tokens that are not one and the same
+        # everywhere (a run on NaN or constant logits would be as fast)
+        distinct = {int(t) for o in out for t in o}
         print(f"[bench] batch {batch}, prompts of {prompt}: {dt / steps * 1e3:.3f} ms a step, "
-              f"{len(distinct)} distinct greedy tokens in {len(seen)} steps", file=sys.stderr, flush=True)
-        if len(seen) >= 16 and len(distinct) < 2:
+              f"{len(distinct)} distinct greedy tokens in {steps + warmup} steps", file=sys.stderr, flush=True)
+        if steps + warmup >= 16 and len(distinct) < 2:
             raise SystemExit(f"bench: the greedy token is {sorted(distinct)} in every step of every "
                              f"sequence at batch {batch}: the logits are degenerate")
         mean_ctx = prompt + 1 + warmup + (steps + 1) / 2.0
-        for s in slots:
-            eng.free_slot(s)
         ms = dt / steps * 1e3
         frac = self.step_bytes(batch, mean_ctx) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
         return batch * steps / dt, ms, frac
 
-    def prefill_run(self, T=2048, reps=6):
+    def prefill_run(self, T=2048, reps=6, prompts=1, max_step_tokens=None, skip=1):
+        """`prompts` prompts of T tokens each in one step (or, with `max_step_tokens`, one prompt in
+        steps of that many tokens that go on from the cache): tokens/s of the fastest of `reps` runs
+        after the first `skip`, the time to the first token in ms, and the fraction of the matrix peak."""
         from inferllm_amd import StepEntry
         from inferllm_amd.kernels import ops
         torch, eng = self.torch, self.eng
-        ids = self.ids(T)
+        ids = [self.ids(T) for _ in range(prompts)]
         times = []
         for i in range(reps):
-            s = eng.alloc_slot()
+            slots = [eng.alloc_slot() for _ in ids]
             torch.cuda.synchronize()
             t = time.perf_counter()
-            logits = eng.step([StepEntry(s, ids, [T - 1])])
+            if max_step_tokens is None:
+                logits = eng.step([StepEntry(s, p, [T - 1]) for s, p in zip(slots, ids)])
+            else:
+                for a in range(0, T, max_step_tokens):
+                    piece = ids[0][a:a + max_step_tokens]
+                    logits = eng.step([StepEntry(slots[0], piece, [len(piece) - 1] if a + len(piece) == T else [])])
             ops.argmax(logits).tolist()
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t)
             if not bool(torch.isfinite(logits).all()):
                 raise SystemExit("bench: non-finite logits in the prefill")
-            eng.free_slot(s)
-        pt = min(times[1:])
-        fl = prefill_flops(self.cfg, self.layers, T)
-        return {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+            for s in slots:
+                eng.free_slot(s)
+        pt = min(times[skip:])
+        fl = prefill_flops(self.cfg, self.layers, T * prompts, prompts, [T] * prompts)
+        return {"value": round(T * prompts / pt, 1), "tokens": T * prompts, "ms": round(pt * 1e3, 3),
                 "frac": round(fl / pt / (PEAK_TFLOPS[self.dkey] * 1e12), 4)}
 
     def generate_run(self, lens, new_tokens):
-        """Prompts of the given lengths through `Engine.generate` (all in one batch), twice; the
-        second run's figures: (prefill tokens/s, its fraction of the matrix peak, decode tokens/s,
-        its fraction of the HBM peak)."""
+        """Prompts of the given lengths through `Engine.generate` (all in one batch), three times
+        (the first sets libraries and graphs up, the second may still take fresh memory from the
+        driver for what the graphs' pools cannot lend it); the third run's figures: (prefill
+        tokens/s, its fraction of the matrix peak, decode tokens/s, its fraction of the HBM peak)."""
         prompts = [self.ids(n) for n in lens]
-        for _ in range(2):
+        for _ in range(3):
             out = self.eng.generate(prompts, max_new_tokens=new_tokens, stop_token_ids=[])
             st = self.eng.last_stats
         assert all(len(o) == new_tokens for o in out)
@@ -217,8 +203,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip everything under `points` and the prefill")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiles); prints its own line")
-    ap.add_argument("--with-70b", action="store_true",
-                    help="add the LLaMA-2-70B shape to `points` (138 GB of weights: minutes)")
+    ap.add_argument("--no-70b", action="store_true",
+                    help="leave the LLaMA-2-70B shape out of `points` (138 GB of weights: half a minute)")
+    ap.add_argument("--with-70b", action="store_true", help="(the default now; kept for old command lines)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only (this library has no multi-GPU path); --gpus must be 1")
@@ -272,12 +259,28 @@ def main() -> int:
             for name, batch in (("decode_b8_ctx3800", 8), ("decode_b64_ctx3800", 64)):
                 v, _, f = b.decode_run(batch, 64, 4, long_ctx)
                 points[name], points[name + "_hbm_frac"] = round(v, 2), round(f, 4)
+            # short prompts: milliseconds to the first token (their steps are replayed from graphs
+            # from the second of a shape on), and 64 prompts of 128 tokens in one step
+            for n in (16, 64, 160):
+                points[f"first_token_ms_prompt{n}"] = b.prefill_run(n, reps=8, skip=3)["ms"]
+            p = b.prefill_run(128, prompts=64)
+            points["prefill_64x128"], points["prefill_64x128_frac"] = p["value"], p["frac"]
             b.close()
+            # the same layer sizes with room for 16,384 positions: one long prompt whole, and in
+            # steps of 2,048 tokens that go on from the paged cache
+            long = Bench(dict(LLAMA2_7B, max_position_embeddings=16384), args.layers, args.dtype, 1, 16384 + 64)
+            for T in (8192, 16384):
+                p = long.prefill_run(T, reps=3)
+                points[f"prefill_{T}"], points[f"prefill_{T}_frac"] = p["value"], p["frac"]
+            p = long.prefill_run(16384, reps=3, max_step_tokens=2048)
+            points["prefill_16384_in_steps_of_2048"], points["prefill_16384_in_steps_of_2048_frac"] = p["value"], p["frac"]
+            long.close()
             # LLaMA-3-8B shape (grouped heads, vocabulary 128,256): 16 prompts of 64 to 4,096
-            # tokens, lengths seeded, one batch through the generation loop, 128 new tokens each
+            # tokens, lengths seeded, one batch through the generation loop, 128 new tokens each;
+            # and 8 sequences decoding from 8,000-token contexts (its context is 8,192)
             import torch
             lens = torch.randint(64, 4097, (16,), generator=torch.Generator().manual_seed(16)).tolist()
-            total = sum(-(-(n + 130) // 64) * 64 for n in lens)
+            total = max(sum(-(-(n + 130) // 64) * 64 for n in lens), 8 * 8192)
             b8 = Bench(LLAMA3_8B, 0, args.dtype, 16, total)
             pf, pf_frac, dc, dc_frac = b8.generate_run(lens, 128)
             points.update({"llama3_8b_ragged16_prompt_tokens": sum(lens),
@@ -285,8 +288,10 @@ def main() -> int:
                            "llama3_8b_ragged16_prefill_frac": round(pf_frac, 4),
                            "llama3_8b_ragged16_decode": round(dc, 2),
                            "llama3_8b_ragged16_decode_hbm_frac": round(dc_frac, 4)})
+            v, _, f = b8.decode_run(8, 64, 4, 8000)
+            points["llama3_8b_decode_b8_ctx8000"], points["llama3_8b_decode_b8_ctx8000_hbm_frac"] = round(v, 2), round(f, 4)
             b8.close()
-            if args.with_70b:
+            if not args.no_70b:
                 b70 = Bench(LLAMA2_70B, 0, args.dtype, 32, 32 * 1280)
                 p70 = b70.prefill_run()
                 points.update({"llama2_70b_prefill": p70["value"], "llama2_70b_prefill_frac": p70["frac"]})

@@ -49,6 +49,9 @@ class GenerationStats:
     decode_seconds: float = 0.0
     decode_steps: int = 0
     batches: int = 0
+    # a stopwatch over the last decode steps of a run, for measurements (`GenerationLoop.time_after`)
+    timed_seconds: float = 0.0
+    timed_steps: int = 0
 
     def summary(self) -> str:
         """Like the reference's decode_summary (src/core/model_imp.cpp:133-141), but the
@@ -143,6 +146,10 @@ class GenerationLoop:
         self.sync = sync or (lambda: None)
         self.on_token = on_token            # called with (request index, token) as tokens are kept
         self.stats = GenerationStats()
+        # measurements: after this many decode steps of a batch the loop waits for the device once
+        # and `stats.timed_seconds` / `timed_steps` count from there to the batch's end (None: off)
+        self.time_after: Optional[int] = None
+        self._mark: Optional[tuple] = None
 
     # ------------------------------------------------------------ decisions
     def room_needed(self, prompt_len: int, max_new_tokens: int) -> int:
@@ -280,6 +287,9 @@ class GenerationLoop:
         self.stats.prefill_seconds += time.perf_counter() - t0
         self.stats.prompt_tokens += sum(len(s.feed) for s in live)
         t0 = time.perf_counter()
+        self._mark = None
+        self._steps0 = self.stats.decode_steps
+        self._stopwatch()
         try:
             if self.draw is not None:
                 self._decode_ahead(live, first, max_new_tokens, stop_ids, include_stop)
@@ -287,7 +297,18 @@ class GenerationLoop:
                 self._decode(live, first, max_new_tokens, stop_ids, include_stop)
         finally:
             self.sync()
-            self.stats.decode_seconds += time.perf_counter() - t0
+            end = time.perf_counter()
+            self.stats.decode_seconds += end - t0
+            if self._mark is not None:
+                self.stats.timed_seconds += end - self._mark[0]
+                self.stats.timed_steps += self.stats.decode_steps - self._mark[1]
+
+    def _stopwatch(self) -> None:
+        """Start the stopwatch when the batch has run `time_after` decode steps."""
+        if (self.time_after is not None and self._mark is None
+                and self.stats.decode_steps - self._steps0 >= self.time_after):
+            self.sync()
+            self._mark = (time.perf_counter(), self.stats.decode_steps)
 
     def _read(self, s: _Live, tok: int, stop_ids, include_stop: bool, max_new_tokens: int) -> None:
         """A drawn token has reached the host: count it, keep it, decide whether its sequence ends."""
@@ -325,6 +346,7 @@ class GenerationLoop:
                                       [s.counter0 + s.drawn + 1 for s in cont],
                                       [s.history for s in cont], tokens)
                 self.stats.decode_steps += 1
+                self._stopwatch()
             for s, tok in zip(rows, pending.tokens()):
                 if s.dead:
                     continue             # it drew a stop token a step ago: this one is void
@@ -353,3 +375,4 @@ class GenerationLoop:
             tokens = self.sample(logits, [s.seed for s in live],
                                  [s.counter0 + s.drawn for s in live], [s.history for s in live])
             self.stats.decode_steps += 1
+            self._stopwatch()

@@ -33,7 +33,7 @@ from typing import Dict, Optional
 import torch
 
 from . import build
-from .plan import NEVER_BELOW, Plan
+from .plan import NEVER_BELOW, Plan, Rules
 
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
@@ -416,13 +416,8 @@ def linear_add(x: torch.Tensor, w, into: torch.Tensor, norm=None,
     return NormedRows(into, weight, eps, act_dtype, xb, ssq)
 
 
-MID_MAX_ROWS = 128       # rows a launch of the kernel takes (the vendor GEMM reads the thin matrices
-                         # at 1.6 TB/s at 128 rows: 58.6 us for the 7B down projection)
-MID_MAX_COLS = 8192      # measured at the 7B and 70B shapes: product and the norm that adds the
-                         # planes take 0.6 to 0.75 of the vendor GEMM's and the norm's time when
-                         # K >= 2 N (the down projection) and 0.8 to 0.95 when K = N
-PLANES_MIN_ELEMENTS = 1 << 22   # smaller matrices are not measured (both ways take a few
-                                # microseconds and the clock would decide): no planes below 17 rows
+MID_MAX_ROWS = 128       # rows a launch of csrc/gemm_mid.hip takes (a limit of the kernel; the break-even
+                         # points of the ways are the plan's: `kernels.plan.Rules` and its tables)
 
 # The tables that products with more than one way are dispatched by (`kernels.plan`).  An engine
 # makes its own current at the start of each of its steps; nothing is timed unless the plan asks.
@@ -445,7 +440,7 @@ def linear_planes_fits(x, w) -> bool:
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == "plain"
             and isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 and x.dim() == 2
             and 1 <= x.shape[0] <= MID_MAX_ROWS and x.shape[1] == w.plain.shape[1]
-            and w.plain.shape[0] % 4 == 0 and w.plain.shape[0] <= MID_MAX_COLS
+            and w.plain.shape[0] % 4 == 0 and w.plain.shape[0] <= _plan.rules.planes_most_cols
             and w.plain.shape[1] >= (2 if x.shape[0] <= SKINNY_BEST_ROWS else 1) * w.plain.shape[0])
 
 
@@ -486,7 +481,7 @@ def measure_planes_from(w: "Weight") -> int:
     """Fewest rows from which `linear_planes` and the norm that adds its planes take less time
     than `linear_add` (whose norm the next product takes), measured at 16, 12, 8 and 4 rows."""
     N, K = w.plain.shape
-    if N * K < PLANES_MIN_ELEMENTS:
+    if N * K < _plan.rules.planes_min_elements:
         return NEVER_BELOW
     dev = w.plain.device
     x = torch.zeros((SKINNY_BEST_ROWS, K), dtype=torch.bfloat16, device=dev)
@@ -517,7 +512,7 @@ def tune_product(plan: Plan, kind: str, w, votes: int = 1, **geometry) -> Option
     N, K = w.shape
     if kind == "plain":
         key, table = (N, K), plan.planes_from
-        fits = K >= 2 * N and N <= MID_MAX_COLS and N % 4 == 0
+        fits = K >= 2 * N and N <= plan.rules.planes_most_cols and N % 4 == 0
         measure = lambda: measure_planes_from(w)
     elif kind == "qkv":
         key, table = ("qkv", N, K), plan.rows_from
@@ -622,9 +617,7 @@ def linear(x, w, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
 # the output columns, each part written into its slice of one result, as the current plan's
 # table says (`kernels.plan`; a plan that measures times the candidates for a shape it lacks).
 # Every output element is still one kernel's sum; plans differ in rounding only.
-PLAN_MIN_ROWS = 1024          # below this no cut ever paid
-PLAN_MIN_COLS = 8192
-PAD_MIN_ROWS, PAD_ROWS = 64, 256     # rows between these may be filled up to PAD_ROWS
+# (from how many rows and columns a cut or a filling-up is a candidate: `kernels.plan.Rules`)
 
 
 def _split_candidates(N: int, M: int = 0):
@@ -682,7 +675,8 @@ def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     M, K = x.shape
     N = w.shape[0]
     capturing = torch.cuda.is_current_stream_capturing()
-    if PAD_MIN_ROWS < M < PAD_ROWS:
+    rules = _plan.rules
+    if rules.pad_rows_above < M < rules.pad_rows_to:
         # the vendor GEMM takes 65 to 255 rows of some shapes slower than 256 (measured: 4096 x
         # 11008 at 192 rows 82 us, at 256 rows 51): whole or filled up to 256, per shape and
         # 32 rows
@@ -691,9 +685,9 @@ def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         if plan is None:
             if not _plan.measure or capturing:
                 return torch.matmul(x, w.t())
-            plan = _plan.cuts[key] = measure_plan(x, w, [(), ("pad", PAD_ROWS)])
+            plan = _plan.cuts[key] = measure_plan(x, w, [(), ("pad", rules.pad_rows_to)])
         return _run_plan(x, w, plan)
-    if M < PLAN_MIN_ROWS or N < PLAN_MIN_COLS:
+    if M < rules.cut_min_rows or N < rules.cut_min_cols:
         return torch.matmul(x, w.t())
     key = (-(-M // 256), N, K)
     plan = _plan.cuts.get(key)
@@ -706,31 +700,31 @@ def _planned_matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return _run_plan(x, w, plan)
 
 
-ROWS_MAX = 128           # rows the products of csrc/gemm_rows.hip take, all in one launch
-ROWS_FUSED_MAX = 128     # and the fused q|k|v and gate|up products (measured against the vendor
-                         # GEMM with the elementwise kernel behind it, 80 / 96 / 128 rows: gate|up
-                         # of the 7B shape 39 / 40 / 44 against 50 / 50 / 49 us, of the 8B shape
-                         # 46 / 48 / 52 against 73 / 59 / 61; q|k|v 12288 x 4096 26 / 27 / 36
-                         # against 30 / 33 / 34 + 5; in two launches of 64 rows they lost)
-ROWS_QKV_SMALL_MAX = 96  # q|k|v matrices of fewer than 8192 rows: 6144 x 4096 takes 21 / 24 / 34
-                         # against 23 / 23 / 25 + 5
-ROWS_FROM = 17           # from this many rows they are taken unless the plan says otherwise for
-                         # the shape (up to 16 rows the few-rows kernels are the other way)
+ROWS_MAX = 128           # rows the products of csrc/gemm_rows.hip take, all in one launch (a limit of
+                         # the kernel; measured against the vendor GEMM with the elementwise kernel
+                         # behind it at 80 / 96 / 128 rows: gate|up of the 7B shape 39 / 40 / 44 against
+                         # 50 / 50 / 49 us, of the 8B shape 46 / 48 / 52 against 73 / 59 / 61; in two
+                         # launches of 64 rows they lost)
 
 
 def rows_from(mode: str, w) -> int:
     """Fewest rows from which the product with `w` in tile order `mode` goes to
-    csrc/gemm_rows.hip: the plan's entry for the shape, else ROWS_FROM."""
-    return _plan.rows_from.get((mode,) + tuple(w.shape), ROWS_FROM)
+    csrc/gemm_rows.hip: the plan's entry for the shape, else the plan's rule."""
+    return _plan.rows_from.get((mode,) + tuple(w.shape), _plan.rules.rows_from)
+
+
+def rows_most(mode: str, w) -> int:
+    """Most rows for which it does: the plan's entry for the shape, else all a launch takes."""
+    return min(ROWS_MAX, _plan.rows_most.get((mode,) + tuple(w.shape), ROWS_MAX))
 
 
 def rows_fits(x, w, mode: str) -> bool:
     """Whether the products of csrc/gemm_rows.hip take these operands: bfloat16 rows (or
     `NormedRows`, up to 16) and a weight with a decode copy in `mode`'s tile order."""
     xt = x.xb if isinstance(x, NormedRows) else x
-    most = 16 if isinstance(x, NormedRows) else (ROWS_MAX if mode == "plain" else ROWS_FUSED_MAX)
-    if mode == "qkv" and isinstance(w, Weight) and w.plain.shape[0] < 8192:
-        most = min(most, ROWS_QKV_SMALL_MAX)
+    if not (isinstance(w, Weight) and w.tiled is not None and w.mode == mode):
+        return False
+    most = 16 if isinstance(x, NormedRows) else rows_most(mode, w)
     return (isinstance(w, Weight) and w.tiled is not None and w.mode == mode
             and isinstance(xt, torch.Tensor) and xt.dtype == torch.bfloat16 and xt.dim() == 2
             and 1 <= xt.shape[0] <= most
@@ -806,10 +800,10 @@ def measure_rows_from_gate_up(w_gate_up: "Weight") -> int:
         _plan.rows_from[key] = threshold
         return _cold_time(lambda: gate_up_silu(x[:rows], w_gate_up))
 
-    first = ROWS_FROM
+    first = _plan.rules.rows_from
     try:
         for rows in (16, 12, 8, 4):
-            if timed(rows, 1) >= 0.97 * timed(rows, ROWS_FROM):
+            if timed(rows, 1) >= 0.97 * timed(rows, _plan.rules.rows_from):
                 break
             first = rows - 3
     finally:
@@ -836,10 +830,10 @@ def measure_rows_from_qkv(w_qkv: "Weight", nh: int, nkv: int, hd: int) -> int:
         return _cold_time(lambda: qkv_rope_store(x[:rows], w_qkv, table, pos[:rows], pos[:rows], kc,
                                                  vc, pages, 64, 0, nh, nkv, hd))
 
-    first = ROWS_FROM
+    first = _plan.rules.rows_from
     try:
         for rows in (16, 12, 8, 4):
-            if timed(rows, 1) >= 0.97 * timed(rows, ROWS_FROM):
+            if timed(rows, 1) >= 0.97 * timed(rows, _plan.rules.rows_from):
                 break
             first = rows - 3
     finally:

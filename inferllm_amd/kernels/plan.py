@@ -23,9 +23,29 @@ The float32 path has one way per product and no plan.
 """
 from __future__ import annotations
 
+from dataclasses import asdict, dataclass
 from typing import Dict, Optional, Tuple
 
 NEVER_BELOW = 17          # planes are not taken below 17 rows (the rule for unlisted shapes)
+
+
+@dataclass
+class Rules:
+    """What a shape that the tables lack gets, and the ranges of shapes in which a way is a
+    candidate at all.  Measured on an MI355X at the LLaMA-2-7B, 13B, 70B and LLaMA-3-8B matrix
+    shapes; a plan for other hardware or other shapes carries other numbers, the code none."""
+    rows_from: int = 17            # rows from which the products that share X through LDS are taken
+                                   # (up to 16 rows the few-rows kernels are the other way)
+    planes_most_cols: int = 8192   # output columns up to which planes were measured to pay: product
+                                   # and the norm that adds the planes take 0.6 to 0.75 of the vendor
+                                   # GEMM's and the norm's time when K >= 2 N, 0.8 to 0.95 when K = N
+    planes_min_elements: int = 1 << 22   # smaller matrices are not timed (both ways take a few
+                                         # microseconds and the clock would decide)
+    pad_rows_above: int = 64       # products of more rows than this and fewer than `pad_rows_to` may be
+    pad_rows_to: int = 256         # filled up to `pad_rows_to` rows (4096 x 11008: 60, 82 and 51 us at
+                                   # 128, 192 and 256 rows)
+    cut_min_rows: int = 1024       # below these no cut of a many-row product ever paid
+    cut_min_cols: int = 8192
 
 # (N, K) of a matrix with K >= 2 N -> fewest rows (1, 5, 9, 13 or 17) from which the planes and
 # the norm that adds them take less time than the residual-adding few-rows product.
@@ -141,34 +161,51 @@ FIXED_ROWS_FROM: Dict[tuple, int] = {
 }
 
 
+# (tile order, N, K) -> most rows for which the product goes to csrc/gemm_rows.hip (its launch
+# takes up to 128; unlisted shapes: all of them).  Measured against the vendor GEMM with the
+# elementwise kernel behind it at 80 / 96 / 128 rows: q|k|v 6144 x 4096 takes 21 / 24 / 34 against
+# 23 / 23 / 25 + 5 us (12288 x 4096: 26 / 27 / 36 against 30 / 33 / 34 + 5, so all rows).
+FIXED_ROWS_MOST: Dict[tuple, int] = {
+    ("qkv", 6144, 4096): 96,
+}
+
+
 class Plan:
     """The tables one engine's products are dispatched by (see the module text)."""
 
     def __init__(self, planes_from: Optional[dict] = None, cuts: Optional[dict] = None,
-                 measure: bool = False, rows_from: Optional[dict] = None):
+                 measure: bool = False, rows_from: Optional[dict] = None,
+                 rows_most: Optional[dict] = None, rules: Optional[Rules] = None):
         self.planes_from: Dict[Tuple[int, int], int] = dict(planes_from or {})
         self.cuts: Dict[tuple, tuple] = dict(cuts or {})
         self.rows_from: Dict[tuple, int] = dict(rows_from or {})
+        self.rows_most: Dict[tuple, int] = dict(rows_most or {})
+        self.rules = rules or Rules()
         self.measure = bool(measure)
 
     @classmethod
     def fixed(cls, measure: bool = False) -> "Plan":
-        return cls(FIXED_PLANES_FROM, FIXED_CUTS, measure, FIXED_ROWS_FROM)
+        return cls(FIXED_PLANES_FROM, FIXED_CUTS, measure, FIXED_ROWS_FROM, FIXED_ROWS_MOST)
 
     # ------------------------------------------------------------ as plain data
     def to_dict(self) -> dict:
         """JSON-able: {"planes_from": [[N, K, rows], ...], "cuts": [[key, plan], ...]}."""
         return {"planes_from": [[n, k, r] for (n, k), r in sorted(self.planes_from.items())],
                 "cuts": [[list(k), list(p)] for k, p in sorted(self.cuts.items(), key=repr)],
-                "rows_from": [[m, n, k, r] for (m, n, k), r in sorted(self.rows_from.items())]}
+                "rows_from": [[m, n, k, r] for (m, n, k), r in sorted(self.rows_from.items())],
+                "rows_most": [[m, n, k, r] for (m, n, k), r in sorted(self.rows_most.items())],
+                "rules": asdict(self.rules)}
 
     @classmethod
     def from_dict(cls, d: dict) -> "Plan":
         """A pinned plan: what `to_dict` gave, nothing measured."""
         return cls({(int(n), int(k)): int(r) for n, k, r in d.get("planes_from", [])},
                    {tuple(k): tuple(p) for k, p in d.get("cuts", [])}, measure=False,
-                   rows_from={(str(m), int(n), int(k)): int(r) for m, n, k, r in d.get("rows_from", [])})
+                   rows_from={(str(m), int(n), int(k)): int(r) for m, n, k, r in d.get("rows_from", [])},
+                   rows_most={(str(m), int(n), int(k)): int(r) for m, n, k, r in d.get("rows_most", [])},
+                   rules=Rules(**{k: int(v) for k, v in d.get("rules", {}).items()}))
 
     def __eq__(self, other) -> bool:
         return (isinstance(other, Plan) and self.planes_from == other.planes_from
-                and self.cuts == other.cuts and self.rows_from == other.rows_from)
+                and self.cuts == other.cuts and self.rows_from == other.rows_from
+                and self.rows_most == other.rows_most and self.rules == other.rules)

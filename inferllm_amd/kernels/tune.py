@@ -19,16 +19,14 @@ import sys
 
 
 def matrices(engine):
-    """Distinct bfloat16 matrices of the engine's parts, as (shape, `ops.Weight` or tensor)."""
+    """Distinct bfloat16 matrices that the engine's parts list as having several ways
+    (`Part.tunables`), as (shape, `ops.Weight` or tensor)."""
     import torch
 
     from . import ops
     seen = {}
     for part in engine.model.every_part():
-        if part is engine.model.head or part is engine.model.embedding:
-            continue                  # float32 logits never go through the products planned
-                                      # here, and the embedding table is not multiplied at all
-        for w in vars(part).values():
+        for _kind, w, _geometry in part.tunables():
             plain = ops.plain_weight(w) if isinstance(w, (ops.Weight, torch.Tensor)) else None
             if plain is not None and plain.dim() == 2 and plain.dtype == torch.bfloat16:
                 seen.setdefault(tuple(plain.shape), w)
@@ -45,50 +43,36 @@ def tune_config(cfg: dict, max_rows: int, repeats: int, say, rows_only: bool = F
     from . import ops
     from .plan import NEVER_BELOW, Plan
     one = dict(cfg, num_hidden_layers=1)
+    plan = Plan()
     eng = Engine.from_random(one, seed=0, dtype="bfloat16", max_batch=1, max_seq_len=64,
-                             decode_copies=True, plan=Plan())
-    ops.use_plan(Plan())
-    planes, cuts, rows = {}, {}, {}
+                             decode_copies=True, plan=plan)
+    ops.use_plan(plan)
+    rules = plan.rules
+    cuts = {}
+    # what the parts themselves list: the thin matrices' planes and the fused products' rows
     for part in eng.model.every_part():
-        # a mixer that keeps a fused q|k|v matrix with its head geometry (the attention part)
-        w = getattr(part, "w_qkv", None)
-        if isinstance(w, ops.Weight) and w.mode == "qkv" and w.tiled is not None and w.shape[1] % 64 == 0:
-            key = ("qkv",) + tuple(w.shape)
-            if key not in rows:
-                votes = sorted(ops.measure_rows_from_qkv(w, part.nh, part.nkv, part.hd)
-                               for _ in range(repeats))
-                rows[key] = votes[len(votes) // 2]
-                say(f"  q|k|v {w.shape[0]} x {w.shape[1]}: shared-X kernel from {rows[key]} rows (runs: {votes})")
-        # a feed-forward that keeps a fused gate|up matrix in its fused kernel's tile order
-        w = getattr(part, "w_gate_up", None)
-        if isinstance(w, ops.Weight) and w.mode == "gate_up" and w.tiled is not None and w.shape[1] % 64 == 0:
-            key = ("gate_up",) + tuple(w.shape)
-            if key not in rows:
-                votes = sorted(ops.measure_rows_from_gate_up(w) for _ in range(repeats))
-                rows[key] = votes[len(votes) // 2]
-                say(f"  gate|up {w.shape[0]} x {w.shape[1]}: shared-X kernel from {rows[key]} rows (runs: {votes})")
-    rows = {k: v for k, v in rows.items() if v != ops.ROWS_FROM}
+        for kind, w, geometry in part.tunables():
+            if rows_only and kind == "plain":
+                continue
+            entry = ops.tune_product(plan, kind, w, votes=repeats, **geometry)
+            if entry is not None:
+                say(f"  {entry[0]} {entry[1]}: {entry[2]}")
+    planes = {k: v for k, v in plan.planes_from.items() if v != NEVER_BELOW}
+    rows = {k: v for k, v in plan.rows_from.items() if v != rules.rows_from}
     if rows_only:
         return planes, cuts, rows
     for (N, K), w in sorted(matrices(eng).items()):
         plain = ops.plain_weight(w)
-        if (isinstance(w, ops.Weight) and w.mode == "plain" and w.tiled is not None and K >= 2 * N
-                and N <= ops.MID_MAX_COLS and N % 4 == 0):
-            votes = sorted(ops.measure_planes_from(w) for _ in range(repeats))
-            first = votes[len(votes) // 2]
-            say(f"  planes {N} x {K}: from {first} rows (runs: {votes})")
-            if first != NEVER_BELOW:
-                planes[(N, K)] = first
-        for rows32 in range(ops.PAD_MIN_ROWS // 32 + 1, ops.PAD_ROWS // 32 + 1):
-            M = min(rows32 * 32, ops.PAD_ROWS - 1)
+        for rows32 in range(rules.pad_rows_above // 32 + 1, rules.pad_rows_to // 32 + 1):
+            M = min(rows32 * 32, rules.pad_rows_to - 1)
             x = torch.randn(M, K, device=plain.device).to(torch.bfloat16)
-            votes = [ops.measure_plan(x, plain, [(), ("pad", ops.PAD_ROWS)], MARGIN) for _ in range(repeats)]
+            votes = [ops.measure_plan(x, plain, [(), ("pad", rules.pad_rows_to)], MARGIN) for _ in range(repeats)]
             best = max(set(votes), key=votes.count)
             if best:
                 cuts[("pad", rows32, N, K)] = best
-        if N < ops.PLAN_MIN_COLS:
+        if N < rules.cut_min_cols:
             continue
-        for rows256 in range(ops.PLAN_MIN_ROWS // 256, max_rows // 256 + 1):
+        for rows256 in range(rules.cut_min_rows // 256, max_rows // 256 + 1):
             M = rows256 * 256
             x = torch.randn(M, K, device=plain.device).to(torch.bfloat16)
             votes = [ops.measure_plan(x, plain, None, MARGIN) for _ in range(repeats)]
