@@ -1,4 +1,5 @@
-// C entry points of the kernel library.  Every function launches on `stream`
+// C entry points of the kernel library (the switches that tests and tuning runs flip are
+// declared apart, in api_test.h: nothing of the product calls them).  Every function launches on `stream`
 // and returns ILLM_OK, ILLM_ERR_ARG (sizes or dtypes it does not take; nothing
 // was launched), ILLM_ERR_LAUNCH or, where said, ILLM_ERR_SCRATCH.  Pointers are device pointers.  dtype codes:
 // 0 = float32, 1 = bfloat16.
@@ -51,9 +52,6 @@ int illm_gemm_f32_mfma(const float* X, const float* W, void* Y, int y_dt, int M,
 // matrix cores' float32 instruction with operands straight from memory.
 int illm_gemm_rows_f32_mfma(const float* X, const float* W, void* Y, int y_dt, int M, int N, int K,
                             void* stream);
-// Tests: tiles of 16 rows of W a block of that kernel takes (1 or 2; 0: the library's choice).
-// The sums are the same bits either way.
-void illm_set_rows_f32_tiles(int tiles);
 
 // The same product for M <= 16 rows when X and W are float32 and K % 4 == 0: W is read once
 // (decoding on the 32-bit path); plain float32 multiply-adds.
@@ -87,16 +85,6 @@ int illm_attn_prefill_paged_bf16(const void* qkv, void* out, const int32_t* cu_s
                                  const void* kcache, const void* vcache, const int32_t* page_table,
                                  int table_stride, int page_size, int ring, int n_seqs, int max_len,
                                  int nh, int nkv, int hd, float scale, int window, void* stream);
-
-// Tests: whether float32 prompts with head sizes 32, 64, 96 and 128 take the kernel on the matrix
-// cores' float32 instruction (1, default) or the multiply-add kernel of every other size (0).
-void illm_set_attn_f32_mfma(int on);
-
-// Tuning and tests: which prefill attention kernel head sizes up to 128 take: 0 the one with one
-// LDS buffer (which larger head sizes use), 2 the one with two buffers and one barrier a tile
-// (needs a positive scale), 1 (default) the second for head sizes 64 to 128 and sequences of
-// 1,024 keys or more.
-void illm_set_prefill_two_buffers(int on);
 
 // One query row per sequence over the paged cache.  partial: float32
 // [B][nh][nsplit][hd + 2] scratch.  seq_len[b] = keys of sequence b, the new one included.
@@ -159,19 +147,6 @@ int illm_gemm_skinny_add(const void* X, const void* W, const void* Wt, float* Y,
 int illm_gemm_mid_bf16(const void* X, const void* Wt, void* Y, int y_dt, int M, int N, int K,
                        int splits, void* stream);
 int illm_gemm_mid_splits(int N, int K);
-void illm_set_mid_tiles_per_wave(int n);
-// Tuning and tests: rows of X a launch of that kernel takes, 64 or 128 (default); W is read once
-// a launch.
-void illm_set_mid_rows_a_launch(int rows);      // tuning: 1 or 2 (0: by the number of tiles)
-
-// Tuning and tests: 0 switches off the variant of the residual-adding product in which, for K up
-// to 4096 and at most 512 tiles, 8 waves each take their whole share of K at once (default 1).
-void illm_set_skinny_one_shot(int on);
-
-// Tuning and tests: 0 sends grouped heads of head sizes up to 128 to the decode attention kernel
-// with P.V on the vector units, which larger head sizes use, instead of the one with both
-// products on the matrix cores (default 1).
-void illm_set_gqa_pv_on_matrix_cores(int on);
 
 // Products of 1 to 128 bfloat16 rows (meant for 9 and more) from the tiled copy
 // Wt of W, K a multiple of 64, X shared by a block's waves through LDS, K cut inside the block
@@ -189,11 +164,6 @@ int illm_qkv_rope_store_rows(const void* X, const void* Wt, void* Y, int M, int 
                              const int32_t* page_table, int table_stride, int page_size, int ring,
                              int nh, int nkv, int hd, const float* ssq, int parts, float eps,
                              void* stream);
-// Tuning and tests: tiles a block of these products takes (2 to 8) and parts of K (1, 2, 4;
-// four tiles and more: 1, 2); 0: the library's own choice.
-void illm_set_rows_shape(int tb, int kp);
-// Tuning and tests: rows of X a launch of these products takes, 64 or 128 (default).
-void illm_set_rows_a_launch(int rows);
 
 // Y[M, F] = silu(X . Wg^T) * (X . Wu^T), W = [Wg | Wu] as [2F, K]; same limits as the skinny
 // product, `ssq` included.  waves_wanted: waves per block (0: the default choice).

@@ -18,6 +18,7 @@
 #include <mutex>
 
 #include "api.h"
+#include "api_test.h"
 #include "common.h"
 
 #define NEG_INF (-INFINITY)

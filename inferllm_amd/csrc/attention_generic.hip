@@ -13,6 +13,7 @@
 #include <math.h>
 
 #include "api.h"
+#include "api_test.h"
 #include "common.h"
 
 #define AQ 32  // query rows of a block

@@ -27,6 +27,7 @@
 #include <mutex>
 
 #include "api.h"
+#include "api_test.h"
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));

@@ -11,6 +11,7 @@
 // The reference's float product is the same sum (src/kern/naive/naive.cpp:363-379);
 // its GPU path calls cublasSgemm (src/kern/gpu/kernel_gpu.cu:420-435).
 #include "api.h"
+#include "api_test.h"
 #include "common.h"
 
 #define GT 64   // tile of outputs per block (GT x GT)

@@ -17,6 +17,7 @@
 // The reference has one GEMM for every number of rows (cublasSgemm,
 // src/kern/gpu/kernel_gpu.cu:420-435).
 #include "api.h"
+#include "api_test.h"
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));

@@ -15,6 +15,7 @@
 //
 // The reference calls cublasSgemm with M = 1 here (src/kern/gpu/kernel_gpu.cu:420-435).
 #include "api.h"
+#include "api_test.h"
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
