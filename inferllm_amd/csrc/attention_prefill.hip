@@ -280,11 +280,12 @@ struct PfBuf {
     static constexpr int v = B;
 };
 
-template <int HD>
+template <int HD, bool PAGED>
 __global__ void __launch_bounds__(256, 2)
 attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out,
                           const int32_t* __restrict__ cu, int n_qblk, int nh, int nkv,
-                          float scale_log2, int window, int hb_per_xcd, int n_hb, int zigzag) {
+                          float scale_log2, int window, int hb_per_xcd, int n_hb, int zigzag,
+                          PfPages pg) {
     constexpr int KS = HD / 16;        // k-steps of the first product
     constexpr int DB = HD / 32;        // 32-row blocks of O^T
     constexpr int UK = HD / 8;         // 16-byte units in a K row
@@ -304,14 +305,19 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
     const int start = cu[b], len = cu[b + 1] - start;
     const int q0 = qb * PF_BM;
     if (q0 >= len) return;
+    // PAGED: the rows stand at positions pos0 .. and see the keys 0 .. of the sequence's cache
+    const int slot = PAGED ? pg.seq_slot[b] : 0;
+    const int pos0 = PAGED ? pg.seq_start[b] : 0;
+    const int total = pos0 + len;                       // keys of the sequence after this step
     const int kvh = h / (nh / nkv);
     const size_t rowlen = (size_t)(nh + 2 * nkv) * HD;
-    const uint32_t row_bytes = (uint32_t)(rowlen * 2);
+    const uint32_t row_bytes = PAGED ? (uint32_t)(HD * 2) : (uint32_t)(rowlen * 2);   // of a key's row
     const int tid = threadIdx.x, wave = wave_index(), lane = tid & 63;
     const int lq = lane & 31, half = lane >> 5;
     const int q_row0 = q0 + wave * 32;
-    const int q = q_row0 + lq;
+    const int q = q_row0 + lq;                          // row within the sequence's rows
     const int qc = q < len ? q : len - 1;
+    const int qp = pos0 + q;                            // its position
 
     illm_u32x4_t qf[KS];
     {
@@ -330,11 +336,11 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
         for (int i = 0; i < 16; ++i) o[d][i] = 0.f;
     float m = NEG_INF, l = 0.f;
 
-    const int k_end = min(len, q0 + PF_BM);
-    int k_begin = window > 0 ? max(0, q0 - window + 1) : 0;
+    const int k_end = min(total, pos0 + q0 + PF_BM);
+    int k_begin = window > 0 ? max(0, pos0 + q0 - window + 1) : 0;
     k_begin = (k_begin / PF_BN) * PF_BN;
-    const int wk_end = min(len, q_row0 + 32);                       // this wave's last key + 1
-    const int wk_begin = window > 0 ? max(0, q_row0 - window + 1) : 0;
+    const int wk_end = min(total, pos0 + q_row0 + 32);              // this wave's last key + 1
+    const int wk_begin = window > 0 ? max(0, pos0 + q_row0 - window + 1) : 0;
 
     // Staging.  K: this thread brings chunks chq + 4 it (it < NLD) of key `skey`.  V: keys
     // 4 g .. 4 g + 3, dims 8 c .. 8 c + 7 (threads with c >= UK, at head sizes below 128, bring
@@ -346,6 +352,8 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
     // lane's 8 keys in the order in which the first product leaves them, is one 16-byte read:
     // bits (sub, sub, m, a, h) -> (.., h, a)
     const int vpg = (vg & 12) | ((vg & 1) << 1) | ((vg >> 1) & 1);
+    // (not PAGED: the keys are the step's own rows; PAGED: a tile of 64 keys is a page or an
+    // aligned part of one, found through the page table when the tile is asked for)
     const char* const kg = (const char*)(qkv + (size_t)start * rowlen + (size_t)(nh + kvh) * HD);
     const char* const vg_base = (const char*)(qkv + (size_t)start * rowlen + (size_t)(nh + nkv + kvh) * HD);
     const uint32_t koff_whole = (uint32_t)skey * row_bytes + chq * 16;
@@ -359,16 +367,27 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
     auto fetch = [&](int k0) __attribute__((always_inline)) {
         uint32_t ko = koff_whole, v0 = voff_whole, v1 = voff_whole + row_bytes,
                  v2 = voff_whole + 2 * row_bytes, v3 = voff_whole + 3 * row_bytes;
-        if (k0 + PF_BN > len) {                    // the sequence's last tile: rows clamped
-            const int last = len - 1 - k0;
+        if (k0 + PF_BN > total) {                  // the sequence's last tile: rows clamped
+            const int last = total - 1 - k0;
             ko = (uint32_t)min(skey, last) * row_bytes + chq * 16;
             v0 = (uint32_t)min(4 * vg + 0, last) * row_bytes + vc * 16;
             v1 = (uint32_t)min(4 * vg + 1, last) * row_bytes + vc * 16;
             v2 = (uint32_t)min(4 * vg + 2, last) * row_bytes + vc * 16;
             v3 = (uint32_t)min(4 * vg + 3, last) * row_bytes + vc * 16;
         }
-        const char* kt = kg + (size_t)k0 * row_bytes;
-        const char* vt = vg_base + (size_t)k0 * row_bytes;
+        const char* kt;
+        const char* vt;
+        if (PAGED) {
+            int lp = k0 / pg.page_size;
+            if (pg.ring > 0) lp %= pg.ring;
+            const int phys = pg.page_table[(size_t)slot * pg.table_stride + lp];
+            const size_t at = (((size_t)phys * nkv + kvh) * pg.page_size + k0 % pg.page_size) * (size_t)(HD * 2);
+            kt = (const char*)pg.kcache + at;
+            vt = (const char*)pg.vcache + at;
+        } else {
+            kt = kg + (size_t)k0 * row_bytes;
+            vt = vg_base + (size_t)k0 * row_bytes;
+        }
 #pragma unroll
         for (int it = 0; it < NLD; ++it) kpre[it] = *(const illm_u32x4_t*)(kt + ko + it * 64);
         vpre0 = *(const illm_u32x4_t*)(vt + v0);
@@ -417,7 +436,7 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
                                                                      *(const bf16x8_t*)&qf[st],
                                                                      s[sub], 0, 0, 0);
                 }
-            const bool need_mask = (k0 + PF_BN > q_row0 + 1) || (k0 + PF_BN > len) || (window > 0);
+            const bool need_mask = (k0 + PF_BN > pos0 + q_row0 + 1) || (k0 + PF_BN > total) || (window > 0);
             float mx = NEG_INF;
             if (need_mask) {                 // the same for the whole wave: one branch, two bodies
 #pragma unroll
@@ -425,7 +444,7 @@ attn_prefill_mfma2_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ o
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int key = k0 + sub * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
-                        const bool ok = key <= q && key < len && (window <= 0 || key > q - window);
+                        const bool ok = key <= qp && key < total && (window <= 0 || key > qp - window);
                         const float v = ok ? s[sub][i] : NEG_INF;
                         s[sub][i] = v;
                         mx = fmaxf(mx, v);
@@ -529,7 +548,7 @@ extern "C" void illm_set_prefill_two_buffers(int on) { PF_TWO_BUFFERS = on; }
 
 // The two-buffer kernel needs more LDS than a kernel may have without asking: asked for once per
 // device and head size.
-template <int HD>
+template <int HD, bool PAGED>
 static int prefill2_lds_ready(size_t bytes) {
     static bool ready[64] = {};
     static std::mutex lock;
@@ -537,7 +556,7 @@ static int prefill2_lds_ready(size_t bytes) {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ILLM_ERR_LAUNCH;
     std::lock_guard<std::mutex> hold(lock);
     if (!ready[dev]) {
-        if (hipFuncSetAttribute((const void*)attn_prefill_mfma2_kernel<HD>,
+        if (hipFuncSetAttribute((const void*)attn_prefill_mfma2_kernel<HD, PAGED>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
             return ILLM_ERR_LAUNCH;
         ready[dev] = true;
@@ -555,20 +574,26 @@ static int launch_prefill(const void* qkv, void* out, const int32_t* cu, int n_s
     const long long hb_per_xcd = (n_hb + 7) / 8;
     const long long blocks = 8 * hb_per_xcd * n_qblk;
     if (blocks > 0x7fffffffLL) return ILLM_ERR_ARG;
-    if constexpr (HD <= 128 && HD % 32 == 0) if (!pg) {
-        // measured at 32 heads: head size 128, 2,048 keys 81 -> 76 us, 4,096 keys 236 -> 214; head
-        // size 64 and sequences of 512 lose a tenth (a tile more of set-up before the first product)
+    if constexpr (HD <= 128 && HD % 32 == 0) {
         // measured at 32 heads of size 128: 2,048 keys 81 -> 71 us, 4,096 keys 228 -> 193, 8,192
         // keys (8 groups) 704 -> 615; size 64, 2,048 keys 46.7 -> 42.7; four sequences of 1,024
-        // 66 -> 64; eight of 512 lose (45 -> 48: a tile more of set-up before the first product)
+        // 66 -> 64; eight of 512 lose (45 -> 48: a tile more of set-up before the first product).
+        // (steps that go on from the cache: `max_len` is the most rows a sequence brings, which
+        // see at least as many keys)
         if (PF_TWO_BUFFERS == 2 || (PF_TWO_BUFFERS == 1 && HD >= 64 && max_len >= 1024 && scale > 0.f)) {
             const size_t lds = (size_t)2 * (PF_BN * (HD + 8) + HD * (PF_BN + 8)) * sizeof(bf16_t);
-            const int rc = prefill2_lds_ready<HD>(lds);
+            const int rc = pg ? prefill2_lds_ready<HD, true>(lds) : prefill2_lds_ready<HD, false>(lds);
             if (rc != ILLM_OK) return rc;
-            hipLaunchKernelGGL(attn_prefill_mfma2_kernel<HD>, dim3((unsigned)blocks), dim3(256), lds, st,
-                               (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
-                               scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
-                               hb_per_xcd * n_qblk <= 64 ? 1 : 0);
+            if (pg)
+                hipLaunchKernelGGL((attn_prefill_mfma2_kernel<HD, true>), dim3((unsigned)blocks), dim3(256), lds,
+                                   st, (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
+                                   scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
+                                   hb_per_xcd * n_qblk <= 64 ? 1 : 0, *pg);
+            else
+                hipLaunchKernelGGL((attn_prefill_mfma2_kernel<HD, false>), dim3((unsigned)blocks), dim3(256), lds,
+                                   st, (const bf16_t*)qkv, (bf16_t*)out, cu, n_qblk, nh, nkv,
+                                   scale * 1.44269504088896340736f, window, (int)hb_per_xcd, (int)n_hb,
+                                   hb_per_xcd * n_qblk <= 64 ? 1 : 0, PfPages());
             return illm_launch_status();
         }
     }

@@ -289,12 +289,42 @@ def test_attn_prefill_paged(dtype, nh, nkv, hd, starts, rows, page):
     cu = torch.tensor([0] + list(torch.tensor(rows).cumsum(0)), dtype=torch.int32)
     st = torch.tensor(starts, dtype=torch.int32)
     scale = 1.0 / math.sqrt(hd)
-    got = ops().attn_prefill_paged(qkv.to(DEV), cu.to(DEV), slots.to(DEV), st.to(DEV), kc.to(DEV), vc.to(DEV),
-                                   pt.to(DEV), page, 0, len(rows), max(rows), nh, nkv, hd, scale, 0)
     want = R.attn_prefill_paged(qkv, cu, slots, st, kc, vc, pt, page, 0, len(rows), max(rows), nh, nkv, hd,
                                 scale, 0)
-    assert torch.isfinite(got.float()).all()
-    close(got, want, dtype, scale=2)
+    lib = ops()._lib()
+    try:
+        # the library's own choice, and for bfloat16 the kernel with two LDS buffers forced
+        # (head sizes 32 to 128 in steps of 32; the others do not have it)
+        for which in ((1, 2) if dtype == torch.bfloat16 else (1,)):
+            lib.illm_set_prefill_two_buffers(which)
+            got = ops().attn_prefill_paged(qkv.to(DEV), cu.to(DEV), slots.to(DEV), st.to(DEV), kc.to(DEV),
+                                           vc.to(DEV), pt.to(DEV), page, 0, len(rows), max(rows), nh, nkv, hd,
+                                           scale, 0)
+            assert torch.isfinite(got.float()).all()
+            close(got, want, dtype, scale=2)
+    finally:
+        lib.illm_set_prefill_two_buffers(1)
+
+
+def test_attn_prefill_paged_long_steps_with_a_window_ring():
+    """Steps of 1,100 rows that go on from 1,500 and from 0 tokens (the kernel with two LDS buffers
+    is the library's choice from 1,024 rows on): all keys, and a window of 500 keys over a ring of
+    26 pages, which the longer sequence's 2,600 positions wrap round."""
+    dtype, nh, nkv, hd, page = torch.bfloat16, 4, 2, 128, 64
+    starts, rows = [1500, 0], [1100, 1030]
+    lens = [s + r for s, r in zip(starts, rows)]
+    qkv = rnd(sum(rows), (nh + 2 * nkv) * hd, dtype=dtype, seed=13)
+    qkv[:, nh * hd:] = float("nan")
+    cu = torch.tensor([0] + list(torch.tensor(rows).cumsum(0)), dtype=torch.int32)
+    st = torch.tensor(starts, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(hd)
+    for window, ring in ((0, 0), (500, 26)):
+        pt, kc, vc, slots, _ = paged_case(dtype, nkv, hd, lens, page, ring=ring)
+        got = ops().attn_prefill_paged(qkv.to(DEV), cu.to(DEV), slots.to(DEV), st.to(DEV), kc.to(DEV), vc.to(DEV),
+                                       pt.to(DEV), page, ring, len(rows), max(rows), nh, nkv, hd, scale, window)
+        want = R.attn_prefill_paged(qkv, cu, slots, st, kc, vc, pt, page, ring, len(rows), max(rows),
+                                    nh, nkv, hd, scale, window)
+        close(got, want, dtype, scale=2)
 
 
 def test_attn_prefill_finds_one_far_key():
