@@ -53,6 +53,9 @@ class DecoderModel:
                 raise ValueError(f"schedule: cache line {e.cache_line} is read before any run writes it")
         self.loaded = False
         self.graph_safe = all(getattr(p, "graph_safe", True) for p in self.every_part())
+        # steps of several tokens a sequence may be replayed from graphs only if every part says so
+        self.graph_safe_prompts = self.graph_safe and all(
+            getattr(p, "graph_safe_prompts", False) for p in self.every_part())
         # mixers that cannot go on from their cache by more than one token a step
         self.one_token_mixers = sorted({type(l.mixer).__name__ for l in self.layers
                                         if not getattr(l.mixer, "takes_continuations", False)})

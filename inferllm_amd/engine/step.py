@@ -171,7 +171,8 @@ class StepRunner:
         self._graphs: Dict[tuple, _DecodeGraph] = {}
         # steps of few rows with several tokens a sequence (short prompts, a conversation's turns):
         # replayed from a graph from the second step of a shape on (the first runs eagerly: one
-        # prompt does not pay for a capture)
+        # prompt does not pay for a capture), if every part of the model says it takes that
+        self.use_prompt_graphs = self.use_graphs and model.graph_safe_prompts
         self._prompt_graphs: Dict[tuple, _PromptGraph] = {}
         self._prompt_uses: Dict[tuple, int] = {}
 
@@ -247,7 +248,7 @@ class StepRunner:
         """The graph that this step of several tokens a sequence is replayed from, or None if it
         runs eagerly: more rows, sequences or wanted rows than the graphs hold, or a shape seen
         for the first time."""
-        if not self.use_graphs:
+        if not self.use_prompt_graphs:
             return None
         rows = sum(len(e.tokens) for e in entries)
         wanted = sum(len(e.want) for e in entries)

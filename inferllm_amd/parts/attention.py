@@ -32,6 +32,8 @@ class Attention(Mixer):
     tokens of earlier steps, over the cache.
     """
 
+    graph_safe_prompts = True
+
     adds_residual = True
     takes_normed_rows = True
 

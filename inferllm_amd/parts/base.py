@@ -59,8 +59,15 @@ class Part:
     `graph_safe`: the part's forward only launches work on the current stream (no host
     synchronisation, no host reads of device data), so decode steps that contain it may
     be captured into a HIP graph.  A part that reads device data on the host sets it False.
+
+    `graph_safe_prompts`: the same holds for steps of several tokens a sequence, which are then
+    replayed from graphs too when they have few rows.  Such a step has the graph's shapes, not its
+    own: `ctx.n_rows`, `ctx.n_seqs`, `ctx.max_len` and `ctx.max_rows` are upper bounds, the rows
+    that fill the graph up are a sequence of their own on the cache's spare slot, and sequences
+    that fill it up have no rows.  A part has to say that it takes this; the library's own do.
     """
     graph_safe = True
+    graph_safe_prompts = False
     # A short cut between a block's parts for steps of few rows (False: the plain protocol, which
     # every part supports).  A mixer or feed-forward with `adds_residual` takes
     # `forward(..., residual=x, next_norm=norm)` and may add its result to the float32 residual

@@ -18,6 +18,8 @@ class PreNormBlock(Block):
     left to add) or `ops.NormedRows`.
     """
 
+    graph_safe_prompts = True
+
     takes_next_norm = True
     takes_prepared_rows = True
 

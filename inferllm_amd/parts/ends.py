@@ -14,6 +14,8 @@ from .base import Embedding, Head, StepContext, register_part
 class TokenEmbedding(Embedding):
     """Row copy, no scaling (src/kern/naive/naive.cpp:43-54); rows become float32."""
 
+    graph_safe_prompts = True
+
     def __init__(self, vocab_size: int, hidden_size: int, tensors=None):
         super().__init__(tensors)
         self.V, self.E = int(vocab_size), int(hidden_size)
@@ -37,6 +39,8 @@ class LMHead(Head):
     last row only).  `tied_fallback` names the tensor used when the head's own is
     absent from the checkpoint (tied embeddings).
     """
+
+    graph_safe_prompts = True
 
     def __init__(self, hidden_size: int, vocab_size: int, tied_fallback: Optional[str] = None,
                  tensors=None):

@@ -20,6 +20,8 @@ class SwiGLU(FeedForward):
     elementwise kernels (src/kern/gpu/kernel_gpu.cu:183-258).
     """
 
+    graph_safe_prompts = True
+
     adds_residual = True
     takes_normed_rows = True
 

@@ -18,6 +18,8 @@ class RMSNorm(Norm):
     (the reference fixes 1e-6 / 1e-5 at src/graph/llama_like.cpp:78 and src/core/graph.h:163).
     """
 
+    graph_safe_prompts = True
+
     adds_planes = True
 
     def __init__(self, size: int, eps: float, tensors=None):

@@ -40,6 +40,8 @@ class Rotary(PositionEncoding):
     (naive.cpp:415-440).  theta, rotary_dim and max_positions are parameters.
     """
 
+    graph_safe_prompts = True
+
     def __init__(self, head_dim: int, rotary_dim: int, theta: float, pairing: str,
                  max_positions: int, tensors=None):
         super().__init__(tensors)
@@ -80,6 +82,8 @@ class Rotary(PositionEncoding):
 @register_part("position", "none")
 class NoPosition(PositionEncoding):
     """No encoding: q and k stay as they are; k and v are still stored."""
+
+    graph_safe_prompts = True
 
     def on_qkv(self, qkv, ctx: StepContext, nh, nkv, hd, kcache, vcache, group) -> None:
         ops.rope_store(qkv, None, 0, 0, ctx.row_pos, ctx.row_slot,

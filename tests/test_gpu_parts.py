@@ -399,6 +399,37 @@ def test_a_mixer_with_state_under_decode_graphs(tmp_path, graphs):
         assert {k[0] for k in eng.runner._graphs} == {1, 2, 4}
 
 
+def test_prompt_steps_are_replayed_from_graphs_only_if_every_part_says_so(tmp_path):
+    """A part that promises no host reads in steps of single tokens (`graph_safe`) has promised
+    nothing about steps of several tokens: the toy mixer reads the step's lengths on the host
+    there, which a capture would refuse.  Its model's short prompt steps run eagerly however
+    often a shape comes back, while its decode steps are replayed from graphs; a model of the
+    library's own parts has both."""
+    import inferllm_amd as I
+    from tiny import TINY_A, make_model_dir, random_ids, read_weights
+    register_toy()
+    cfg = {"architectures": ["ToyRunningMeanForTests"], "hidden_size": 48, "vocab_size": 100, "layers": 2,
+           "eps": 1e-5, "mixer": "toy_running_mean_on_device"}
+    d = I.write_random_model(str(tmp_path / "toy"), I.config_from_dict(cfg), seed=8)
+    w = read_weights(d)
+    eng = I.Engine.from_pretrained(d, dtype="float32", max_batch=2, max_seq_len=256)
+    assert eng.runner.use_graphs and not eng.runner.use_prompt_graphs
+    for turn in range(3):                                   # the same shapes three times
+        ids = random_ids(14, 100, 60 + turn)
+        want = toy_plain(w, cfg, ids)
+        s = eng.alloc_slot()
+        out = eng.step([I.StepEntry(s, ids[:9], [0, 8])])
+        assert rel(out[0], want[0]) < 2e-5 and rel(out[1], want[8]) < 2e-5
+        out = eng.step([I.StepEntry(s, ids[9:12], [2])])    # goes on by three tokens
+        assert rel(out[0], want[11]) < 2e-5
+        for t in (12, 13):
+            assert rel(eng.step([I.StepEntry(s, [ids[t]], [0])])[0], want[t]) < 2e-5
+        eng.free_slot(s)
+    assert not eng.runner._prompt_graphs and {k[0] for k in eng.runner._graphs} == {1}
+    la = I.Engine.from_pretrained(make_model_dir(tmp_path, TINY_A, seed=1), dtype="float32", max_batch=2)
+    assert la.runner.use_prompt_graphs
+
+
 def test_a_mixer_says_whether_it_goes_on_by_several_tokens(tmp_path):
     """The rule "all start, or all go on by one" belongs to the mixers: a mixer that says it takes
     continuations (one with state of fixed size here; attention without a window too) lets a
