@@ -61,13 +61,22 @@ def _length_class(n: int, limit: int) -> int:
     return min(c, max(limit, 1))
 
 
-class _DecodeGraph:
-    """Static buffers and the captured graph for decode steps of one bucket size and one class
-    of lengths."""
+def _ragged(lens: Sequence[int]) -> bool:
+    """Whether the sequences of a decode step differ widely in length: the longest has 1,024 keys
+    or more and the mean is at most 0.6 of it.  Attention then cuts the keys into more ranges, so
+    that the blocks of the long sequences do not outlast everything else."""
+    longest = max(lens)
+    return longest >= 1024 and 10 * sum(lens) <= 6 * longest * len(lens)
 
-    def __init__(self, runner: "StepRunner", size: int, max_len: int):
+
+class _DecodeGraph:
+    """Static buffers and the captured graph for decode steps of one bucket size, one class
+    of lengths and one answer to "do the lengths differ widely"."""
+
+    def __init__(self, runner: "StepRunner", size: int, max_len: int, ragged: bool = False):
         self.size = size
         self.max_len = max_len
+        self.ragged = ragged
         dev = runner.device
         self.meta = torch.zeros(4 * size, dtype=torch.int32, device=dev)   # tokens | pos | slot | len
         # host side of `meta`: pinned, so that one asynchronous copy brings a step's numbers over
@@ -86,7 +95,7 @@ class _DecodeGraph:
             device=runner.device, act_dtype=runner.act_dtype, prefill=False, n_rows=n, n_seqs=n,
             tokens=self.meta[:n], row_pos=self.meta[n:2 * n], row_slot=self.meta[2 * n:3 * n],
             cu_seqlens=self.cu, seq_slot=self.meta[2 * n:3 * n], seq_len=self.meta[3 * n:],
-            max_len=self.max_len, cache=runner.cache)
+            max_len=self.max_len, cache=runner.cache, ragged=self.ragged)
 
 
 PROMPT_GRAPH_ROWS = (16, 32, 64, 96, 128, 192, 256)   # rows of the graphs that short prompt steps are replayed from
@@ -378,10 +387,11 @@ class StepRunner:
                 tokens=meta[:B], row_pos=meta[B:2 * B], row_slot=meta[2 * B:3 * B],
                 cu_seqlens=torch.arange(B + 1, dtype=torch.int32, device=self.device),
                 seq_slot=meta[2 * B:3 * B], seq_len=meta[3 * B:], max_len=max(starts) + 1,
-                cache=self.cache)
+                cache=self.cache, ragged=_ragged([s + 1 for s in starts]))
             rows = torch.tensor(wanted, dtype=torch.int32, device=self.device) if wanted else None
             return self.model.forward(ctx, rows)
-        key = (size, _length_class(max(starts) + 1, self.cache.max_seq_len))
+        key = (size, _length_class(max(starts) + 1, self.cache.max_seq_len),
+               _ragged([s + 1 for s in starts]))
         g = self._graphs.get(key)
         if g is None:
             g = self._graphs[key] = _DecodeGraph(self, *key)
@@ -418,7 +428,7 @@ class StepRunner:
         for n in sorted(set(int(b) for b in batch_sizes)):
             if n < 1:
                 raise StepError("warm_up: batch sizes are positive")
-            key = (_bucket(n), _length_class(max(int(longest), 1), self.cache.max_seq_len))
+            key = (_bucket(n), _length_class(max(int(longest), 1), self.cache.max_seq_len), False)
             g = self._graphs.get(key)
             if g is None:
                 g = self._graphs[key] = _DecodeGraph(self, *key)

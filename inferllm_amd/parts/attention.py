@@ -116,7 +116,8 @@ class Attention(Mixer):
                                  self.scale, window)
         else:
             longest = min(ctx.max_len, window) if window else ctx.max_len
-            nsplit, waves = ops.decode_splits(ctx.n_seqs, nkv, longest, nh, hd)
+            nsplit, waves = ops.decode_splits(ctx.n_seqs, nkv, longest, nh, hd,
+                                              ragged=ctx.ragged and not window)
             o = ops.attn_decode(qkv, kc, vc, group.table, group.page_size, group.ring,
                                 ctx.seq_slot, ctx.seq_len, nh, nkv, hd, self.scale, window,
                                 nsplit, waves)

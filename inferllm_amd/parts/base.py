@@ -50,6 +50,9 @@ class StepContext:
     seq_start: Optional[torch.Tensor] = None     # [seqs] position of the sequence's first row
     max_rows: int = 0                 # most rows a sequence brings (host number)
     continues: bool = False
+    # a step of single tokens whose sequences differ widely in length (their mean is at most 0.6
+    # of the longest): work that is cut evenly by sequence is then uneven by block
+    ragged: bool = False
     exchange: Dict[Any, Any] = field(default_factory=dict)   # between runs of layers in one step
 
 

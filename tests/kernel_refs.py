@@ -159,7 +159,7 @@ def attn_prefill_paged(qkv, cu_seqlens, seq_slot, seq_start, kcache, vcache, pag
     return out
 
 
-def decode_splits(B, nkv, max_len, nh=0, hd=0):
+def decode_splits(B, nkv, max_len, nh=0, hd=0, ragged=False):
     return 2, 1
 
 

@@ -675,6 +675,37 @@ def test_decoding_across_a_class_of_lengths(tmp_path_factory):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("graphs", [True, False])
+def test_decoding_sequences_of_widely_different_lengths(tmp_path_factory, graphs):
+    """A decode step whose sequences differ widely in length (the longest 1,024 keys or more, the
+    mean at most 0.6 of it) has its keys cut into more ranges, and graphs of its own: sequences
+    of 1,100, 40 and 200 keys side by side, until the short ones end and the long one alone is
+    no longer such a step."""
+    from inferllm_amd import StepEntry
+    eng, plain, config = setup(tmp_path_factory, "D", "bfloat16", max_batch=3, max_seq_len=2048,
+                               max_tokens=1152 + 64 + 256, use_graphs=graphs)
+    heads = [1100, 40, 200]
+    tails = [12, 5, 8]
+    reqs = requests_for(config, [h + t for h, t in zip(heads, tails)], seed=27)
+    slots = [eng.alloc_slot() for _ in reqs]
+    eng.step([StepEntry(s, r[:h], []) for s, r, h in zip(slots, reqs, heads)])
+    got = [[] for _ in reqs]
+    for t in range(max(tails)):
+        live = [i for i in range(3) if t < tails[i]]
+        out = eng.step([StepEntry(slots[i], [reqs[i][heads[i] + t]], [0]) for i in live])
+        for row, i in enumerate(live):
+            got[i].append(out[row:row + 1].clone())
+    if graphs:       # three and two sequences in the graph of 4 and of 2 rows, the last one alone
+        assert set(eng.runner._graphs) == {(4, 2048, True), (2, 2048, True), (1, 2048, False)}
+    for i, r in enumerate(reqs):
+        want = plain(r)[heads[i]:]
+        per = (torch.cat(got[i]).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
+        assert float(per.max()) < BUDGET["bfloat16"], (i, per.tolist())
+    for s in slots:
+        eng.free_slot(s)
+    eng.cache.check()
+
+
 def test_kernel_timing_reports_every_op(tmp_path_factory):
     from inferllm_amd.kernels.profile import kernel_timing
     eng, plain, config = setup(tmp_path_factory, "A", "bfloat16", use_graphs=False)
@@ -812,7 +843,7 @@ def test_real_layer_sizes_with_many_sequences(tmp_path_factory, monkeypatch, nkv
             got[i].append(out[row:row + 1].clone())
     monkeypatch.setattr(torch, "matmul", real)
     assert not vendor, f"products of decode steps went to the vendor GEMM: rows x width {sorted(set(vendor))}"
-    assert sorted(size for size, _ in eng.runner._graphs) == buckets
+    assert sorted(k[0] for k in eng.runner._graphs) == buckets
     for i in sorted({0, 7, 16, later - 1, later, n - 7, n - 1}):   # the plain model is slow at these sizes
         want = plain_llama.forward_logits(config, w, reqs[i])[heads[i]:heads[i] + len(got[i])]
         per_pos = (torch.cat(got[i]).double().cpu() - want).abs().max(dim=1).values / want.abs().max()
@@ -906,7 +937,7 @@ def test_a_session_decodes_through_graphs_across_a_class_of_lengths(tmp_path_fac
         assert len(a1) == 40 and talk.length == 1039
         a2 = talk.say(second, max_new_tokens=8)
         assert talk.last_stats.prompt_tokens == 31 and talk.length == 1039 + 31 + 7
-    assert {k for k in eng.runner._graphs} == {(1, 1024), (1, 2048)}
+    assert {k for k in eng.runner._graphs} == {(1, 1024, False), (1, 2048, False)}
     seq = list(first) + a1 + list(second) + a2
     want = plain(seq)
     if dtype == "float32":
