@@ -971,15 +971,19 @@ def decode_splits(B: int, nkv: int, max_len: int, nh: int = 0, hd: int = 0, ragg
     microsecond of it, in at most 16 ranges; 8 waves a block (idle ones cost nothing) until
     there are 512 blocks, then 4.  `ragged` (the lengths differ widely, the longest has 1,024
     keys or more): every sequence has the same number of ranges, so the long sequences' blocks
-    outlast the others'; at least 8 ranges of 4 waves then (16 sequences of 64 to 4,096 keys,
-    32/8 heads: 30.5 -> 26.6 us, 32/32 heads: 82 -> 72; 8 of 50 to 4,000 keys: 49.5 -> 37.8)."""
+    outlast the others'; the ranges are doubled, up to 8, while that makes no more than 1,024
+    blocks (16 sequences of 64 to 4,096 keys, 32/8 heads: 30.5 -> 26.3 us, 32/32 heads: 80 -> 74;
+    one of 4,000 among 15 of 200: 27.7 -> 21.7 and 51.5 -> 40.7; beyond 1,024 blocks more ranges
+    cost more than they even out: one of 2,000 among 63 of 100, 32/32 heads, 34 us whole, 88 in
+    8 ranges)."""
     base = max(1, B * nkv)
     if nh > nkv > 0 and hd % 32 == 0 and 0 < hd <= 128:
         base *= -(-(nh // nkv) // 16)          # the grouped kernel takes 16 heads a block
     tiles = max(1, (max_len + 63) // 64)
     nsplit = max(1, min(-(-256 // base), 16, tiles))
-    if ragged and tiles >= 16 and nsplit < 8:
-        return 8, 4
+    if ragged and tiles >= 16:
+        while nsplit < 8 and base * nsplit * 2 <= 1024:
+            nsplit *= 2
     return nsplit, (8 if base * nsplit < 512 else 4)
 
 
