@@ -293,6 +293,33 @@ def test_rows_of_the_decode_graphs():
         assert b == _bucket(b)
 
 
+def test_steps_whose_lengths_differ_widely_get_more_key_ranges_within_bounds():
+    """The step function calls a decode step ragged when its longest sequence has 1,024 keys or
+    more and the mean length is at most 0.6 of that; attention then doubles the key ranges of
+    every sequence while there are fewer than 8, as long as that makes no more than 1,024 blocks, and never cuts
+    into fewer ranges than for even lengths."""
+    from inferllm_amd.engine.step import _ragged
+    from inferllm_amd.kernels.ops import decode_splits
+    assert _ragged([1101, 41, 201]) and _ragged([4000] + [200] * 15)
+    assert not _ragged([1101]) and not _ragged([1000, 10]) and not _ragged([2000, 1900, 1500])
+    assert not _ragged([1024, 1024 * 6 // 10 + 1]) and _ragged([1030, 200])
+    for nh, nkv in ((32, 32), (32, 8), (64, 8), (4, 2), (7, 7)):
+        blocks_a_range = nkv * -(-(nh // nkv) // 16) if nh > nkv else nkv
+        for B in (1, 2, 3, 4, 8, 16, 24, 32, 64, 128, 256):
+            for longest in (1024, 2048, 4096, 32768):
+                even, waves = decode_splits(B, nkv, longest, nh, 128)
+                more, waves_r = decode_splits(B, nkv, longest, nh, 128, ragged=True)
+                assert more >= even and more in (even, 2 * even, 4 * even, 8 * even) and waves_r in (4, 8)
+                if more > even:
+                    assert more < 16 and B * blocks_a_range * more <= 1024      # doubled only from fewer than 8
+                elif even < 8:
+                    assert B * blocks_a_range * even * 2 > 1024
+            # short sequences are left alone: a range is at least a tile of keys anyway
+            assert decode_splits(B, nkv, 640, nh, 128, ragged=True) == decode_splits(B, nkv, 640, nh, 128)
+    assert decode_splits(16, 8, 3800, 32, 128, ragged=True) == (8, 4)
+    assert decode_splits(64, 32, 2000, 32, 128, ragged=True) == decode_splits(64, 32, 2000, 32, 128) == (1, 4)
+
+
 def test_command_line_text_through_a_sentencepiece_model(tmp_path, capsys):
     """`bin/chat -p` takes text through the folder's tokenizer.json or, without one, through its
     tokenizer.model (SentencePiece, as LLaMA-2 checkpoints bring it): a small model trained here
